@@ -1,0 +1,43 @@
+"""CPU oracle for the diagonal-tiled MXFP attention path.
+
+TEST INFRASTRUCTURE ONLY.  This package restates, in plain torch/numpy on the
+CPU, the algorithm of the reference's MXFP path (format classes, MX quantizer,
+block-scaled matmul, tile-by-tile online-softmax attention).  It exists so the
+HIP kernels can be checked against it and so a CPU baseline can be timed next
+to them.  Nothing in the shipped package may import it: only the test-suite,
+the smoke check and the benchmark's CPU-baseline leg do.
+
+Each function names the reference file:line it follows (paths are relative to
+the reference checkout).
+
+Parity status of each restated function:
+
+* ``decode_e2m1``, ``pack_fp4``/``unpack_fp4``, ``encode_e8m0``/``decode_e8m0``
+  -- pinned by closed forms and exhaustive enumeration (tests/test_oracle_formats.py).
+* ``encode_e2m1`` -- pinned by an exhaustive brute-force nearest/ties-to-even
+  search over every bf16 and fp16 value, and by golden vectors minted from the
+  reference's own ``MXFP4Tensor._from_float`` for the near-tie bias
+  (tests/golden/mxfp_vectors.npz).
+* ``encode_e4m3`` -- not in the reference (which stores E5M2); pinned by an
+  independent closed-form encoder and torch's own float8_e4m3fn cast.
+* ``quantize_mx`` -- composition of the above; pinned by invariants and
+  hand-worked blocks.  Two corners are PARITY UNPINNED against the reference's
+  Triton kernel (it cannot run here): (1) ``floor(log2(amax))`` is the true
+  floor (bit extraction), whereas a float32 ``log2`` may round up for an amax
+  one ulp below a power of two; (2) an all-zero block gets scale byte 0 and
+  codes +0.
+* ``gemm_mx`` -- dequantise + matmul; pinned against exact integer arithmetic.
+* ``attn_mx`` -- pinned against dense float64 softmax attention on the same
+  per-tile dequantised operands, and special cases (single tile, V = 1,
+  identical keys, GQA == repeat_interleave).
+"""
+
+from .mx_formats import (  # noqa: F401
+    E2M1_VALUES, decode_e2m1, encode_e2m1, pack_fp4, unpack_fp4,
+    encode_e8m0, decode_e8m0, encode_e4m3, decode_e4m3, encode_e5m2, decode_e5m2,
+)
+from .mx_quantize import (  # noqa: F401
+    FMT_E2M1, FMT_E4M3, FMT_E5M2, EMAX_ELEM, q_pre_scale, quantize_mx, dequantize_mx, smooth_k,
+)
+from .mx_gemm import gemm_mx  # noqa: F401
+from .mx_attention import attn_mx, attn_dense_f64, precision_metric, v_fragment_order  # noqa: F401

@@ -1,0 +1,158 @@
+"""Diagonal-tiled mixed-precision MXFP attention, restated on the CPU.
+
+TEST INFRASTRUCTURE ONLY (see the package docstring).
+
+Loop structure and numerics follow the reference's fused kernel
+(``ours/mxfp_attn_kernel.py:216-359``: exp2 online softmax, float32 running max / sum, P summed
+in float32 before the down-cast, low-precision P.V, ``acc / l`` epilogue); the causal
+decomposition (tiles left of the diagonal unmasked, the diagonal tile masked ``row >= col``,
+tiles right of it never visited) follows ``ours/online_routing.py:68-77, :113-118``; the
+grouped-query head mapping follows ``ours/online_routing.py:160-171``.  The benchmark contract
+adds per-tile precision: tile ``j == i`` uses the 8-bit operands, every other tile the 4-bit
+ones.
+"""
+
+import torch
+import torch.nn.functional as Fnn
+
+from .mx_quantize import FMT_E2M1, FMT_E4M3, quantize_mx, dequantize_mx, q_pre_scale, smooth_k as _smooth_k
+
+MODES = ("mxfp4", "mxfp8", "diag")
+
+
+def _tile_is_8bit(mode: str, i: int, j: int) -> bool:
+    if mode == "mxfp8":
+        return True
+    if mode == "mxfp4":
+        return False
+    if mode == "diag":
+        return i == j
+    raise ValueError(f"unknown block_scale_type {mode}")
+
+
+def _prepare(q, k, mode, scale, fmt8):
+    """Quantize + dequantize Q and K in the formats the mode needs (float32 fake-quant)."""
+    D = q.shape[-1]
+    pre = q_pre_scale(D, scale)
+    ops = {}
+    if mode in ("mxfp4", "diag"):
+        ops["q4"] = dequantize_mx(*quantize_mx(q, pre, FMT_E2M1), FMT_E2M1)
+        ops["k4"] = dequantize_mx(*quantize_mx(k, 1.0, FMT_E2M1), FMT_E2M1)
+    if mode in ("mxfp8", "diag"):
+        ops["q8"] = dequantize_mx(*quantize_mx(q, pre, fmt8), fmt8)
+        ops["k8"] = dequantize_mx(*quantize_mx(k, 1.0, fmt8), fmt8)
+    return ops
+
+
+def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=False,
+            fmt8=FMT_E4M3, out_dtype=None, heads=None) -> torch.Tensor:
+    """Tile-by-tile MXFP attention.  q ``[B,Hq,N,D]``, k/v ``[B,Hkv,N,D]`` in bf16 or fp16.
+
+    P is rounded to v's dtype before P.V and the product of a tile is accumulated in float32
+    (ours/mxfp_attn_kernel.py:339-340).  ``heads`` restricts the computation to a list of query
+    heads (the output then has ``len(heads)`` heads).  N need not be a multiple of ``tile``:
+    the last key tile is cut at N."""
+    B, Hq, N, D = q.shape
+    Hkv = k.shape[1]
+    assert Hq % Hkv == 0
+    group = Hq // Hkv
+    if smooth_k:
+        k = _smooth_k(k)
+    lp = v.dtype
+    assert lp in (torch.bfloat16, torch.float16)
+    out_dtype = out_dtype or lp
+    head_list = list(range(Hq)) if heads is None else list(heads)
+    ops = _prepare(q[:, head_list], k, mode, scale, fmt8)
+    vf = v.to(torch.float32)
+    nt = (N + tile - 1) // tile
+    out = torch.empty((B, len(head_list), N, D), dtype=out_dtype)
+    for b in range(B):
+        for hi_, h in enumerate(head_list):
+            kvh = h // group
+            for i in range(nt):
+                r0, r1 = i * tile, min((i + 1) * tile, N)
+                rows = r1 - r0
+                m = torch.full((rows,), float("-inf"))
+                l = torch.zeros((rows,))
+                acc = torch.zeros((rows, D))
+                last = i if causal else nt - 1
+                for j in range(last + 1):
+                    c0, c1 = j * tile, min((j + 1) * tile, N)
+                    tag = "8" if _tile_is_8bit(mode, i, j) else "4"
+                    qt = ops["q" + tag][b, hi_, r0:r1]
+                    kt = ops["k" + tag][b, kvh, c0:c1]
+                    s = qt @ kt.T                                    # float32, already in log2 units
+                    if causal and j == i:
+                        rr = torch.arange(r0, r1).unsqueeze(1)
+                        cc = torch.arange(c0, c1).unsqueeze(0)
+                        s = torch.where(cc > rr, torch.tensor(float("-inf")), s)
+                    m_new = torch.maximum(m, s.amax(dim=1))
+                    p = torch.exp2(s - m_new.unsqueeze(1))
+                    alpha = torch.exp2(m - m_new)
+                    l = l * alpha + p.sum(dim=1)
+                    pv = p.to(lp).to(torch.float32) @ vf[b, kvh, c0:c1]
+                    acc = acc * alpha.unsqueeze(1) + pv
+                    m = m_new
+                out[b, hi_, r0:r1] = (acc / l.unsqueeze(1)).to(out_dtype)
+    return out
+
+
+def attn_dense_f64(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=False,
+                   fmt8=FMT_E4M3, heads=None) -> torch.Tensor:
+    """Brute-force check of :func:`attn_mx`: the full score matrix is assembled tile by tile from
+    the per-tile-precision dequantised operands, then a dense base-2 softmax and P.V in float64
+    (no online rescaling, no low-precision P)."""
+    B, Hq, N, D = q.shape
+    Hkv = k.shape[1]
+    group = Hq // Hkv
+    if smooth_k:
+        k = _smooth_k(k)
+    head_list = list(range(Hq)) if heads is None else list(heads)
+    ops = {n: t.double() for n, t in _prepare(q[:, head_list], k, mode, scale, fmt8).items()}
+    nt = (N + tile - 1) // tile
+    out = torch.empty((B, len(head_list), N, D), dtype=torch.float64)
+    for b in range(B):
+        for hi_, h in enumerate(head_list):
+            kvh = h // group
+            s = torch.full((N, N), float("-inf"), dtype=torch.float64)
+            for i in range(nt):
+                for j in range((i if causal else nt - 1) + 1):
+                    tag = "8" if _tile_is_8bit(mode, i, j) else "4"
+                    r = slice(i * tile, min((i + 1) * tile, N))
+                    c = slice(j * tile, min((j + 1) * tile, N))
+                    s[r, c] = ops["q" + tag][b, hi_, r] @ ops["k" + tag][b, kvh, c].T
+            if causal:
+                s = s.masked_fill(torch.ones(N, N, dtype=torch.bool).triu(1), float("-inf"))
+            p = torch.exp2(s - s.amax(dim=1, keepdim=True))
+            out[b, hi_] = (p / p.sum(dim=1, keepdim=True)) @ v[b, kvh].double()
+    return out
+
+
+def precision_metric(x: torch.Tensor, ref: torch.Tensor) -> dict:
+    """Cosine similarity over the flattened tensors, relative L1, RMSE and max-abs error.
+    Definition of the first three: spas_sage_attn/utils.py:25-36."""
+    a, b = x.double().reshape(1, -1), ref.double().reshape(1, -1)
+    return {
+        "cos": Fnn.cosine_similarity(a, b).item(),
+        "l1": ((a - b).abs().sum() / b.abs().sum()).item(),
+        "rmse": torch.sqrt(torch.mean((a - b) ** 2)).item(),
+        "max_abs": (a - b).abs().max().item(),
+    }
+
+
+def v_fragment_order(v: torch.Tensor, tile: int) -> torch.Tensor:
+    """Value-tile layout the HIP attention kernel consumes, restated for checking the repack kernel.
+
+    v ``[B,H,N,D]`` -> ``[B,H,Npad/tile, tile/32, 2, D/32, 64, 8]`` with
+    ``out[.., kb, c, db, lane, t] = v[key, dim]`` where ``lane = 32*h + r``, ``dim = 32*db + r`` and
+    ``key = tile*it + 32*kb + 16*c + 8*(t//4) + 4*h + t%4``; keys past N read as zero.  (This is the
+    build's own operand layout, not a reference format: it lets a 64-lane wave fetch one
+    32x16 value block for the matrix core with a single 16-byte load per lane.)"""
+    B, H, N, D = v.shape
+    nt = (N + tile - 1) // tile
+    vp = torch.zeros((B, H, nt * tile, D), dtype=v.dtype)
+    vp[:, :, :N] = v
+    # key index decomposition: key = tile*it + 32*kb + 16*c + 8*t1 + 4*h + t0
+    x = vp.reshape(B, H, nt, tile // 32, 2, 2, 2, 4, D // 32, 32)    # it kb c t1 h t0 db r
+    x = x.permute(0, 1, 2, 3, 4, 8, 6, 9, 5, 7)                       # it kb c db h r t1 t0
+    return x.reshape(B, H, nt, tile // 32, 2, D // 32, 64, 8).contiguous()
