@@ -1,0 +1,208 @@
+#!/usr/bin/env python3
+"""Benchmark of the diagonal-tiled MXFP attention path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c1] [--no-cpu-baseline]
+
+One "step" is one full pass of the hot path over one synthetic batch already resident in HBM:
+MX-quantize Q and K (E2M1 + E4M3 in one pass each), repack V, fused attention (diagonal tiles MXFP8,
+off-diagonal MXFP4, causal, GQA).  Prints ONE JSON line: whole-step attention TFLOP/s
+(FlashAttention convention 2*B*Hq*N^2*D for causal), the roofline of the dominant kernel (the fused
+attention kernel, timed alone with HIP events on its launch stream), secondary figures for the
+quantizer and the standalone block-scaled GEMM, and the CPU oracle timed on the host cores on a bounded
+sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "mp-sparse-attn_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+import torch  # noqa: E402
+
+# published MI355X dense peaks
+PEAK_FP4_TFLOPS = 10100.0
+PEAK_FP8_TFLOPS = 5000.0
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (B, Hq, Hkv, N, D, tile, seed, description)
+    "c1": (1, 8, 8, 1024, 64, 64, 0, "C1 B1 H8 N1024 D64 causal tile64 diag"),
+    "c3": (1, 32, 8, 8192, 128, 128, 2, "C3 llama3-8b prefill B1 Hq32 Hkv8 N8192 D128 causal tile128 diag(MXFP8)/offdiag(MXFP4), outlier channels"),
+    "c4": (1, 32, 8, 131072, 128, 128, 3, "C4 long-context prefill B1 Hq32 Hkv8 N131072 D128 causal tile128 diag, outlier channels"),
+}
+
+
+def make_inputs(B, Hq, Hkv, N, D, seed, device):
+    g = torch.Generator(device=device).manual_seed(seed)
+    q = torch.randn(B, Hq, N, D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    k = torch.randn(B, Hkv, N, D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    v = torch.randn(B, Hkv, N, D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    n_out = max(1, round(0.01 * D))
+    gc = torch.Generator().manual_seed(seed)
+    for t, H in ((q, Hq), (k, Hkv)):
+        for h in range(H):
+            idx = torch.randint(0, D, (n_out,), generator=gc).to(device)
+            t[:, h, :, idx] *= 20.0
+    return q, k, v
+
+
+def composite_peak_tflops(nt):
+    """Bound when Q.K^T runs at the MXFP4 / MXFP8 peak (diagonal share 2/(nt+1) of the visited tiles) and
+    P.V at the bf16 peak: half of the FLOPs each."""
+    diag = 2.0 / (nt + 1)
+    t = 0.5 * ((1 - diag) / PEAK_FP4_TFLOPS + diag / PEAK_FP8_TFLOPS) + 0.5 / PEAK_BF16_TFLOPS
+    return 1.0 / t
+
+
+def time_events(fn, iters):
+    """Average duration (ms) of fn() over iters launches, HIP events on torch's current stream -- the stream
+    libmpsa launches on."""
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def cpu_baseline(q, k, v, tile, D):
+    """The CPU oracle (a port of the reference's fake-quant path) on one KV group of the workload."""
+    import oracle as O
+    Hq, Hkv = q.shape[1], k.shape[1]
+    group = Hq // Hkv
+    n = min(q.shape[2], 8192)
+    qs = q[:, :group, :n].cpu()
+    ks = k[:, :1, :n].cpu()
+    vs = v[:, :1, :n].cpu()
+    t0 = time.perf_counter()
+    O.attn_mx(qs, ks, vs, tile=tile, causal=True, mode="diag")
+    dt = time.perf_counter() - t0
+    flops = 2.0 * qs.shape[0] * group * n * n * D
+    return {
+        "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"oracle.attn_mx (quantize+dequantize+tiled attention, torch CPU) on {group} query heads / 1 KV head, "
+                  f"N={n}, D={D}, causal, diag mode: {dt:.2f} s",
+        "seconds": dt,
+    }
+
+
+def secondary(device, quick):
+    """Quantizer GB/s on the 8192x8192 GEMM operand and block-scaled GEMM TFLOP/s at 8192^3."""
+    from ours import _lib
+    from ours.quant_mxint8 import quantize_mx, quantize_mx_dual
+    from ours.block_scaled_matmul import block_scaled_matmul, make_configs
+    out = {}
+    M = N = K = 8192
+    g = torch.Generator(device=device).manual_seed(1)
+    a = torch.randn(M, K, generator=g, device=device).to(torch.bfloat16)[None, None]
+    b = torch.randn(N, K, generator=g, device=device).to(torch.bfloat16)[None, None]
+    it = 5 if quick else 20
+    for name, fmt, bpe in (("quant_e2m1", _lib.FMT_E2M1, 2 + 0.5 + 1 / 32), ("quant_e4m3", _lib.FMT_E4M3, 2 + 1 + 1 / 32)):
+        quantize_mx(a, 1.0, fmt)
+        ms = time_events(lambda: quantize_mx(a, 1.0, fmt), it)
+        gbs = M * K * bpe / ms / 1e6
+        out[name] = {"GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4), "ms": round(ms, 4)}
+    quantize_mx_dual(a, 1.0)
+    ms = time_events(lambda: quantize_mx_dual(a, 1.0), it)
+    gbs = M * K * (2 + 0.5 + 1 + 2 / 32) / ms / 1e6
+    out["quant_dual"] = {"GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4), "ms": round(ms, 4)}
+    for bst, fmt, peak in (("mxfp4", _lib.FMT_E2M1, PEAK_FP4_TFLOPS), ("mxfp8", _lib.FMT_E4M3, PEAK_FP8_TFLOPS)):
+        ac, asc = quantize_mx(a, 1.0, fmt)
+        bc, bsc = quantize_mx(b, 1.0, fmt)
+        cfg = make_configs(bst)
+        args = (ac[0, 0], asc[0, 0], bc[0, 0], bsc[0, 0], torch.bfloat16, M, N, K, cfg)
+        block_scaled_matmul(*args)
+        ms = time_events(lambda: block_scaled_matmul(*args), it)
+        tf = 2.0 * M * N * K / ms / 1e9
+        out["gemm_" + bst] = {"TFLOP/s": round(tf, 1), "frac_peak": round(tf / peak, 4), "ms": round(ms, 4)}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the kernel is measured on one GPU's "
+              "share at its real shape); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        sys.exit(1)
+
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands
+
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
+    q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device)
+    out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
+
+    def step():
+        ops = prepare_operands(q, k, v, tile, "diag")
+        attention_from_operands(ops, out, True)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt * 1e3 / args.steps
+    flops = 2.0 * B * Hq * N * N * D
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+
+    # dominant kernel alone: the fused attention kernel on prepared operands
+    ops = prepare_operands(q, k, v, tile, "diag")
+    attention_from_operands(ops, out, True)
+    torch.cuda.synchronize()
+    k_iters = max(5, args.steps)
+    attn_ms = time_events(lambda: attention_from_operands(ops, out, True), k_iters)
+    prep_ms = time_events(lambda: prepare_operands(q, k, v, tile, "diag"), k_iters)
+    achieved = flops / (attn_ms * 1e-3) / 1e12
+    nt = (N + tile - 1) // tile
+    comp = composite_peak_tflops(nt)
+    roofline = {
+        "bound": "mfma", "kernel": "attn_fwd_kernel", "achieved": round(achieved, 2), "peak": PEAK_FP4_TFLOPS,
+        "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP4_TFLOPS, 5), "traffic": None,
+        "kernel_ms": round(attn_ms, 4), "prepare_ms": round(prep_ms, 4),
+        "composite_peak": round(comp, 1), "frac_composite": round(achieved / comp, 5),
+        "flops_per_launch": flops,
+    }
+
+    result = {
+        "metric": "MXFP attn TFLOPS + % of scaled-MFMA peak, causal N=8K/128K D=128, 1 GPU",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "mxfp4/mxfp8 scores (E2M1/E4M3 + E8M0), bf16 P.V, f32 accumulate", "data": "synthetic",
+        "config": {"workload": desc, "B": B, "Hq": Hq, "Hkv": Hkv, "N": N, "D": D, "tile": tile,
+                   "step": "quantize Q,K (dual) + V repack + fused attention"},
+        "frac_mxfp4_peak": round(tflops / PEAK_FP4_TFLOPS, 5),
+        "roofline": roofline,
+    }
+    if not args.no_secondary:
+        result["secondary"] = secondary(device, quick=args.steps < 10)
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(q, k, v, tile, D)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

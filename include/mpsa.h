@@ -1,0 +1,142 @@
+/*
+ * mpsa.h -- C ABI of the MI355X (gfx950) MXFP attention path.
+ *
+ * One shared library, libmpsa.so, exports the functions below.  Every pointer is a plain
+ * device (HBM) pointer unless stated otherwise; every function enqueues its kernels on the
+ * given HIP stream and returns without synchronising.  The library keeps no reference to
+ * caller memory and allocates none: inputs, outputs and intermediates are all caller-owned.
+ * Return value: 0 on success, a negative MPSA_E* code otherwise; mpsa_last_error() then gives
+ * a human-readable reason (thread-local).  No exception or torch type crosses this boundary.
+ *
+ * Citations name the reference interface each entry point replaces (paths relative to the
+ * reference checkout).
+ */
+#ifndef MPSA_H
+#define MPSA_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* hipStream_t is an opaque pointer; the ABI takes it as void* so this header needs no HIP. */
+typedef void* mpsa_stream_t;
+
+/* element dtypes of unquantized tensors */
+#define MPSA_BF16 0
+#define MPSA_F16  1
+#define MPSA_F32  2
+
+/* MX element formats; the values are the CDNA4 scaled-MFMA format selectors */
+#define MPSA_FMT_E4M3 0
+#define MPSA_FMT_E5M2 1
+#define MPSA_FMT_E2M1 4
+
+/* per-tile precision of the attention score product */
+#define MPSA_MODE_MXFP4 0   /* every tile 4-bit */
+#define MPSA_MODE_MXFP8 1   /* every tile 8-bit */
+#define MPSA_MODE_DIAG  2   /* tile j == i 8-bit, all others 4-bit */
+
+#define MPSA_OK             0
+#define MPSA_EINVAL        -1   /* null pointer, bad enum, bad shape */
+#define MPSA_EALIGN        -2   /* pointer or stride not 16-byte aligned */
+#define MPSA_EUNSUPPORTED  -3   /* shape outside the compiled variants */
+#define MPSA_ELAUNCH       -4   /* the HIP runtime refused the launch */
+
+int mpsa_version(void);
+const char* mpsa_last_error(void);
+
+/*
+ * Elementwise format conversions behind the MXFP4Tensor / MXScaleTensor helper classes; contiguous
+ * arrays of n elements.
+ *   mpsa_e2m1_encode  float32 -> one E2M1 code per byte (round to nearest, ties to even mantissa,
+ *                     NaN/Inf/overflow -> magnitude 6).      Replaces MXFP4Tensor._from_float, ours/mxfp.py:84-170.
+ *   mpsa_e2m1_decode  code byte -> float32.                  Replaces MXFP4Tensor.to, ours/mxfp.py:44-77.
+ *   mpsa_e8m0_encode  float32 -> E8M0 byte (<=0, NaN, Inf -> 255; else clamp(floor(log2 v)+127, 0, 254)).
+ *                                                            Replaces MXScaleTensor._from_float, ours/mxfp.py:286-307.
+ *   mpsa_e8m0_decode  E8M0 byte -> float32 2^(e-127), 255 -> NaN.  Replaces MXScaleTensor.to, ours/mxfp.py:275-284.
+ */
+int mpsa_e2m1_encode(const float* x, int64_t n, uint8_t* codes, mpsa_stream_t stream);
+int mpsa_e2m1_decode(const uint8_t* codes, int64_t n, float* out, mpsa_stream_t stream);
+int mpsa_e8m0_encode(const float* x, int64_t n, uint8_t* codes, mpsa_stream_t stream);
+int mpsa_e8m0_decode(const uint8_t* codes, int64_t n, float* out, mpsa_stream_t stream);
+
+/*
+ * MX quantizer.  Replaces quant_mxfp4 / quant_mxfp8e5 and their Triton kernels
+ * (ours/quant_mxint8.py:453-512, :276-351, :223-272, :164-219) together with the host-side
+ * nibble packing MXFP4Tensor.to_packed_tensor (ours/mxfp.py:172-205).
+ *
+ *   x          [B,H,N,D] of x_dtype (MPSA_BF16 | MPSA_F16), element strides x_strides[4],
+ *              last dim contiguous, D % 32 == 0, rows 16-byte aligned
+ *   pre_scale  float32 factor multiplied in before quantizing (sm_scale*log2(e) for Q, 1 for K)
+ *   fmt        MPSA_FMT_E2M1 | MPSA_FMT_E4M3 | MPSA_FMT_E5M2
+ *   emax_elem  shared exponent = floor(log2(amax)) - emax_elem (reference: 3 for E2M1, 7 for 8-bit)
+ *   codes      [B,H,out_rows,D/2] (E2M1, two codes per byte, even element in the low nibble)
+ *              or [B,H,out_rows,D] (8-bit), contiguous
+ *   scales     [B,H,out_rows,D/32] E8M0 bytes, contiguous
+ *   out_rows   rows per (b,h) in the outputs, >= N; rows N..out_rows-1 are written as zero
+ */
+int mpsa_quantize_mx(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                     const int64_t x_strides[4], float pre_scale, int fmt, int emax_elem,
+                     uint8_t* codes, uint8_t* scales, int64_t out_rows, mpsa_stream_t stream);
+
+/*
+ * Both precisions in one pass over x (the diagonal-tiled attention needs Q and K in E2M1 and in
+ * an 8-bit format).  Same contract as two mpsa_quantize_mx calls with (E2M1, emax4) and
+ * (fmt8, emax8); x is read once.  Replaces the same reference functions as above.
+ */
+int mpsa_quantize_mx_dual(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                          const int64_t x_strides[4], float pre_scale, int emax4, int fmt8, int emax8,
+                          uint8_t* codes4, uint8_t* scales4, uint8_t* codes8, uint8_t* scales8,
+                          int64_t out_rows, mpsa_stream_t stream);
+
+/*
+ * Block-scaled matmul  C[M,N] = (A o 2^(sa-127)) (B o 2^(sb-127))^T.  Replaces block_scaled_matmul
+ * and its Triton kernel (ours/block_scaled_matmul.py:271-296, :154-267).
+ *
+ *   a, b     packed codes [M,K/2] / [N,K/2] (E2M1) or [M,K] / [N,K] (8-bit), row-major, contiguous
+ *   sa, sb   E8M0 bytes [M,K/32] / [N,K/32], row-major (the linear layout, not the 5-D packed one)
+ *   fmt      element format of both operands
+ *   c        [M,N] of c_dtype (MPSA_BF16 | MPSA_F16 | MPSA_F32), leading dimension ldc elements
+ *   M % 256 == 0, N % 256 == 0, K % 128 == 0
+ */
+int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
+                 int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream);
+
+/*
+ * Value-tile repack: v [B,H,N,D] (bf16 | f16, strided, last dim contiguous) -> v_tiles
+ * [B,H,ceil(N/tile),tile*D] of the same dtype in matrix-core operand order, keys past N zero.
+ * Replaces the dtype normalisation / .contiguous() of V in the reference wrapper
+ * (ours/mxfp_attn_kernel.py:27-31); the layout is this library's own.
+ */
+int mpsa_v_tiles(const void* v, int v_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                 const int64_t v_strides[4], int tile, void* v_tiles, mpsa_stream_t stream);
+
+/*
+ * Fused attention forward.  Replaces block_scaled_batched_attn and its Triton kernel
+ * (ours/mxfp_attn_kernel.py:362-423, :103-359), with the causal tile structure and grouped-query
+ * head mapping of ours/online_routing.py:68-77, :113-118, :160-171.
+ *
+ *   q4,qs4 / q8,qs8   Q codes + scales from the quantizer, rows padded to n_pad per head:
+ *                     [B,Hq,n_pad,D/2],[B,Hq,n_pad,D/32] and [B,Hq,n_pad,D],[B,Hq,n_pad,D/32]
+ *   k4,ks4 / k8,ks8   same for K with Hkv heads
+ *                     (the 4-bit set may be null in MPSA_MODE_MXFP8, the 8-bit set in MPSA_MODE_MXFP4)
+ *   fmt8              MPSA_FMT_E4M3 | MPSA_FMT_E5M2
+ *   v_tiles           output of mpsa_v_tiles for the same tile, pv_dtype (MPSA_BF16 | MPSA_F16);
+ *                     P is rounded to that dtype before P.V
+ *   o                 [B,Hq,N,D] of o_dtype (MPSA_BF16 | MPSA_F16 | MPSA_F32), element strides o_strides[4],
+ *                     last dim contiguous
+ *   n                 valid sequence length, n_pad = ceil(n/tile)*tile
+ *   tile              64 | 128 (score tile edge = precision granularity), D in {64,128}
+ */
+int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
+                  const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
+                  const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
+                  int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                  mpsa_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MPSA_H */

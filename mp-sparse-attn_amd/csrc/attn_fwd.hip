@@ -1,0 +1,380 @@
+// Fused diagonal-tiled MXFP attention forward for gfx950.
+//
+// Per query tile i of one head: for every visited key tile j, S = Q_i K_j^T on the scaled matrix cores
+// (8-bit operands when the tile's precision is 8-bit, 4-bit otherwise), base-2 online softmax with
+// float32 running max / sum, P rounded to 16 bits, O += P V_j, and O / l at the end -- the loop of the
+// reference's block_scaled_batched_attn_kernel (ours/mxfp_attn_kernel.py:216-359).  Causal runs visit
+// tiles j <= i and mask only tile j == i (ours/online_routing.py:68-77, :113-118); query head hq reads
+// key/value head hq / (Hq/Hkv) (ours/online_routing.py:160-171).  Q already carries sm_scale*log2(e)
+// (folded in by the quantizer, ours/quant_mxint8.py:494), so scores are in log2 units.
+//
+// Mapping.  A workgroup owns one TILE-query tile; each of its TILE/32 waves owns 32 queries and walks all
+// keys of every tile.  Both products are computed transposed so that a lane always owns ONE query:
+//   S^T = K Q^T   on v_mfma_scale_f32_32x32x64_f8f6f4: lane (h = lane/32, r = lane%32) of the K operand
+//                 supplies one 32-element MX block of key row r with its E8M0 byte, the Q operand the
+//                 same for query r; the result leaves query r's scores for 16 keys per 32-key block in
+//                 that lane's registers, so the row maximum is a register reduction plus one exchange
+//                 with lane^32, and running max / sum / rescale factors are plain per-lane scalars.
+//   O^T += V^T P^T on v_mfma_f32_32x32x16_{bf16,f16}: the P^T operand of lane (h, r) is exactly the eight
+//                 scores that lane already holds (keys are contracted in the order the score MFMA left
+//                 them); V is pre-arranged by mpsa_v_tiles to match, one 16-byte LDS read per operand.
+// K codes, K scales and the V tile are staged through LDS (K rows padded by 16 bytes so that 128-bit
+// reads are bank-conflict free; the V tile is read lane-contiguously), double-buffered, with the next
+// tile's global loads issued before the current tile's math.
+#include "mpsa_common.h"
+
+namespace {
+
+struct AttnArgs {
+    const uint8_t *q4, *qs4, *q8, *qs8, *k4, *ks4, *k8, *ks8;
+    const void* v;
+    void* o;
+    int64_t o_sb, o_sh, o_sn;
+    int B, Hq, Hkv, n, n_pad, nt;
+    int causal, mode, fmt8, o_dtype;
+};
+
+template <int PVT> struct PV;
+template <> struct PV<MPSA_BF16> {
+    typedef v8bf vec;
+    typedef __bf16 elem;
+    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+template <> struct PV<MPSA_F16> {
+    typedef v8h vec;
+    typedef _Float16 elem;
+    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+
+template <int FMT8>
+__device__ __forceinline__ v16f score_mfma8(v8i k, v8i q, v16f c, int sel, int ks, int qs) {
+    if (sel == 0) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, FMT8, FMT8, 0, ks, 0, qs);
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, FMT8, FMT8, 2, ks, 2, qs);
+}
+__device__ __forceinline__ v16f score_mfma4(v8i k, v8i q, v16f c, int sel, int ks, int qs) {
+    if (sel == 0) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, 4, 4, 0, ks, 0, qs);
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, 4, 4, 2, ks, 2, qs);
+}
+
+template <int D, int TILE>
+struct Geom {
+    static constexpr int NW = TILE / 32;          // waves per workgroup
+    static constexpr int NT = NW * 64;            // threads
+    static constexpr int KB = TILE / 32;          // 32-key blocks per tile
+    static constexpr int SST = D / 64;            // score matrix instructions along D
+    static constexpr int NDB = D / 32;            // 32-wide output dim blocks
+    static constexpr int PK4 = D / 2 + 16;        // LDS row pitch of 4-bit K rows
+    static constexpr int PK8 = D + 16;            // LDS row pitch of 8-bit K rows
+    static constexpr int K_BYTES = TILE * PK8;
+    static constexpr int S_BYTES = TILE * 4;
+    static constexpr int V_BYTES = TILE * D * 2;
+    static constexpr int BUF = K_BYTES + S_BYTES + V_BYTES;
+    static constexpr int KC4 = TILE * (D / 2) / 16 / NT;   // 16-byte K chunks per thread, 4-bit
+    static constexpr int KC8 = 2 * KC4;
+    static constexpr int VC = V_BYTES / 16 / NT;
+};
+
+template <int D, int TILE, int PVT, int FMT8>
+__global__ __launch_bounds__(TILE * 2, 1) void attn_fwd_kernel(AttnArgs a) {
+    typedef Geom<D, TILE> G;
+    typedef PV<PVT> P;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, w = tid >> 6;
+    const int h = lane >> 5, r = lane & 31;
+
+    // ---- which (batch, kv head, query head, query tile) -- XCD-aware, heavy causal tiles first ----
+    const int group = a.Hq / a.Hkv;
+    const int total = a.B * a.Hq * a.nt;
+    int L = blockIdx.x;
+    if ((total & 7) == 0) L = (L & 7) * (total >> 3) + (L >> 3);      // XCD x gets one contiguous logical range
+    const int per_unit = group * a.nt;
+    const int unit = L / per_unit;
+    const int rem = L - unit * per_unit;
+    const int rank = rem / group;
+    const int hq = (unit % a.Hkv) * group + (rem - rank * group);
+    const int b = unit / a.Hkv;
+    const int kvh = unit % a.Hkv;
+    const int i = a.causal ? a.nt - 1 - rank : rank;
+
+    const int64_t qhead_row = ((int64_t)b * a.Hq + hq) * a.n_pad;
+    const int64_t khead_row = ((int64_t)b * a.Hkv + kvh) * a.n_pad;
+    const int q_local = 32 * w + r;
+    const int64_t q_row = qhead_row + (int64_t)i * TILE + q_local;
+
+    const bool need4 = a.mode != MPSA_MODE_MXFP8;
+    const bool need8 = a.mode != MPSA_MODE_MXFP4;
+
+    // ---- Q fragments stay in registers for the whole tile row ----
+    v8i q4f[G::SST], q8f[G::SST];
+    int qsc4 = 0, qsc8 = 0;
+#pragma unroll
+    for (int s = 0; s < G::SST; ++s) {
+        q4f[s] = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
+        q8f[s] = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
+    }
+    if (need4) {
+#pragma unroll
+        for (int s = 0; s < G::SST; ++s) {
+            const v4i x = *reinterpret_cast<const v4i*>(a.q4 + q_row * (D / 2) + (2 * s + h) * 16);
+            q4f[s] = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+        }
+        const uint32_t sw = (D == 128) ? *reinterpret_cast<const uint32_t*>(a.qs4 + q_row * 4)
+                                       : (uint32_t)*reinterpret_cast<const uint16_t*>(a.qs4 + q_row * 2);
+        qsc4 = (int)(sw >> (8 * h));
+    }
+    if (need8) {
+#pragma unroll
+        for (int s = 0; s < G::SST; ++s) {
+            const v4i x0 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + (2 * s + h) * 32);
+            const v4i x1 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + (2 * s + h) * 32 + 16);
+            q8f[s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        }
+        const uint32_t sw = (D == 128) ? *reinterpret_cast<const uint32_t*>(a.qs8 + q_row * 4)
+                                       : (uint32_t)*reinterpret_cast<const uint16_t*>(a.qs8 + q_row * 2);
+        qsc8 = (int)(sw >> (8 * h));
+    }
+
+    // ---- staging registers: next tile's K codes, K scales, V ----
+    v4i rk[G::KC8], rv[G::VC];
+#pragma unroll
+    for (int c = 0; c < G::KC8; ++c) rk[c] = (v4i){0, 0, 0, 0};
+    uint32_t rs = 0;
+    auto tile_is8 = [&](int j) { return a.mode == MPSA_MODE_MXFP8 || (a.mode == MPSA_MODE_DIAG && j == i); };
+    auto load_tile = [&](int j, bool is8) __attribute__((always_inline)) {
+        const int64_t krow0 = khead_row + (int64_t)j * TILE;
+        const uint8_t* src = is8 ? a.k8 + krow0 * D : a.k4 + krow0 * (D / 2);
+        const int nchunk = is8 ? G::KC8 : G::KC4;
+#pragma unroll
+        for (int c = 0; c < G::KC8; ++c)
+            if (c < nchunk) rk[c] = *reinterpret_cast<const v4i*>(src + (int64_t)(tid + G::NT * c) * 16);
+        if (tid < TILE) {
+            const uint8_t* sp = (is8 ? a.ks8 : a.ks4) + (krow0 + tid) * (D / 32);
+            rs = (D == 128) ? *reinterpret_cast<const uint32_t*>(sp) : (uint32_t)*reinterpret_cast<const uint16_t*>(sp);
+        }
+        const uint8_t* vsrc = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)j * TILE) * (D * 2);
+#pragma unroll
+        for (int c = 0; c < G::VC; ++c) rv[c] = *reinterpret_cast<const v4i*>(vsrc + (int64_t)(tid + G::NT * c) * 16);
+    };
+    auto store_tile = [&](int buf, bool is8) __attribute__((always_inline)) {
+        uint8_t* kb_ = smem + buf * G::BUF;
+        const int cpr_shift = is8 ? (D == 128 ? 3 : 2) : (D == 128 ? 2 : 1);   // log2(16-byte chunks per K row)
+        const int pitch = is8 ? G::PK8 : G::PK4;
+        const int nchunk = is8 ? G::KC8 : G::KC4;
+#pragma unroll
+        for (int c = 0; c < G::KC8; ++c)
+            if (c < nchunk) {
+                const int q = tid + G::NT * c;
+                *reinterpret_cast<v4i*>(kb_ + (q >> cpr_shift) * pitch + (q & ((1 << cpr_shift) - 1)) * 16) = rk[c];
+            }
+        if (tid < TILE) *reinterpret_cast<uint32_t*>(kb_ + G::K_BYTES + tid * 4) = rs;
+        uint8_t* vb = kb_ + G::K_BYTES + G::S_BYTES;
+#pragma unroll
+        for (int c = 0; c < G::VC; ++c) *reinterpret_cast<v4i*>(vb + (tid + G::NT * c) * 16) = rv[c];
+    };
+
+    v16f acc[G::NDB];
+#pragma unroll
+    for (int d = 0; d < G::NDB; ++d)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[d][e] = 0.0f;
+    float m_run = -__builtin_inff();
+    float l_run = 0.0f;
+
+    const int j_end = a.causal ? i + 1 : a.nt;
+    bool cur8 = tile_is8(0);
+    load_tile(0, cur8);
+    store_tile(0, cur8);
+    __syncthreads();
+
+    for (int j = 0; j < j_end; ++j) {
+        const int buf = j & 1;
+        const bool nxt = j + 1 < j_end;
+        const bool nxt8 = nxt ? tile_is8(j + 1) : false;
+        if (nxt) load_tile(j + 1, nxt8);
+
+        const uint8_t* kl = smem + buf * G::BUF;
+        const uint8_t* sl = kl + G::K_BYTES;
+        const uint8_t* vl = sl + G::S_BYTES;
+
+        // ---- S^T = K Q^T ----
+        v16f st[G::KB];
+#pragma unroll
+        for (int kb = 0; kb < G::KB; ++kb) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) st[kb][e] = 0.0f;
+            const int krow = 32 * kb + r;
+            const int ksc = (int)(*reinterpret_cast<const uint32_t*>(sl + krow * 4) >> (8 * h));
+            if (cur8) {
+#pragma unroll
+                for (int s = 0; s < G::SST; ++s) {
+                    const uint8_t* p = kl + krow * G::PK8 + (2 * s + h) * 32;
+                    const v4i x0 = *reinterpret_cast<const v4i*>(p);
+                    const v4i x1 = *reinterpret_cast<const v4i*>(p + 16);
+                    const v8i kf = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+                    st[kb] = score_mfma8<FMT8>(kf, q8f[s], st[kb], s, ksc, qsc8);
+                }
+            } else {
+#pragma unroll
+                for (int s = 0; s < G::SST; ++s) {
+                    const v4i x = *reinterpret_cast<const v4i*>(kl + krow * G::PK4 + (2 * s + h) * 16);
+                    const v8i kf = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+                    st[kb] = score_mfma4(kf, q4f[s], st[kb], s, ksc, qsc4);
+                }
+            }
+        }
+
+        // ---- masks: causal on the diagonal tile, key tail on the last tile ----
+        const bool diag_mask = a.causal && j == i;
+        const bool tail_mask = (j == a.nt - 1) && (a.n < a.n_pad);
+        if (diag_mask || tail_mask) {
+            const int kmax = tail_mask ? a.n - j * TILE : TILE;        // keys >= kmax are padding
+#pragma unroll
+            for (int kb = 0; kb < G::KB; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int key = 32 * kb + 8 * (e >> 2) + 4 * h + (e & 3);
+                    const bool dead = (diag_mask && key > q_local) || key >= kmax;
+                    if (dead) st[kb][e] = -__builtin_inff();
+                }
+        }
+
+        // ---- online softmax (per lane = per query) ----
+        float mx = st[0][0];
+#pragma unroll
+        for (int kb = 0; kb < G::KB; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, st[kb][e]);
+        mx = __builtin_fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = __builtin_fmaxf(m_run, mx);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        m_run = m_new;
+        float psum = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < G::KB; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float p = __builtin_amdgcn_exp2f(st[kb][e] - m_new);
+                st[kb][e] = p;
+                psum += p;
+            }
+        l_run = l_run * alpha + psum;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int d = 0; d < G::NDB; ++d)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[d][e] *= alpha;
+        }
+
+        // ---- O^T += V^T P^T ----
+#pragma unroll
+        for (int kb = 0; kb < G::KB; ++kb)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                typename P::vec pf;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) pf[t] = (typename P::elem)st[kb][8 * c + t];
+#pragma unroll
+                for (int d = 0; d < G::NDB; ++d) {
+                    const typename P::vec vf =
+                        *reinterpret_cast<const typename P::vec*>(vl + (((kb * 2 + c) * G::NDB + d) * 64 + lane) * 16);
+                    acc[d] = P::mfma(vf, pf, acc[d]);
+                }
+            }
+
+        if (nxt) store_tile(buf ^ 1, nxt8);
+        cur8 = nxt8;
+        __syncthreads();
+    }
+
+    // ---- epilogue: O = acc / l ; register e of lane (h, r): dim 32*db + 8*(e/4) + 4*h + e%4 of query r ----
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float inv = 1.0f / l_tot;
+    const int q_global = i * TILE + q_local;
+    if (q_global < a.n) {
+        uint8_t* orow = static_cast<uint8_t*>(a.o);
+        const int64_t off = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh + (int64_t)q_global * a.o_sn;
+#pragma unroll
+        for (int d = 0; d < G::NDB; ++d)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int dim = 32 * d + 8 * g4 + 4 * h;
+                const float o0 = acc[d][4 * g4 + 0] * inv, o1 = acc[d][4 * g4 + 1] * inv;
+                const float o2 = acc[d][4 * g4 + 2] * inv, o3 = acc[d][4 * g4 + 3] * inv;
+                if (a.o_dtype == MPSA_BF16) {
+                    typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+                    const v4bf pk = {(__bf16)o0, (__bf16)o1, (__bf16)o2, (__bf16)o3};
+                    *reinterpret_cast<v4bf*>(orow + (off + dim) * 2) = pk;
+                } else if (a.o_dtype == MPSA_F16) {
+                    typedef _Float16 v4hh __attribute__((ext_vector_type(4)));
+                    const v4hh pk = {(_Float16)o0, (_Float16)o1, (_Float16)o2, (_Float16)o3};
+                    *reinterpret_cast<v4hh*>(orow + (off + dim) * 2) = pk;
+                } else {
+                    const v4f pk = {o0, o1, o2, o3};
+                    *reinterpret_cast<v4f*>(orow + (off + dim) * 4) = pk;
+                }
+            }
+    }
+}
+
+template <int D, int TILE, int PVT, int FMT8>
+int launch_one(const AttnArgs& a, hipStream_t st) {
+    typedef Geom<D, TILE> G;
+    constexpr int smem = 2 * G::BUF;
+    static bool attr_set = false;      // idempotent; a race only repeats the same call
+    auto kern = attn_fwd_kernel<D, TILE, PVT, FMT8>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "attn: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
+        attr_set = true;
+    }
+    dim3 grid((unsigned)(a.B * a.Hq * a.nt));
+    hipLaunchKernelGGL(kern, grid, dim3(G::NT), smem, st, a);
+    MPSA_CHECK_LAUNCH("attn");
+    return MPSA_OK;
+}
+
+template <int D, int TILE>
+int launch_dt(const AttnArgs& a, int pv_dtype, hipStream_t st) {
+    if (pv_dtype == MPSA_BF16)
+        return a.fmt8 == MPSA_FMT_E5M2 ? launch_one<D, TILE, MPSA_BF16, MPSA_FMT_E5M2>(a, st) : launch_one<D, TILE, MPSA_BF16, MPSA_FMT_E4M3>(a, st);
+    return a.fmt8 == MPSA_FMT_E5M2 ? launch_one<D, TILE, MPSA_F16, MPSA_FMT_E5M2>(a, st) : launch_one<D, TILE, MPSA_F16, MPSA_FMT_E4M3>(a, st);
+}
+
+}  // namespace
+
+extern "C" int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
+                             const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
+                             const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
+                             int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                             mpsa_stream_t stream) {
+    if (mode != MPSA_MODE_MXFP4 && mode != MPSA_MODE_MXFP8 && mode != MPSA_MODE_DIAG) return mpsa_fail(MPSA_EINVAL, "attn: unknown mode %d", mode);
+    const bool need4 = mode != MPSA_MODE_MXFP8, need8 = mode != MPSA_MODE_MXFP4;
+    if (need4 && (!q4 || !qs4 || !k4 || !ks4)) return mpsa_fail(MPSA_EINVAL, "attn: 4-bit operands missing");
+    if (need8 && (!q8 || !qs8 || !k8 || !ks8)) return mpsa_fail(MPSA_EINVAL, "attn: 8-bit operands missing");
+    if (!v_tiles || !o || !o_strides) return mpsa_fail(MPSA_EINVAL, "attn: null pointer");
+    if (need8 && fmt8 != MPSA_FMT_E4M3 && fmt8 != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "attn: 8-bit format must be E4M3 or E5M2");
+    if (pv_dtype != MPSA_BF16 && pv_dtype != MPSA_F16) return mpsa_fail(MPSA_EINVAL, "attn: pv_dtype must be bf16 or f16");
+    if (o_dtype != MPSA_BF16 && o_dtype != MPSA_F16 && o_dtype != MPSA_F32) return mpsa_fail(MPSA_EINVAL, "attn: bad output dtype");
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || n <= 0 || Hq % Hkv) return mpsa_fail(MPSA_EINVAL, "attn: bad shape (B=%lld Hq=%lld Hkv=%lld n=%lld)", (long long)B, (long long)Hq, (long long)Hkv, (long long)n);
+    if ((D != 64 && D != 128) || (tile != 64 && tile != 128)) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: D=%lld tile=%d (both must be 64 or 128)", (long long)D, tile);
+    if (o_strides[3] != 1 || (o_strides[0] % 4) || (o_strides[1] % 4) || (o_strides[2] % 4)) return mpsa_fail(MPSA_EALIGN, "attn: output rows must be contiguous and 8-byte aligned");
+    const uintptr_t al = reinterpret_cast<uintptr_t>(q4) | reinterpret_cast<uintptr_t>(q8) | reinterpret_cast<uintptr_t>(k4) |
+                         reinterpret_cast<uintptr_t>(k8) | reinterpret_cast<uintptr_t>(v_tiles) | reinterpret_cast<uintptr_t>(o);
+    const uintptr_t al4 = reinterpret_cast<uintptr_t>(qs4) | reinterpret_cast<uintptr_t>(qs8) | reinterpret_cast<uintptr_t>(ks4) | reinterpret_cast<uintptr_t>(ks8);
+    if ((al & 15) || (al4 & 3)) return mpsa_fail(MPSA_EALIGN, "attn: operands must be 16-byte (codes, v, o) / 4-byte (scales) aligned");
+    const int64_t nt = (n + tile - 1) / tile;
+    if (B * Hq * nt >= (int64_t(1) << 31) || nt * tile >= (int64_t(1) << 30)) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: problem too large");
+    AttnArgs a;
+    a.q4 = q4; a.qs4 = qs4; a.q8 = q8; a.qs8 = qs8; a.k4 = k4; a.ks4 = ks4; a.k8 = k8; a.ks8 = ks8;
+    a.v = v_tiles; a.o = o;
+    a.o_sb = o_strides[0]; a.o_sh = o_strides[1]; a.o_sn = o_strides[2];
+    a.B = (int)B; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.n = (int)n; a.nt = (int)nt; a.n_pad = (int)(nt * tile);
+    a.causal = causal ? 1 : 0; a.mode = mode; a.fmt8 = fmt8; a.o_dtype = o_dtype;
+    hipStream_t st = (hipStream_t)stream;
+    if (D == 128 && tile == 128) return launch_dt<128, 128>(a, pv_dtype, st);
+    if (D == 64 && tile == 64)   return launch_dt<64, 64>(a, pv_dtype, st);
+    if (D == 128 && tile == 64)  return launch_dt<128, 64>(a, pv_dtype, st);
+    return launch_dt<64, 128>(a, pv_dtype, st);
+}

@@ -1,0 +1,29 @@
+// Shared host/device helpers of libmpsa (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include "../../include/mpsa.h"
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef unsigned short v8us __attribute__((ext_vector_type(8)));
+
+// thread-local error text, filled by mpsa_fail()
+int mpsa_fail(int code, const char* fmt, ...);
+
+static inline bool mpsa_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+#define MPSA_CHECK_LAUNCH(what)                                                        \
+    do {                                                                               \
+        hipError_t e__ = hipGetLastError();                                            \
+        if (e__ != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "%s: %s", what, hipGetErrorString(e__)); \
+    } while (0)
+
+__device__ __forceinline__ float mpsa_u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t mpsa_f2u(float f) { return __builtin_bit_cast(uint32_t, f); }

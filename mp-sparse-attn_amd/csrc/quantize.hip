@@ -1,0 +1,207 @@
+// MX quantizer for gfx950: bf16/f16 rows -> E2M1 / E4M3 / E5M2 codes + one E8M0 scale per 32 elements.
+//
+// Semantics follow the reference's quantizer (ours/quant_mxint8.py:276-351 for E2M1, :164-219 for the
+// 8-bit format): x32 = f32(x) * pre; amax per 32 elements of the last dim; shared exponent
+// floor(log2(amax)) - emax_elem; divide by that power of two; clamp; encode; scale byte
+// clamp(shared_exp + 127, 0, 254).  The E2M1 encoder reproduces MXFP4Tensor._from_float
+// (ours/mxfp.py:84-170) bit for bit, including its float32 1e-6 tie-break bias; codes leave the
+// kernel already nibble-packed (ours/mxfp.py:196-205: even element in the low nibble).
+//
+// Work mapping: one lane owns 8 consecutive elements (one 128-bit load), four neighbouring lanes
+// own one MX block, so the block maximum is two DPP quad exchanges.  The kernel is HBM-bound:
+// 2 B/element in, 0.5 (+1) B/element of codes and 1/32 (x2) B/element of scales out.
+#include "mpsa_common.h"
+#include "mx_codec.h"
+
+namespace {
+
+struct QuantArgs {
+    const void* x;
+    int64_t sb, sh, sn;        // element strides of x
+    int n, d;                  // valid rows, row length
+    int out_rows;              // rows per (b,h) in the outputs
+    float pre;
+    int emax4, emax8;
+    uint8_t *codes4, *scales4, *codes8, *scales8;
+};
+
+template <int DPP_CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), DPP_CTRL, 0xf, 0xf, false));
+}
+
+template <int FMT8, bool SW8>
+__device__ __forceinline__ uint32_t fp8_pack4(float y0, float y1, float y2, float y3) {
+    if constexpr (SW8) {
+        if constexpr (FMT8 == MPSA_FMT_E4M3)
+            return e4m3_encode_sw(y0) | (e4m3_encode_sw(y1) << 8) | (e4m3_encode_sw(y2) << 16) | (e4m3_encode_sw(y3) << 24);
+        else
+            return e5m2_encode_sw(y0) | (e5m2_encode_sw(y1) << 8) | (e5m2_encode_sw(y2) << 16) | (e5m2_encode_sw(y3) << 24);
+    } else {
+        int w = 0;
+        if constexpr (FMT8 == MPSA_FMT_E4M3) {
+            w = __builtin_amdgcn_cvt_pk_fp8_f32(y0, y1, w, false);
+            w = __builtin_amdgcn_cvt_pk_fp8_f32(y2, y3, w, true);
+        } else {
+            w = __builtin_amdgcn_cvt_pk_bf8_f32(y0, y1, w, false);
+            w = __builtin_amdgcn_cvt_pk_bf8_f32(y2, y3, w, true);
+        }
+        return (uint32_t)w;
+    }
+}
+
+template <int XDT>
+__device__ __forceinline__ void load8(const void* p, float (&x)[8]) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if constexpr (XDT == MPSA_BF16) {
+            x[2 * i] = mpsa_u2f(w[i] << 16);
+            x[2 * i + 1] = mpsa_u2f(w[i] & 0xFFFF0000u);
+        } else {
+            x[2 * i] = (float)__builtin_bit_cast(_Float16, (unsigned short)(w[i] & 0xFFFFu));
+            x[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(w[i] >> 16));
+        }
+    }
+}
+
+template <int XDT, bool DO4, bool DO8, int FMT8, bool SW8>
+__global__ __launch_bounds__(256) void quantize_kernel(QuantArgs a) {
+    const uint32_t cpr = (uint32_t)a.d >> 3;                              // 16-byte chunks per row
+    const uint32_t chunks = (uint32_t)a.out_rows * cpr;                   // per (b,h)
+    const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+    if (c >= chunks) return;                                              // whole quads leave together (cpr % 4 == 0)
+    const uint32_t row = c / cpr;
+    const uint32_t col8 = c - row * cpr;
+    const int64_t head = (int64_t)blockIdx.z * gridDim.y + blockIdx.y;    // flat (b,h)
+
+    float x[8];
+    if (row < (uint32_t)a.n) {
+        const char* base = static_cast<const char*>(a.x) +
+                           2 * ((int64_t)blockIdx.z * a.sb + (int64_t)blockIdx.y * a.sh + (int64_t)row * a.sn + 8 * (int64_t)col8);
+        load8<XDT>(base, x);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = 0.0f;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        x[i] = x[i] * a.pre;
+        amax = __builtin_fmaxf(amax, __builtin_fabsf(x[i]));
+    }
+    amax = __builtin_fmaxf(amax, dpp_f32<0xB1>(amax));   // quad_perm [1,0,3,2]
+    amax = __builtin_fmaxf(amax, dpp_f32<0x4E>(amax));   // quad_perm [2,3,0,1]
+
+    const uint32_t ab = mpsa_f2u(amax);
+    const bool zero = (ab == 0u);
+    const uint32_t ef = ab >> 23;
+    const int e = ef ? (int)ef - 127 : (31 - __builtin_clz(ab | 1u)) - 149;   // floor(log2(amax)), subnormals included
+
+    const int64_t oc = head * chunks + c;                                 // flat output chunk
+    const bool quad_leader = (threadIdx.x & 3u) == 0u;
+
+    if constexpr (DO4) {
+        const int se = e - a.emax4;
+        uint32_t word = 0;
+        if (!zero) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) word |= e2m1_encode(ldexpf(x[i], -se)) << (4 * i);
+        }
+        reinterpret_cast<uint32_t*>(a.codes4)[oc] = word;
+        const int sbyte = zero ? 0 : min(max(se + 127, 0), 254);
+        if (quad_leader) a.scales4[oc >> 2] = (uint8_t)sbyte;
+    }
+    if constexpr (DO8) {
+        const int se = e - a.emax8;
+        const float lim = (FMT8 == MPSA_FMT_E4M3) ? 448.0f : 57344.0f;
+        uint2 w = make_uint2(0u, 0u);
+        if (!zero) {
+            float y[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) y[i] = __builtin_fminf(__builtin_fmaxf(ldexpf(x[i], -se), -lim), lim);
+            w.x = fp8_pack4<FMT8, SW8>(y[0], y[1], y[2], y[3]);
+            w.y = fp8_pack4<FMT8, SW8>(y[4], y[5], y[6], y[7]);
+        }
+        reinterpret_cast<uint2*>(a.codes8)[oc] = w;
+        const int sbyte = zero ? 0 : min(max(se + 127, 0), 254);
+        if (quad_leader) a.scales8[oc >> 2] = (uint8_t)sbyte;
+    }
+}
+
+bool use_sw_fp8() {
+    static const bool sw = [] {
+        const char* v = getenv("MPSA_FP8_ENCODE");
+        return v && v[0] == 's';
+    }();
+    return sw;
+}
+
+template <int XDT, bool DO4, bool DO8>
+void launch(const QuantArgs& a, int fmt8, dim3 grid, hipStream_t st) {
+    const bool sw = use_sw_fp8();
+    if (!DO8 || fmt8 == MPSA_FMT_E4M3) {
+        if (sw) hipLaunchKernelGGL((quantize_kernel<XDT, DO4, DO8, MPSA_FMT_E4M3, true>), grid, dim3(256), 0, st, a);
+        else    hipLaunchKernelGGL((quantize_kernel<XDT, DO4, DO8, MPSA_FMT_E4M3, false>), grid, dim3(256), 0, st, a);
+    } else {
+        if (sw) hipLaunchKernelGGL((quantize_kernel<XDT, DO4, DO8, MPSA_FMT_E5M2, true>), grid, dim3(256), 0, st, a);
+        else    hipLaunchKernelGGL((quantize_kernel<XDT, DO4, DO8, MPSA_FMT_E5M2, false>), grid, dim3(256), 0, st, a);
+    }
+}
+
+int quantize_common(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D, const int64_t* xs,
+                    float pre, bool do4, int emax4, bool do8, int fmt8, int emax8,
+                    uint8_t* c4, uint8_t* s4, uint8_t* c8, uint8_t* s8, int64_t out_rows, hipStream_t st) {
+    if (!x || !xs) return mpsa_fail(MPSA_EINVAL, "quantize: null input");
+    if ((do4 && (!c4 || !s4)) || (do8 && (!c8 || !s8))) return mpsa_fail(MPSA_EINVAL, "quantize: null output");
+    if (x_dtype != MPSA_BF16 && x_dtype != MPSA_F16) return mpsa_fail(MPSA_EINVAL, "quantize: x_dtype must be bf16 or f16");
+    if (do8 && fmt8 != MPSA_FMT_E4M3 && fmt8 != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "quantize: 8-bit format must be E4M3 or E5M2");
+    if (B < 0 || H < 0 || N < 0 || D <= 0 || out_rows < N) return mpsa_fail(MPSA_EINVAL, "quantize: bad shape");
+    if (D % 32) return mpsa_fail(MPSA_EINVAL, "quantize: D=%lld is not a multiple of 32", (long long)D);
+    if (xs[3] != 1) return mpsa_fail(MPSA_EINVAL, "quantize: last dim of x must be contiguous");
+    if (!mpsa_aligned16(x) || (xs[0] % 8) || (xs[1] % 8) || (xs[2] % 8)) return mpsa_fail(MPSA_EALIGN, "quantize: x rows must be 16-byte aligned");
+    if ((do4 && !mpsa_aligned16(c4)) || (do8 && !mpsa_aligned16(c8))) return mpsa_fail(MPSA_EALIGN, "quantize: outputs must be 16-byte aligned");
+    if (B == 0 || H == 0 || out_rows == 0) return MPSA_OK;
+    const int64_t chunks = out_rows * (D / 8);
+    if (chunks >= (int64_t(1) << 31) || H > 65535 || B > 65535) return mpsa_fail(MPSA_EUNSUPPORTED, "quantize: a head has too many elements, or too many heads");
+    QuantArgs a;
+    a.x = x; a.sb = xs[0]; a.sh = xs[1]; a.sn = xs[2];
+    a.n = (int)N; a.d = (int)D; a.out_rows = (int)out_rows; a.pre = pre;
+    a.emax4 = emax4; a.emax8 = emax8;
+    a.codes4 = c4; a.scales4 = s4; a.codes8 = c8; a.scales8 = s8;
+    dim3 grid((unsigned)((chunks + 255) / 256), (unsigned)H, (unsigned)B);
+    if (x_dtype == MPSA_BF16) {
+        if (do4 && do8) launch<MPSA_BF16, true, true>(a, fmt8, grid, st);
+        else if (do4)   launch<MPSA_BF16, true, false>(a, fmt8, grid, st);
+        else            launch<MPSA_BF16, false, true>(a, fmt8, grid, st);
+    } else {
+        if (do4 && do8) launch<MPSA_F16, true, true>(a, fmt8, grid, st);
+        else if (do4)   launch<MPSA_F16, true, false>(a, fmt8, grid, st);
+        else            launch<MPSA_F16, false, true>(a, fmt8, grid, st);
+    }
+    MPSA_CHECK_LAUNCH("quantize");
+    return MPSA_OK;
+}
+
+}  // namespace
+
+extern "C" int mpsa_quantize_mx(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                                const int64_t x_strides[4], float pre_scale, int fmt, int emax_elem,
+                                uint8_t* codes, uint8_t* scales, int64_t out_rows, mpsa_stream_t stream) {
+    if (fmt == MPSA_FMT_E2M1)
+        return quantize_common(x, x_dtype, B, H, N, D, x_strides, pre_scale, true, emax_elem, false, 0, 0,
+                               codes, scales, nullptr, nullptr, out_rows, (hipStream_t)stream);
+    if (fmt == MPSA_FMT_E4M3 || fmt == MPSA_FMT_E5M2)
+        return quantize_common(x, x_dtype, B, H, N, D, x_strides, pre_scale, false, 0, true, fmt, emax_elem,
+                               nullptr, nullptr, codes, scales, out_rows, (hipStream_t)stream);
+    return mpsa_fail(MPSA_EINVAL, "quantize: unknown format %d", fmt);
+}
+
+extern "C" int mpsa_quantize_mx_dual(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                                     const int64_t x_strides[4], float pre_scale, int emax4, int fmt8, int emax8,
+                                     uint8_t* codes4, uint8_t* scales4, uint8_t* codes8, uint8_t* scales8,
+                                     int64_t out_rows, mpsa_stream_t stream) {
+    return quantize_common(x, x_dtype, B, H, N, D, x_strides, pre_scale, true, emax4, true, fmt8, emax8,
+                           codes4, scales4, codes8, scales8, out_rows, (hipStream_t)stream);
+}

@@ -1,0 +1,99 @@
+"""ctypes binding of libmpsa.so (the C ABI declared in include/mpsa.h).
+
+PyTorch is used for device memory and streams only: tensors are handed over as raw device
+pointers, sizes and element strides, and kernels are enqueued on torch's current stream.
+"""
+
+import ctypes
+import os
+
+import torch
+
+BF16, F16, F32 = 0, 1, 2
+FMT_E4M3, FMT_E5M2, FMT_E2M1 = 0, 1, 4
+MODE_MXFP4, MODE_MXFP8, MODE_DIAG = 0, 1, 2
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libmpsa.so")
+
+_i64, _int, _vp, _f32 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_float
+_p64 = ctypes.POINTER(ctypes.c_int64)
+
+# name -> (restype, argtypes); must list every symbol include/mpsa.h declares
+SIGNATURES = {
+    "mpsa_version": (_int, []),
+    "mpsa_last_error": (ctypes.c_char_p, []),
+    "mpsa_e2m1_encode": (_int, [_vp, _i64, _vp, _vp]),
+    "mpsa_e2m1_decode": (_int, [_vp, _i64, _vp, _vp]),
+    "mpsa_e8m0_encode": (_int, [_vp, _i64, _vp, _vp]),
+    "mpsa_e8m0_decode": (_int, [_vp, _i64, _vp, _vp]),
+    "mpsa_quantize_mx": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _f32, _int, _int, _vp, _vp, _i64, _vp]),
+    "mpsa_quantize_mx_dual": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _f32, _int, _int, _int,
+                                     _vp, _vp, _vp, _vp, _i64, _vp]),
+    "mpsa_gemm_mx": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
+    "mpsa_v_tiles": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _int, _vp, _vp]),
+    "mpsa_attn_fwd": (_int, [_vp] * 8 + [_int, _vp, _int, _vp, _int, _p64,
+                             _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
+}
+
+_lib = None
+
+
+class MpsaError(RuntimeError):
+    """A libmpsa entry point returned a negative status."""
+
+    def __init__(self, code, message):
+        super().__init__(f"libmpsa error {code}: {message}")
+        self.code = code
+
+
+def lib():
+    """Load libmpsa.so once.  Raises if it has not been built -- there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python mp-sparse-attn_amd/build.py` "
+                "(hipcc, gfx950). The MXFP path has no CPU or eager fallback.")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(status):
+    if status != 0:
+        raise MpsaError(status, lib().mpsa_last_error().decode("utf-8", "replace"))
+
+
+def dtype_id(dtype):
+    if dtype == torch.bfloat16:
+        return BF16
+    if dtype == torch.float16:
+        return F16
+    if dtype == torch.float32:
+        return F32
+    raise ValueError(f"unsupported dtype {dtype}")
+
+
+def require_device(*tensors):
+    for t in tensors:
+        if not isinstance(t, torch.Tensor) or not t.is_cuda:
+            raise RuntimeError("the MXFP path runs on HIP device tensors only (got a %s tensor); "
+                               "there is no CPU fallback" % (t.device if isinstance(t, torch.Tensor) else type(t)))
+
+
+def stream_ptr(device=None):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def strides4(t):
+    assert t.dim() == 4
+    return (ctypes.c_int64 * 4)(*t.stride())

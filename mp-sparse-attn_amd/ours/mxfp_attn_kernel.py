@@ -1,0 +1,113 @@
+"""Fused MXFP attention -- the reference's ``ours/mxfp_attn_kernel.py::mxfp_attn_kernel`` on HIP kernels.
+
+Pipeline per call (all on torch's current stream, no host synchronisation):
+  1. MX-quantize Q (with ``scale*log2e`` folded in) and K -- ``mpsa_quantize_mx`` / ``_dual``;
+  2. repack V into matrix-core operand order -- ``mpsa_v_tiles``;
+  3. fused attention -- ``mpsa_attn_fwd``.
+"""
+
+import torch
+
+from . import _lib
+from .quant_mxint8 import quantize_mx, quantize_mx_dual, pre_scale_q, _as_bhnd
+
+_MODES = {"mxfp4": _lib.MODE_MXFP4, "mxfp8": _lib.MODE_MXFP8, "mxfp8e5": _lib.MODE_MXFP8, "diag": _lib.MODE_DIAG,
+          "diag_e5": _lib.MODE_DIAG}
+
+
+def prepare_operands(q, k, v, tile, block_scale_type, scale=None):
+    """Quantize Q/K and repack V for one attention call.  q ``[B,Hq,N,D]``, k/v ``[B,Hkv,N,D]`` of one
+    16-bit dtype.  Returns a dict of device tensors (rows padded to whole tiles) the launcher consumes."""
+    if block_scale_type not in _MODES:
+        raise ValueError(f"Invalid block scale type: {block_scale_type}")
+    mode = _MODES[block_scale_type]
+    fmt8 = _lib.FMT_E5M2 if block_scale_type.endswith("e5") else _lib.FMT_E4M3
+    B, Hq, N, D = q.shape
+    Hkv = k.shape[1]
+    nt = (N + tile - 1) // tile
+    n_pad = nt * tile
+    pre = pre_scale_q(D, scale)
+    ops = {"mode": mode, "fmt8": fmt8, "tile": tile, "n": N, "q4": None, "qs4": None, "q8": None, "qs8": None,
+           "k4": None, "ks4": None, "k8": None, "ks8": None}
+    if mode == _lib.MODE_DIAG:
+        ops["q4"], ops["qs4"], ops["q8"], ops["qs8"] = quantize_mx_dual(q, pre, fmt8, n_pad)
+        ops["k4"], ops["ks4"], ops["k8"], ops["ks8"] = quantize_mx_dual(k, 1.0, fmt8, n_pad)
+    elif mode == _lib.MODE_MXFP4:
+        ops["q4"], ops["qs4"] = quantize_mx(q, pre, _lib.FMT_E2M1, out_rows=n_pad)
+        ops["k4"], ops["ks4"] = quantize_mx(k, 1.0, _lib.FMT_E2M1, out_rows=n_pad)
+    else:
+        ops["q8"], ops["qs8"] = quantize_mx(q, pre, fmt8, out_rows=n_pad)
+        ops["k8"], ops["ks8"] = quantize_mx(k, 1.0, fmt8, out_rows=n_pad)
+    v_tiles = torch.empty((B, Hkv, nt, tile * D), dtype=v.dtype, device=v.device)
+    with torch.cuda.device(v.device):
+        _lib.check(_lib.lib().mpsa_v_tiles(_lib.ptr(v), _lib.dtype_id(v.dtype), B, Hkv, N, D, _lib.strides4(v), tile,
+                                           _lib.ptr(v_tiles), _lib.stream_ptr(v.device)))
+    ops["v_tiles"] = v_tiles
+    ops["shape"] = (B, Hq, Hkv, N, D)
+    return ops
+
+
+def attention_from_operands(ops, out, is_causal):
+    """Launch ``mpsa_attn_fwd`` on prepared operands; ``out`` is a ``[B,Hq,N,D]`` view (last dim contiguous)."""
+    B, Hq, Hkv, N, D = ops["shape"]
+    dev = out.device
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mpsa_attn_fwd(
+            _lib.ptr(ops["q4"]), _lib.ptr(ops["qs4"]), _lib.ptr(ops["q8"]), _lib.ptr(ops["qs8"]),
+            _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]), _lib.ptr(ops["ks8"]), ops["fmt8"],
+            _lib.ptr(ops["v_tiles"]), _lib.dtype_id(ops["v_tiles"].dtype), _lib.ptr(out), _lib.dtype_id(out.dtype),
+            _lib.strides4(out), B, Hq, Hkv, N, D, ops["tile"], 1 if is_causal else 0, ops["mode"],
+            _lib.stream_ptr(dev)))
+    return out
+
+
+def _normalise(q, k, v):
+    """Reference prologue (ours/mxfp_attn_kernel.py:27-31): fp32/fp16 inputs run in fp16, everything else in
+    bf16.  V follows Q/K's 16-bit dtype here (the reference always used fp16 for V)."""
+    lp = torch.float16 if q.dtype in (torch.float32, torch.float16) else torch.bfloat16
+    return q.to(lp), k.to(lp), v.to(lp)
+
+
+def _reject_unsupported(attn_mask, dropout_p, attention_sink, return_sparsity, skip_thresh):
+    if attn_mask is not None or dropout_p != 0.0 or attention_sink or return_sparsity:
+        raise NotImplementedError("attn_mask, dropout_p, attention_sink and return_sparsity are not implemented "
+                                  "(the reference accepts and ignores them)")
+    if skip_thresh is not None:
+        raise NotImplementedError("tile skipping (skip_thresh) is not implemented")
+
+
+@torch.compiler.disable
+def mxfp_attn_kernel(q, k, v, attn_mask=None, dropout_p=0.0,
+                     is_causal=False, scale=None, smooth_k=False, attention_sink=False, tensor_layout="HND",
+                     output_dtype=torch.float16, return_sparsity=False, block_scale_type="mxfp4", skip_thresh=None,
+                     tile=128):
+    """Attention output ``[B,Hq,N,D]`` (``"NHD"``: ``[B,N,Hq,D]``) from MX-quantized Q.K^T and 16-bit P.V.
+
+    Signature of the reference (ours/mxfp_attn_kernel.py:19-22) plus ``tile`` (score tile edge, 64 or 128).
+    ``block_scale_type``: ``"mxfp4"``, ``"mxfp8"`` (E4M3), ``"mxfp8e5"`` (E5M2, the reference's 8-bit format),
+    ``"diag"`` (tile j == i in MXFP8, the rest in MXFP4) or ``"diag_e5"``.  K/V may have fewer heads than Q
+    (grouped-query attention); ``is_causal`` is honoured."""
+    _lib.require_device(q, k, v)
+    _reject_unsupported(attn_mask, dropout_p, attention_sink, return_sparsity, skip_thresh)
+    torch.cuda.set_device(v.device)
+    q, k, v = _normalise(q, k, v)
+    q, k, v = _as_bhnd(q, tensor_layout), _as_bhnd(k, tensor_layout), _as_bhnd(v, tensor_layout)
+    if smooth_k:
+        k = k - k.mean(dim=-2, keepdim=True)                        # ours/mxfp_attn_kernel.py:33-34
+    B, Hq, N, D = q.shape
+    assert D in [64, 128], "headdim should be in [64, 128]."
+    assert k.shape[2] == N and v.shape[2] == N, "q, k and v must have the same sequence length"
+    assert k.shape[1] == v.shape[1] and Hq % k.shape[1] == 0, "query heads must be a multiple of key/value heads"
+    assert tile in (64, 128), "tile must be 64 or 128"
+    if output_dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise ValueError(f"Unsupported dtype: {output_dtype}")       # ours/mxfp_attn_kernel.py:389
+    if v.stride(-1) != 1:
+        v = v.contiguous()
+    ops = prepare_operands(q, k, v, tile, block_scale_type, scale)
+    if tensor_layout == "HND":
+        out = torch.empty((B, Hq, N, D), dtype=output_dtype, device=q.device)
+        attention_from_operands(ops, out, is_causal)
+        return out
+    out = torch.empty((B, N, Hq, D), dtype=output_dtype, device=q.device)
+    attention_from_operands(ops, out.transpose(1, 2), is_causal)
+    return out

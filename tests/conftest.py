@@ -1,0 +1,40 @@
+import os
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "mp-sparse-attn_amd")
+for p in (ROOT, PKG):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (HIP device); run with -m gpu")
+
+
+def pytest_collection_modifyitems(config, items):
+    if torch.cuda.is_available():
+        return
+    skip = pytest.mark.skip(reason="no HIP device")
+    for item in items:
+        if "gpu" in item.keywords:
+            item.add_marker(skip)
+
+
+def make_qkv(B, Hq, Hkv, N, D, seed, dtype=torch.bfloat16, sigma=1.0, outliers=False):
+    """Seeded synthetic q/k/v on the CPU (float32 draw, then cast), so the oracle and the GPU see the same
+    bits.  ``outliers``: per head one channel (1% of 128 rounds to 1) of q and of k is multiplied by 20."""
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, Hq, N, D, generator=g) * sigma
+    k = torch.randn(B, Hkv, N, D, generator=g) * sigma
+    v = torch.randn(B, Hkv, N, D, generator=g) * sigma
+    if outliers:
+        n_out = max(1, round(0.01 * D))
+        for t, H in ((q, Hq), (k, Hkv)):
+            for h in range(H):
+                idx = torch.randint(0, D, (n_out,), generator=g)
+                t[:, h, :, idx] *= 20.0
+    return q.to(dtype), k.to(dtype), v.to(dtype)

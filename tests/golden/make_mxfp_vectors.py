@@ -45,6 +45,9 @@ def e2m1_inputs():
         parts.append(base - offs)
     parts.append(torch.tensor([0.0, -0.0, float("inf"), float("-inf"), float("nan"), 6.5, 7.0, 8.0, 100.0, 1e-30,
                               1e-45, 0.1, 0.2499999, 5.9999995], dtype=torch.float32))
+    # large magnitudes: float32 cancellation makes the distances to several candidates equal there
+    big = torch.ldexp(torch.ones(20), torch.arange(20, 40, dtype=torch.int32))
+    parts.append(torch.cat([big, big * 1.25, big + 6.0, big + 2.0, torch.tensor([1e9, 3e38, 16777222.0, 33554438.0])]))
     parts.append(torch.rand(4096, generator=g) * 8.0)
     parts.append(torch.randn(4096, generator=g) * 2.0)
     x = torch.cat(parts)

@@ -1,0 +1,89 @@
+"""The C-ABI library loads, exports every symbol include/mpsa.h declares, and rejects bad arguments on the
+host (no kernel is launched; runs without a GPU)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from conftest import ROOT
+from ours import _lib
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "mpsa.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mpsa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared()
+    assert "mpsa_attn_fwd" in names and "mpsa_quantize_mx" in names and len(names) >= 11
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(handle, n), f"{n} declared in mpsa.h but not exported"
+    assert sorted(_lib.SIGNATURES) == names
+    assert _lib.lib().mpsa_version() >= 100
+
+
+def test_host_side_argument_validation():
+    L = _lib.lib()
+    null = ctypes.c_void_p(0)
+    one = ctypes.c_void_p(16)           # never dereferenced: validation fails first
+    st = (ctypes.c_int64 * 4)(1, 1, 32, 1)
+    assert L.mpsa_quantize_mx(null, 0, 1, 1, 1, 32, st, 1.0, 4, 3, one, one, 1, null) == -1
+    assert b"null" in L.mpsa_last_error()
+    st_ok = (ctypes.c_int64 * 4)(64, 64, 64, 1)
+    assert L.mpsa_quantize_mx(one, 0, 1, 1, 1, 48, st_ok, 1.0, 4, 3, one, one, 1, null) == -1      # D % 32
+    assert L.mpsa_quantize_mx(one, 2, 1, 1, 1, 64, st_ok, 1.0, 4, 3, one, one, 1, null) == -1      # f32 input
+    assert L.mpsa_quantize_mx(one, 0, 1, 1, 1, 64, st_ok, 1.0, 9, 3, one, one, 1, null) == -1      # bad format
+    assert L.mpsa_quantize_mx(one, 0, 1, 1, 2, 64, st_ok, 1.0, 4, 3, one, one, 1, null) == -1      # out_rows < N
+    assert L.mpsa_quantize_mx(ctypes.c_void_p(24), 0, 1, 1, 1, 64, st_ok, 1.0, 4, 3, one, one, 1, null) == -2
+    assert L.mpsa_gemm_mx(one, one, one, one, 4, 100, 256, 128, one, 0, 256, null) == -3           # M % 256
+    assert L.mpsa_gemm_mx(one, one, one, one, 4, 256, 256, 128, one, 7, 256, null) == -1           # bad dtype
+    assert L.mpsa_v_tiles(one, 0, 1, 1, 128, 96, st_ok, 128, one, null) == -3                      # D = 96
+    so = (ctypes.c_int64 * 4)(128 * 128, 128 * 128, 128, 1)
+    args = [one] * 8 + [0, one, 0, one, 0, so, 1, 4, 3, 128, 128, 128, 1, 2, null]
+    assert L.mpsa_attn_fwd(*args) == -1                                                            # Hq % Hkv
+    args = [null] * 4 + [one] * 4 + [0, one, 0, one, 0, so, 1, 4, 2, 128, 128, 128, 1, 2, null]
+    assert L.mpsa_attn_fwd(*args) == -1                                                            # diag needs 4-bit Q
+    args = [one] * 8 + [0, one, 0, one, 0, so, 1, 4, 2, 128, 96, 128, 1, 2, null]
+    assert L.mpsa_attn_fwd(*args) == -3                                                            # D = 96
+    assert L.mpsa_e2m1_encode(null, 4, one, null) == -1
+    assert L.mpsa_e2m1_encode(null, 0, null, null) == 0                                            # empty is fine
+
+
+def test_python_entry_points_refuse_cpu_tensors_and_bad_arguments():
+    from ours.mxfp import MXFP4Tensor, MXScaleTensor
+    from ours.mxfp_attn import mxfp_attn
+    from ours.mxfp_attn_kernel import mxfp_attn_kernel
+    from ours.block_scaled_matmul import block_scaled_matmul, make_configs
+    x = torch.zeros(1, 2, 128, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        mxfp_attn(x, x, x)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        MXFP4Tensor(data=torch.zeros(4))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        MXScaleTensor(data=torch.ones(4))
+    with pytest.raises(AssertionError, match="seq_len"):
+        mxfp_attn(x[:, :, :64], x[:, :, :64], x[:, :, :64])
+    with pytest.raises(AssertionError, match="headdim"):
+        mxfp_attn(torch.zeros(1, 2, 128, 96), torch.zeros(1, 2, 128, 96), torch.zeros(1, 2, 128, 96))
+    with pytest.raises(ValueError):
+        MXFP4Tensor()
+    with pytest.raises(ValueError, match="Unsupported dtype"):
+        block_scaled_matmul(x, x, x, x, torch.int8, 256, 256, 128, make_configs("mxfp4"))
+    with pytest.raises(ValueError, match="Invalid block scale type"):
+        make_configs("nvfp4")
+    # packing is pure byte shuffling and keeps the reference's semantics on any device
+    t = MXFP4Tensor(data=torch.arange(16, dtype=torch.uint8).reshape(2, 8), dtype=torch.uint8)
+    p = t.to_packed_tensor(dim=1)
+    assert p.tolist() == [[0x10, 0x32, 0x54, 0x76], [0x98, 0xBA, 0xDC, 0xFE]]
+    assert torch.equal(t.unpack_packed_tensor(p, 1, (2, 8)), t.data)
+    odd = MXFP4Tensor(data=torch.arange(6, dtype=torch.uint8).reshape(2, 3), dtype=torch.uint8)
+    po = odd.to_packed_tensor(dim=1)
+    assert po.tolist() == [[0x10, 0x02], [0x43, 0x05]]
+    assert torch.equal(odd.unpack_packed_tensor(po, 1, (2, 3)), odd.data)
+    p0 = t.to_packed_tensor(dim=0)
+    assert p0.shape == (1, 8) and p0[0, 3] == (11 << 4 | 3)

@@ -1,0 +1,118 @@
+"""HIP fused attention against the CPU oracle's tile-by-tile MXFP attention.
+
+Bar (floating point): cosine similarity >= 0.999 over the flattened output and max-abs error <= 2e-2, on
+identical seeded inputs.  The oracle consumes the same quantized operands semantics (codes are bit-exact,
+see test_gpu_quantize.py), so what remains is float32 summation order inside the matrix cores, the
+hardware exp2 and the 16-bit rounding of P."""
+import pytest
+import torch
+
+import oracle as O
+from conftest import make_qkv
+from ours import _lib
+from ours.mxfp_attn import mxfp_attn
+from ours.mxfp_attn_kernel import mxfp_attn_kernel
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+COS_MIN, MAXABS_MAX = 0.999, 2e-2
+
+
+def _compare(got, want, what=""):
+    m = O.precision_metric(got.cpu(), want)
+    assert m["cos"] >= COS_MIN and m["max_abs"] <= MAXABS_MAX, f"{what}: {m}"
+    return m
+
+
+def _run(q, k, v, **kw):
+    return mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), **kw)
+
+
+@pytest.mark.parametrize("mode", ["diag", "mxfp4", "mxfp8"])
+def test_c1_cpu_plumbing_config(mode):
+    """B=1 H=8 N=1024 D=64, seed 0, causal, 64x64 tiles."""
+    q, k, v = make_qkv(1, 8, 8, 1024, 64, seed=0)
+    got = _run(q, k, v, is_causal=True, block_scale_type=mode, tile=64, output_dtype=torch.bfloat16)
+    want = O.attn_mx(q, k, v, tile=64, causal=True, mode=mode)
+    _compare(got, want, f"C1 {mode}")
+
+
+@pytest.mark.parametrize("D,tile", [(128, 128), (64, 128), (128, 64), (64, 64)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_all_kernel_variants_gqa(D, tile, causal):
+    q, k, v = make_qkv(2, 4, 2, 512, D, seed=10 + D + tile)
+    got = _run(q, k, v, is_causal=causal, block_scale_type="diag", tile=tile, output_dtype=torch.float32)
+    want = O.attn_mx(q, k, v, tile=tile, causal=causal, mode="diag", out_dtype=torch.float32)
+    _compare(got, want, f"D={D} tile={tile} causal={causal}")
+
+
+def test_c3_llama_shape_one_kv_group_with_outliers():
+    """B=1 Hq=32 Hkv=8 N=8192 D=128 causal, outlier channels, 128x128 tiles: the full problem runs on the GPU,
+    the oracle checks query heads 4..7 (KV head 1) and head 31."""
+    q, k, v = make_qkv(1, 32, 8, 8192, 128, seed=2, outliers=True)
+    got = _run(q, k, v, is_causal=True, block_scale_type="diag", tile=128, output_dtype=torch.bfloat16)
+    heads = [4, 5, 6, 7, 31]
+    want = O.attn_mx(q, k, v, tile=128, causal=True, mode="diag", heads=heads)
+    _compare(got[:, heads], want, "C3 heads")
+    assert torch.isfinite(got.float()).all()
+
+
+def test_full_size_properties():
+    """Size-independent checks at the C3 shape: V = 1 gives 1 everywhere; repeating K/V heads explicitly
+    (no GQA) gives the same bits as GQA indexing; the first causal row returns V[0]."""
+    q, k, v = make_qkv(1, 32, 8, 8192, 128, seed=2, outliers=True)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    ones = torch.ones_like(vd)
+    o = mxfp_attn_kernel(qd, kd, ones, is_causal=True, block_scale_type="diag", output_dtype=torch.float32)
+    assert (o - 1).abs().max().item() < 8e-3
+    a = mxfp_attn_kernel(qd, kd, vd, is_causal=True, block_scale_type="diag", output_dtype=torch.bfloat16)
+    b = mxfp_attn_kernel(qd, kd.repeat_interleave(4, dim=1), vd.repeat_interleave(4, dim=1), is_causal=True,
+                         block_scale_type="diag", output_dtype=torch.bfloat16)
+    assert torch.equal(a, b)
+    assert torch.equal(a[:, :, 0].cpu(), v[:, :, 0].repeat_interleave(4, dim=1))
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_ragged_length_tail_masking(causal):
+    """N = 1000 is not a multiple of the tile: the last key tile is masked, the last query rows are not stored."""
+    q, k, v = make_qkv(1, 4, 4, 1000, 128, seed=33, sigma=0.5)
+    got = _run(q, k, v, is_causal=causal, block_scale_type="diag", tile=128, output_dtype=torch.bfloat16)
+    assert got.shape == (1, 4, 1000, 128)
+    want = O.attn_mx(q, k, v, tile=128, causal=causal, mode="diag")
+    _compare(got, want, f"ragged causal={causal}")
+
+
+def test_fp16_inputs_nhd_layout_scale_and_public_entry():
+    q, k, v = make_qkv(1, 4, 2, 256, 64, seed=44, dtype=torch.float16)
+    want = O.attn_mx(q, k, v, tile=128, causal=True, mode="mxfp4", scale=0.2, out_dtype=torch.float16)
+    qn, kn, vn = (t.transpose(1, 2).contiguous().to(DEV) for t in (q, k, v))
+    got = mxfp_attn(qn, kn, vn, is_causal=True, scale=0.2, smooth_k=False, tensor_layout="NHD",
+                    output_dtype=torch.float16, block_scale_type="mxfp4", BLKQ=128)
+    assert got.shape == (1, 256, 4, 64) and got.dtype == torch.float16
+    _compare(got.transpose(1, 2), want, "fp16 NHD")
+    # float32 inputs run in fp16, like the reference wrapper
+    got32 = mxfp_attn(q.float().to(DEV), k.float().to(DEV), v.float().to(DEV), is_causal=True, scale=0.2,
+                      smooth_k=False, block_scale_type="mxfp4")
+    _compare(got32, want, "fp32 in")
+    # smooth_k (default of the public entry): same as the oracle on pre-smoothed K
+    want_s = O.attn_mx(q, k, v, tile=128, causal=False, mode="mxfp8", smooth_k=True, out_dtype=torch.float16)
+    got_s = mxfp_attn(q.to(DEV), k.to(DEV), v.to(DEV), block_scale_type="mxfp8")
+    _compare(got_s, want_s, "smooth_k")
+    # the reference's own 8-bit format
+    want_e5 = O.attn_mx(q, k, v, tile=64, causal=True, mode="diag", fmt8=O.FMT_E5M2, out_dtype=torch.float16)
+    got_e5 = mxfp_attn(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=True, smooth_k=False, block_scale_type="diag_e5", BLKQ=64)
+    _compare(got_e5, want_e5, "diag e5m2")
+
+
+def test_error_behaviour():
+    q, k, v = (t.to(DEV) for t in make_qkv(1, 4, 2, 128, 64, seed=1))
+    with pytest.raises(AssertionError, match="seq_len"):
+        mxfp_attn(q[:, :, :64], k[:, :, :64], v[:, :, :64])
+    with pytest.raises(ValueError, match="Invalid block scale type"):
+        mxfp_attn(q, k, v, block_scale_type="nvfp4")
+    with pytest.raises(ValueError, match="Unsupported dtype"):
+        mxfp_attn(q, k, v, output_dtype=torch.int8)
+    with pytest.raises(NotImplementedError):
+        mxfp_attn(q, k, v, skip_thresh=0.5)
+    with pytest.raises(AssertionError, match="multiple of key/value heads"):
+        mxfp_attn(q[:, :3], k, v)

@@ -1,0 +1,56 @@
+"""HIP format kernels behind MXFP4Tensor / MXScaleTensor against the golden vectors and the oracle (bit-exact)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from ours.mxfp import MXFP4Tensor, MXScaleTensor
+
+pytestmark = pytest.mark.gpu
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "mxfp_vectors.npz"))
+DEV = "cuda:0"
+
+
+def _f32(bits):
+    return torch.from_numpy(np.ascontiguousarray(bits)).view(torch.float32)
+
+
+def test_e2m1_encode_golden_and_oracle():
+    x = _f32(GOLD["e2m1_in_bits"])
+    got = MXFP4Tensor(data=x.to(DEV)).data.cpu()
+    assert torch.equal(got, torch.from_numpy(GOLD["e2m1_codes"]))
+    g = torch.Generator().manual_seed(1)
+    y = torch.randn(1 << 20, generator=g) * 3
+    assert torch.equal(MXFP4Tensor(data=y.to(DEV)).data.cpu(), O.encode_e2m1(y))
+    bits = torch.arange(0, 1 << 16, dtype=torch.int32).to(torch.int16)
+    for dt in (torch.bfloat16, torch.float16):
+        z = bits.view(dt).to(torch.float32)
+        assert torch.equal(MXFP4Tensor(data=z.to(DEV)).data.cpu(), O.encode_e2m1(z))
+
+
+def test_e2m1_decode_pack_roundtrip():
+    codes = torch.arange(16, dtype=torch.uint8, device=DEV)
+    dec = MXFP4Tensor(data=codes, dtype=torch.uint8).to(torch.float32).cpu()
+    assert np.array_equal(dec.view(torch.int32).numpy(), GOLD["e2m1_decode_all16_bits"])
+    t = MXFP4Tensor(size=(4, 6, 64), device=DEV).random()
+    assert t.data.max() < 16
+    for dim in (0, 1, 2):
+        p = t.to_packed_tensor(dim)
+        assert torch.equal(t.unpack_packed_tensor(p, dim, t.data.shape), t.data)
+    assert torch.equal(t.to_packed_tensor(2).cpu(), O.pack_fp4(t.data.cpu()))
+    assert torch.equal(MXFP4Tensor(data=t.to(torch.float32)).data, t.data & 0xF | (t.data & 8))
+
+
+def test_e8m0_golden():
+    x = _f32(GOLD["e8m0_in_bits"])
+    got = MXScaleTensor(data=x.to(DEV)).data.cpu()
+    assert torch.equal(got, torch.from_numpy(GOLD["e8m0_codes"]))
+    s = MXScaleTensor(size=(256,), device=DEV)
+    s.data = torch.arange(256, dtype=torch.uint8, device=DEV)
+    dec = s.to(torch.float32).cpu()
+    ref = _f32(GOLD["e8m0_decode_all256_bits"])
+    assert torch.equal(dec[:255], ref[:255]) and torch.isnan(dec[255])
+    r = MXScaleTensor(size=(1000,), device=DEV).random(low=1 / 16, high=16)
+    assert r.data.min() >= 123 and r.data.max() <= 131

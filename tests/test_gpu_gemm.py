@@ -1,0 +1,103 @@
+"""HIP block-scaled matmul against the CPU oracle (dequantise + matmul).
+
+Every product of two codes and two power-of-two scales is exact in float32, so the kernel and the oracle
+differ only by float32 summation order: tolerance atol = rtol = 1e-3, the reference's own
+(ours/block_scaled_matmul.py:440), against a float64 oracle; bf16 / f16 outputs add one rounding."""
+import pytest
+import torch
+
+import oracle as O
+from ours import _lib
+from ours.block_scaled_matmul import block_scaled_matmul, initialize_block_scaled_from_tensor, make_configs
+from ours.mxfp import MXFP4Tensor, MXScaleTensor
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TYPES = {"mxfp4": O.FMT_E2M1, "mxfp8": O.FMT_E4M3, "mxfp8e5": O.FMT_E5M2}
+
+
+def _operands(M, N, K, bst, seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(M, K, generator=g).bfloat16()
+    b = torch.randn(N, K, generator=g).bfloat16()
+    return a, b, initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst)
+
+
+@pytest.mark.parametrize("bst", ["mxfp4", "mxfp8", "mxfp8e5"])
+@pytest.mark.parametrize("shape", [(256, 256, 128), (512, 768, 1024), (256, 1024, 4096)])
+def test_quantize_then_matmul_matches_oracle(bst, shape):
+    M, N, K = shape
+    a, b, (ac, asc, bc, bsc, cfg) = _operands(M, N, K, bst, seed=M + K)
+    fmt = TYPES[bst]
+    oa, osa = O.quantize_mx(a, 1.0, fmt)
+    ob, osb = O.quantize_mx(b, 1.0, fmt)
+    assert torch.equal(ac.cpu(), oa) and torch.equal(bsc.cpu(), osb)
+    want = O.gemm_mx(oa, osa, ob, osb, fmt, acc_dtype=torch.float64)
+    got = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg).cpu()
+    torch.testing.assert_close(got.double(), want, atol=1e-3, rtol=1e-3)
+    got16 = block_scaled_matmul(ac, asc, bc, bsc, torch.bfloat16, M, N, K, cfg).cpu()
+    torch.testing.assert_close(got16.double(), want, atol=1e-3, rtol=2 ** -8)
+    gotf16 = block_scaled_matmul(ac, asc, bc, bsc, torch.float16, M, N, K, cfg).cpu()
+    torch.testing.assert_close(gotf16.double(), want, atol=1e-3, rtol=2 ** -10)
+
+
+def test_random_codes_and_scales_exact_integers():
+    """Reference-tutorial style operands (random codes, random scales; ours/block_scaled_matmul.py:423-429):
+    with scale exponents >= 0 the result is an integer/4 that float32 holds exactly -> bit-exact check."""
+    M, N, K = 256, 256, 256
+    a = MXFP4Tensor(size=(M, K), device=DEV).random()
+    b = MXFP4Tensor(size=(N, K), device=DEV).random()
+    sa = MXScaleTensor(size=(M, K // 32), device=DEV).random(low=1, high=8)
+    sb = MXScaleTensor(size=(N, K // 32), device=DEV).random(low=1, high=8)
+    got = block_scaled_matmul(a.to_packed_tensor(dim=1), sa.data, b.to_packed_tensor(dim=1), sb.data, torch.float32,
+                              M, N, K, make_configs("mxfp4")).cpu()
+    want = O.gemm_mx(O.pack_fp4(a.data.cpu()), sa.data.cpu(), O.pack_fp4(b.data.cpu()), sb.data.cpu(), O.FMT_E2M1,
+                     acc_dtype=torch.float64)
+    assert torch.equal(got.double(), want)
+    # the helper classes' own decode gives the same reference (ours/block_scaled_matmul.py:382-392)
+    ref = (a.to(torch.float32) * sa.to(torch.float32).repeat_interleave(32, 1)).cpu() @ \
+          (b.to(torch.float32) * sb.to(torch.float32).repeat_interleave(32, 1)).cpu().T
+    assert torch.equal(got, ref)
+
+
+def test_identity_like_operand_selects_rows():
+    """B = 2^k * one-hot rows: C[m, n] must be the dequantised A[m, k_n] -- catches any k / row permutation."""
+    M, N, K = 256, 256, 512
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(M, K, generator=g).bfloat16()
+    b = torch.zeros(N, K)
+    cols = torch.randint(0, K, (N,), generator=g)
+    b[torch.arange(N), cols] = 4.0
+    ac, asc, bc, bsc, cfg = initialize_block_scaled_from_tensor(a.to(DEV), b.bfloat16().to(DEV), "mxfp8")
+    got = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg).cpu()
+    adq = O.dequantize_mx(*O.quantize_mx(a, 1.0, O.FMT_E4M3), O.FMT_E4M3)
+    assert torch.equal(got, adq[:, cols] * 4.0)
+
+
+@pytest.mark.parametrize("bst", ["mxfp4", "mxfp8"])
+def test_c2_full_size_rows_against_oracle_and_linearity(bst):
+    """8192^3: a slab of 256 rows and a slab of 256 columns against the float64 oracle, plus a checksum:
+    sum_n C[m, n] must equal dq(A)[m, :] . sum_n dq(B)[n, :]."""
+    M = N = K = 8192
+    a, b, (ac, asc, bc, bsc, cfg) = _operands(M, N, K, bst, seed=1)
+    fmt = TYPES[bst]
+    got = block_scaled_matmul(ac, asc, bc, bsc, torch.bfloat16, M, N, K, cfg)
+    ac_, asc_, bc_, bsc_ = ac.cpu(), asc.cpu(), bc.cpu(), bsc.cpu()
+    rows = slice(4096 + 128, 4096 + 384)
+    want_r = O.gemm_mx(ac_[rows], asc_[rows], bc_, bsc_, fmt, acc_dtype=torch.float64)
+    torch.testing.assert_close(got[rows].cpu().double(), want_r, atol=1e-3, rtol=2 ** -8)
+    cols = slice(7936, 8192)
+    want_c = O.gemm_mx(ac_, asc_, bc_[cols], bsc_[cols], fmt, acc_dtype=torch.float64)
+    torch.testing.assert_close(got[:, cols].cpu().double(), want_c, atol=1e-3, rtol=2 ** -8)
+    got32 = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg)
+    adq = O.dequantize_mx(ac_, asc_, fmt, torch.float64)
+    bsum = O.dequantize_mx(bc_, bsc_, fmt, torch.float64).sum(dim=0)
+    torch.testing.assert_close(got32.double().sum(dim=1).cpu(), adq @ bsum, atol=0.5, rtol=1e-4)
+
+
+def test_errors():
+    ac, asc, bc, bsc, cfg = _operands(256, 256, 128, "mxfp4", 0)[2]
+    with pytest.raises(ValueError, match="Unsupported dtype"):
+        block_scaled_matmul(ac, asc, bc, bsc, torch.int32, 256, 256, 128, cfg)
+    with pytest.raises(_lib.MpsaError, match="multiples of 256"):
+        block_scaled_matmul(ac[:128], asc[:128], bc, bsc, torch.float32, 128, 256, 128, cfg)
