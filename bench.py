@@ -74,21 +74,22 @@ def time_events(fn, iters):
 
 
 def cpu_baseline(q, k, v, tile, D):
-    """The CPU oracle (a port of the reference's fake-quant path) on one KV group of the workload."""
+    """The CPU oracle (a port of the reference's fake-quant path) on the first 8192 positions of the workload
+    (all of it for C1/C3), every head."""
     import oracle as O
     Hq, Hkv = q.shape[1], k.shape[1]
-    group = Hq // Hkv
+    group = Hq
     n = min(q.shape[2], 8192)
-    qs = q[:, :group, :n].cpu()
-    ks = k[:, :1, :n].cpu()
-    vs = v[:, :1, :n].cpu()
+    qs = q[:, :, :n].cpu()
+    ks = k[:, :, :n].cpu()
+    vs = v[:, :, :n].cpu()
     t0 = time.perf_counter()
     O.attn_mx(qs, ks, vs, tile=tile, causal=True, mode="diag")
     dt = time.perf_counter() - t0
     flops = 2.0 * qs.shape[0] * group * n * n * D
     return {
         "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-        "sample": f"oracle.attn_mx (quantize+dequantize+tiled attention, torch CPU) on {group} query heads / 1 KV head, "
+        "sample": f"oracle.attn_mx (quantize+dequantize+tiled attention, torch CPU) on {group} query heads / {Hkv} KV heads, "
                   f"N={n}, D={D}, causal, diag mode: {dt:.2f} s",
         "seconds": dt,
     }

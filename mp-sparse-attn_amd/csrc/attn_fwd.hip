@@ -11,8 +11,9 @@
 // Mapping.  A workgroup owns one TILE-query tile; each of its TILE/32 waves owns 32 queries and walks all
 // keys of every tile.  Both products are computed transposed so that a lane always owns ONE query:
 //   S^T = K Q^T   on v_mfma_scale_f32_32x32x64_f8f6f4: lane (h = lane/32, r = lane%32) of the K operand
-//                 supplies one 32-element MX block of key row r with its E8M0 byte, the Q operand the
-//                 same for query r; the result leaves query r's scores for 16 keys per 32-key block in
+//                 supplies 32 elements of key row r and the E8M0 byte of MX block h of the 64-wide step
+//                 (4-bit: the lane's registers are block h; 8-bit: registers 0-3 of both lane halves are
+//                 block 0, registers 4-7 block 1), the Q operand the same for query r; the result leaves query r's scores for 16 keys per 32-key block in
 //                 that lane's registers, so the row maximum is a register reduction plus one exchange
 //                 with lane^32, and running max / sum / rescale factors are plain per-lane scalars.
 //   O^T += V^T P^T on v_mfma_f32_32x32x16_{bf16,f16}: the P^T operand of lane (h, r) is exactly the eight
@@ -127,8 +128,9 @@ __global__ __launch_bounds__(TILE * 2, 1) void attn_fwd_kernel(AttnArgs a) {
     if (need8) {
 #pragma unroll
         for (int s = 0; s < G::SST; ++s) {
-            const v4i x0 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + (2 * s + h) * 32);
-            const v4i x1 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + (2 * s + h) * 32 + 16);
+            // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
+            const v4i x0 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + s * 64 + h * 16);
+            const v4i x1 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + s * 64 + h * 16 + 32);
             q8f[s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
         }
         const uint32_t sw = (D == 128) ? *reinterpret_cast<const uint32_t*>(a.qs8 + q_row * 4)
@@ -209,9 +211,9 @@ __global__ __launch_bounds__(TILE * 2, 1) void attn_fwd_kernel(AttnArgs a) {
             if (cur8) {
 #pragma unroll
                 for (int s = 0; s < G::SST; ++s) {
-                    const uint8_t* p = kl + krow * G::PK8 + (2 * s + h) * 32;
+                    const uint8_t* p = kl + krow * G::PK8 + s * 64 + h * 16;
                     const v4i x0 = *reinterpret_cast<const v4i*>(p);
-                    const v4i x1 = *reinterpret_cast<const v4i*>(p + 16);
+                    const v4i x1 = *reinterpret_cast<const v4i*>(p + 32);
                     const v8i kf = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
                     st[kb] = score_mfma8<FMT8>(kf, q8f[s], st[kb], s, ksc, qsc8);
                 }

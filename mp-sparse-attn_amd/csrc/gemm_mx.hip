@@ -8,9 +8,11 @@
 //
 // Mapping.  A workgroup of four waves owns a 256x256 tile of C; each wave owns 128x128 as a 4x4 grid of
 // v_mfma_scale_f32_32x32x64_f8f6f4 accumulators (256 accumulator registers).  For that instruction
-// lane (h = lane/32, r = lane%32) supplies 32 consecutive K elements -- exactly one MX block -- of row r
-// of its operand together with that block's E8M0 byte, so the row-major HBM layout is already the
-// operand layout.  K advances 64 bytes of codes per row per stage (128 E2M1 or 64 8-bit elements).
+// lane (h = lane/32, r = lane%32) supplies 32 K elements of row r of its operand and the E8M0 byte of MX
+// block h of the 64-element step.  With 4-bit elements the lane's four registers are exactly block h;
+// with 8-bit elements registers 0-3 of the two lane halves together are block 0 and registers 4-7 block 1
+// (each half holds 16 bytes of either block).  Either way fragments are plain 16-byte pieces of the
+// row-major HBM layout.  K advances 64 bytes of codes per row per stage (128 E2M1 or 64 8-bit elements).
 // Stages are double-buffered in LDS with rows padded from 64 to 80 bytes: the 16 lanes of a 128-bit
 // LDS access phase then fall into 16 distinct 4-bank groups.  Wave tiles of 128x128 keep LDS reads at
 // 8 operand fragments per 16 matrix instructions.
@@ -131,10 +133,12 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
                     fa[i] = (v8i){xa[0], xa[1], xa[2], xa[3], 0, 0, 0, 0};
                     fb[i] = (v8i){xb[0], xb[1], xb[2], xb[3], 0, 0, 0, 0};
                 } else {
-                    const v4i xa0 = *reinterpret_cast<const v4i*>(pa + h * 32);
-                    const v4i xa1 = *reinterpret_cast<const v4i*>(pa + h * 32 + 16);
-                    const v4i xb0 = *reinterpret_cast<const v4i*>(pb + h * 32);
-                    const v4i xb1 = *reinterpret_cast<const v4i*>(pb + h * 32 + 16);
+                    // 8-bit operands: registers 0-3 of both lane halves form MX block 0 (scaled by the byte
+                    // lane half 0 supplies), registers 4-7 form block 1 (scaled by lane half 1's byte)
+                    const v4i xa0 = *reinterpret_cast<const v4i*>(pa + h * 16);
+                    const v4i xa1 = *reinterpret_cast<const v4i*>(pa + h * 16 + 32);
+                    const v4i xb0 = *reinterpret_cast<const v4i*>(pb + h * 16);
+                    const v4i xb1 = *reinterpret_cast<const v4i*>(pb + h * 16 + 32);
                     fa[i] = (v8i){xa0[0], xa0[1], xa0[2], xa0[3], xa1[0], xa1[1], xa1[2], xa1[3]};
                     fb[i] = (v8i){xb0[0], xb0[1], xb0[2], xb0[3], xb1[0], xb1[1], xb1[2], xb1[3]};
                 }
