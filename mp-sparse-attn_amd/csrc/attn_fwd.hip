@@ -19,9 +19,14 @@
 //   O^T += V^T P^T on v_mfma_f32_32x32x16_{bf16,f16}: the P^T operand of lane (h, r) is exactly the eight
 //                 scores that lane already holds (keys are contracted in the order the score MFMA left
 //                 them); V is pre-arranged by mpsa_v_tiles to match, one 16-byte LDS read per operand.
-// K codes, K scales and the V tile are staged through LDS (K rows padded by 16 bytes so that 128-bit
-// reads are bank-conflict free; the V tile is read lane-contiguously), double-buffered, with the next
-// tile's global loads issued before the current tile's math.
+// Staging.  K codes and the V tile travel HBM/L2 -> LDS with direct-to-LDS loads (global_load_lds_dwordx4: each
+// lane names a 16-byte global source, the wave's 64 pieces land contiguously in LDS), so they cost neither
+// registers nor LDS-write instructions.  The V tile is already in operand order (a flat copy); K rows keep their
+// row-major order but the 16-byte chunks of a row are XOR-swizzled with the row index, which makes the 128-bit
+// operand reads of 16 consecutive rows hit 16 distinct 4-bank groups.  K is double-buffered (tile j+1 streams in
+// during tile j), V is single-buffered (it streams in during the score MFMAs and the softmax of the same tile);
+// K scales are read straight from global memory one tile ahead.  64 KiB of LDS and at most 256 registers per
+// workgroup let two workgroups share a CU, so one's matrix instructions overlap the other's softmax VALU work.
 #include "mpsa_common.h"
 
 namespace {
@@ -64,19 +69,26 @@ struct Geom {
     static constexpr int KB = TILE / 32;          // 32-key blocks per tile
     static constexpr int SST = D / 64;            // score matrix instructions along D
     static constexpr int NDB = D / 32;            // 32-wide output dim blocks
-    static constexpr int PK4 = D / 2 + 16;        // LDS row pitch of 4-bit K rows
-    static constexpr int PK8 = D + 16;            // LDS row pitch of 8-bit K rows
-    static constexpr int K_BYTES = TILE * PK8;
-    static constexpr int S_BYTES = TILE * 4;
+    static constexpr int ROW4 = D / 2, ROW8 = D;  // bytes per K row
+    static constexpr int CPR4 = ROW4 / 16, CPR8 = ROW8 / 16;          // 16-byte chunks per K row (2|4, 4|8)
+    static constexpr int SH4 = CPR4 == 2 ? 3 : 2;                     // log2(rows per 256 bytes)
+    static constexpr int SH8 = CPR8 == 4 ? 2 : 1;
+    static constexpr int K_BYTES = TILE * ROW8;   // one K buffer holds a tile in either precision
     static constexpr int V_BYTES = TILE * D * 2;
-    static constexpr int BUF = K_BYTES + S_BYTES + V_BYTES;
-    static constexpr int KC4 = TILE * (D / 2) / 16 / NT;   // 16-byte K chunks per thread, 4-bit
-    static constexpr int KC8 = 2 * KC4;
-    static constexpr int VC = V_BYTES / 16 / NT;
+    static constexpr int SMEM = 2 * K_BYTES + V_BYTES;
+    static constexpr int KI4 = TILE * ROW4 / 1024 / NW;               // direct-load instructions per wave, 4-bit K
+    static constexpr int KI8 = TILE * ROW8 / 1024 / NW;
+    static constexpr int VI = V_BYTES / 1024 / NW;
 };
 
+// One wave-wide direct-to-LDS load: lane l copies 16 bytes from its own global address to lds_wave_base + 16*l.
+__device__ __forceinline__ void load16_to_lds(const uint8_t* gsrc, uint8_t* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
 template <int D, int TILE, int PVT, int FMT8>
-__global__ __launch_bounds__(TILE * 2, 1) void attn_fwd_kernel(AttnArgs a) {
+__global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     typedef Geom<D, TILE> G;
     typedef PV<PVT> P;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -104,76 +116,78 @@ __global__ __launch_bounds__(TILE * 2, 1) void attn_fwd_kernel(AttnArgs a) {
     const int q_local = 32 * w + r;
     const int64_t q_row = qhead_row + (int64_t)i * TILE + q_local;
 
-    const bool need4 = a.mode != MPSA_MODE_MXFP8;
-    const bool need8 = a.mode != MPSA_MODE_MXFP4;
-
-    // ---- Q fragments stay in registers for the whole tile row ----
-    v8i q4f[G::SST], q8f[G::SST];
-    int qsc4 = 0, qsc8 = 0;
+    // ---- Q fragments of the current tile precision stay in registers; they are re-read from global memory when
+    //      the precision changes (once per workgroup in causal "diag" runs: the diagonal tile comes last) ----
+    v8i qf[G::SST];
+    int qsc = 0;
+    auto load_q = [&](bool is8) __attribute__((always_inline)) {
+        if (is8) {
 #pragma unroll
-    for (int s = 0; s < G::SST; ++s) {
-        q4f[s] = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
-        q8f[s] = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
-    }
-    if (need4) {
-#pragma unroll
-        for (int s = 0; s < G::SST; ++s) {
-            const v4i x = *reinterpret_cast<const v4i*>(a.q4 + q_row * (D / 2) + (2 * s + h) * 16);
-            q4f[s] = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
-        }
-        const uint32_t sw = (D == 128) ? *reinterpret_cast<const uint32_t*>(a.qs4 + q_row * 4)
-                                       : (uint32_t)*reinterpret_cast<const uint16_t*>(a.qs4 + q_row * 2);
-        qsc4 = (int)(sw >> (8 * h));
-    }
-    if (need8) {
-#pragma unroll
-        for (int s = 0; s < G::SST; ++s) {
-            // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
-            const v4i x0 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + s * 64 + h * 16);
-            const v4i x1 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + s * 64 + h * 16 + 32);
-            q8f[s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-        }
-        const uint32_t sw = (D == 128) ? *reinterpret_cast<const uint32_t*>(a.qs8 + q_row * 4)
-                                       : (uint32_t)*reinterpret_cast<const uint16_t*>(a.qs8 + q_row * 2);
-        qsc8 = (int)(sw >> (8 * h));
-    }
-
-    // ---- staging registers: next tile's K codes, K scales, V ----
-    v4i rk[G::KC8], rv[G::VC];
-#pragma unroll
-    for (int c = 0; c < G::KC8; ++c) rk[c] = (v4i){0, 0, 0, 0};
-    uint32_t rs = 0;
-    auto tile_is8 = [&](int j) { return a.mode == MPSA_MODE_MXFP8 || (a.mode == MPSA_MODE_DIAG && j == i); };
-    auto load_tile = [&](int j, bool is8) __attribute__((always_inline)) {
-        const int64_t krow0 = khead_row + (int64_t)j * TILE;
-        const uint8_t* src = is8 ? a.k8 + krow0 * D : a.k4 + krow0 * (D / 2);
-        const int nchunk = is8 ? G::KC8 : G::KC4;
-#pragma unroll
-        for (int c = 0; c < G::KC8; ++c)
-            if (c < nchunk) rk[c] = *reinterpret_cast<const v4i*>(src + (int64_t)(tid + G::NT * c) * 16);
-        if (tid < TILE) {
-            const uint8_t* sp = (is8 ? a.ks8 : a.ks4) + (krow0 + tid) * (D / 32);
-            rs = (D == 128) ? *reinterpret_cast<const uint32_t*>(sp) : (uint32_t)*reinterpret_cast<const uint16_t*>(sp);
-        }
-        const uint8_t* vsrc = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)j * TILE) * (D * 2);
-#pragma unroll
-        for (int c = 0; c < G::VC; ++c) rv[c] = *reinterpret_cast<const v4i*>(vsrc + (int64_t)(tid + G::NT * c) * 16);
-    };
-    auto store_tile = [&](int buf, bool is8) __attribute__((always_inline)) {
-        uint8_t* kb_ = smem + buf * G::BUF;
-        const int cpr_shift = is8 ? (D == 128 ? 3 : 2) : (D == 128 ? 2 : 1);   // log2(16-byte chunks per K row)
-        const int pitch = is8 ? G::PK8 : G::PK4;
-        const int nchunk = is8 ? G::KC8 : G::KC4;
-#pragma unroll
-        for (int c = 0; c < G::KC8; ++c)
-            if (c < nchunk) {
-                const int q = tid + G::NT * c;
-                *reinterpret_cast<v4i*>(kb_ + (q >> cpr_shift) * pitch + (q & ((1 << cpr_shift) - 1)) * 16) = rk[c];
+            for (int s = 0; s < G::SST; ++s) {
+                // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
+                const v4i x0 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + s * 64 + h * 16);
+                const v4i x1 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + s * 64 + h * 16 + 32);
+                qf[s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
             }
-        if (tid < TILE) *reinterpret_cast<uint32_t*>(kb_ + G::K_BYTES + tid * 4) = rs;
-        uint8_t* vb = kb_ + G::K_BYTES + G::S_BYTES;
+        } else {
 #pragma unroll
-        for (int c = 0; c < G::VC; ++c) *reinterpret_cast<v4i*>(vb + (tid + G::NT * c) * 16) = rv[c];
+            for (int s = 0; s < G::SST; ++s) {
+                const v4i x = *reinterpret_cast<const v4i*>(a.q4 + q_row * (D / 2) + (2 * s + h) * 16);
+                qf[s] = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+            }
+        }
+        const uint8_t* qs = (is8 ? a.qs8 : a.qs4) + q_row * (D / 32);
+        const uint32_t sw = (D == 128) ? *reinterpret_cast<const uint32_t*>(qs) : (uint32_t)*reinterpret_cast<const uint16_t*>(qs);
+        qsc = (int)(sw >> (8 * h));
+    };
+
+    // ---- staging: direct-to-LDS loads of K (swizzled rows, double-buffered) and V (flat, single buffer) ----
+    uint8_t* const kbuf0 = smem;
+    uint8_t* const vbuf = smem + 2 * G::K_BYTES;
+    auto tile_is8 = [&](int j) { return a.mode == MPSA_MODE_MXFP8 || (a.mode == MPSA_MODE_DIAG && j == i); };
+    auto issue_k = [&](int j, bool is8) __attribute__((always_inline)) {
+        const int64_t krow0 = khead_row + (int64_t)j * TILE;
+        uint8_t* dst = kbuf0 + (j & 1) * G::K_BYTES;
+        if (is8) {
+            const uint8_t* src = a.k8 + krow0 * G::ROW8;
+#pragma unroll
+            for (int c = 0; c < G::KI8; ++c) {
+                const int ci = w * G::KI8 + c;
+                const int p = ci * 64 + lane;
+                const int row = p / G::CPR8, slot = p % G::CPR8;
+                const int cb = slot ^ ((row >> G::SH8) & (G::CPR8 - 1));
+                load16_to_lds(src + row * G::ROW8 + cb * 16, dst + ci * 1024);
+            }
+        } else {
+            const uint8_t* src = a.k4 + krow0 * G::ROW4;
+#pragma unroll
+            for (int c = 0; c < G::KI4; ++c) {
+                const int ci = w * G::KI4 + c;
+                const int p = ci * 64 + lane;
+                const int row = p / G::CPR4, slot = p % G::CPR4;
+                const int cb = slot ^ ((row >> G::SH4) & (G::CPR4 - 1));
+                load16_to_lds(src + row * G::ROW4 + cb * 16, dst + ci * 1024);
+            }
+        }
+    };
+    auto issue_v = [&](int j) __attribute__((always_inline)) {
+        const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)j * TILE) * (D * 2);
+#pragma unroll
+        for (int c = 0; c < G::VI; ++c) {
+            const int ci = w * G::VI + c;
+            load16_to_lds(src + ci * 1024 + lane * 16, vbuf + ci * 1024);
+        }
+    };
+    // E8M0 bytes of this lane's key rows (32*kb + r), shifted so that byte 0 / byte 2 belong to MX block h / 2+h
+    int ksc_next[G::KB];
+    auto load_kscales = [&](int j, bool is8) __attribute__((always_inline)) {
+        const uint8_t* sp = (is8 ? a.ks8 : a.ks4) + (khead_row + (int64_t)j * TILE + r) * (D / 32);
+#pragma unroll
+        for (int kb = 0; kb < G::KB; ++kb) {
+            const uint32_t sw = (D == 128) ? *reinterpret_cast<const uint32_t*>(sp + kb * 32 * (D / 32))
+                                           : (uint32_t)*reinterpret_cast<const uint16_t*>(sp + kb * 32 * (D / 32));
+            ksc_next[kb] = (int)(sw >> (8 * h));
+        }
     };
 
     v16f acc[G::NDB];
@@ -186,19 +200,26 @@ __global__ __launch_bounds__(TILE * 2, 1) void attn_fwd_kernel(AttnArgs a) {
 
     const int j_end = a.causal ? i + 1 : a.nt;
     bool cur8 = tile_is8(0);
-    load_tile(0, cur8);
-    store_tile(0, cur8);
-    __syncthreads();
+    issue_k(0, cur8);
+    load_kscales(0, cur8);
+    load_q(cur8);
 
     for (int j = 0; j < j_end; ++j) {
-        const int buf = j & 1;
+        // every wave is done with tile j-1: the V buffer and the other K buffer are free; K_j is in flight or landed
+        __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): this wave's pieces of K_j (and its scales) have landed
+        __syncthreads();
         const bool nxt = j + 1 < j_end;
         const bool nxt8 = nxt ? tile_is8(j + 1) : false;
-        if (nxt) load_tile(j + 1, nxt8);
+        int ksc[G::KB];
+#pragma unroll
+        for (int kb = 0; kb < G::KB; ++kb) ksc[kb] = ksc_next[kb];
+        issue_v(j);
+        if (nxt) {
+            issue_k(j + 1, nxt8);
+            load_kscales(j + 1, nxt8);
+        }
 
-        const uint8_t* kl = smem + buf * G::BUF;
-        const uint8_t* sl = kl + G::K_BYTES;
-        const uint8_t* vl = sl + G::S_BYTES;
+        const uint8_t* kl = kbuf0 + (j & 1) * G::K_BYTES;
 
         // ---- S^T = K Q^T ----
         v16f st[G::KB];
@@ -207,22 +228,24 @@ __global__ __launch_bounds__(TILE * 2, 1) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) st[kb][e] = 0.0f;
             const int krow = 32 * kb + r;
-            const int ksc = (int)(*reinterpret_cast<const uint32_t*>(sl + krow * 4) >> (8 * h));
             if (cur8) {
+                const int f = (krow >> G::SH8) & (G::CPR8 - 1);
 #pragma unroll
                 for (int s = 0; s < G::SST; ++s) {
-                    const uint8_t* p = kl + krow * G::PK8 + s * 64 + h * 16;
-                    const v4i x0 = *reinterpret_cast<const v4i*>(p);
-                    const v4i x1 = *reinterpret_cast<const v4i*>(p + 32);
+                    // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
+                    const uint8_t* p = kl + krow * G::ROW8;
+                    const v4i x0 = *reinterpret_cast<const v4i*>(p + (((4 * s + h) ^ f) * 16));
+                    const v4i x1 = *reinterpret_cast<const v4i*>(p + (((4 * s + h + 2) ^ f) * 16));
                     const v8i kf = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-                    st[kb] = score_mfma8<FMT8>(kf, q8f[s], st[kb], s, ksc, qsc8);
+                    st[kb] = score_mfma8<FMT8>(kf, qf[s], st[kb], s, ksc[kb], qsc);
                 }
             } else {
+                const int f = (krow >> G::SH4) & (G::CPR4 - 1);
 #pragma unroll
                 for (int s = 0; s < G::SST; ++s) {
-                    const v4i x = *reinterpret_cast<const v4i*>(kl + krow * G::PK4 + (2 * s + h) * 16);
+                    const v4i x = *reinterpret_cast<const v4i*>(kl + krow * G::ROW4 + (((2 * s + h) ^ f) * 16));
                     const v8i kf = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
-                    st[kb] = score_mfma4(kf, q4f[s], st[kb], s, ksc, qsc4);
+                    st[kb] = score_mfma4(kf, qf[s], st[kb], s, ksc[kb], qsc);
                 }
             }
         }
@@ -269,6 +292,10 @@ __global__ __launch_bounds__(TILE * 2, 1) void attn_fwd_kernel(AttnArgs a) {
                 for (int e = 0; e < 16; ++e) acc[d][e] *= alpha;
         }
 
+        // V_j (and K_{j+1}) pieces issued by this wave have landed; after the barrier everybody's have
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+
         // ---- O^T += V^T P^T ----
 #pragma unroll
         for (int kb = 0; kb < G::KB; ++kb)
@@ -280,14 +307,12 @@ __global__ __launch_bounds__(TILE * 2, 1) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
                 for (int d = 0; d < G::NDB; ++d) {
                     const typename P::vec vf =
-                        *reinterpret_cast<const typename P::vec*>(vl + (((kb * 2 + c) * G::NDB + d) * 64 + lane) * 16);
+                        *reinterpret_cast<const typename P::vec*>(vbuf + (((kb * 2 + c) * G::NDB + d) * 64 + lane) * 16);
                     acc[d] = P::mfma(vf, pf, acc[d]);
                 }
             }
-
-        if (nxt) store_tile(buf ^ 1, nxt8);
+        if (nxt && nxt8 != cur8) load_q(nxt8);
         cur8 = nxt8;
-        __syncthreads();
     }
 
     // ---- epilogue: O = acc / l ; register e of lane (h, r): dim 32*db + 8*(e/4) + 4*h + e%4 of query r ----
@@ -323,7 +348,7 @@ __global__ __launch_bounds__(TILE * 2, 1) void attn_fwd_kernel(AttnArgs a) {
 template <int D, int TILE, int PVT, int FMT8>
 int launch_one(const AttnArgs& a, hipStream_t st) {
     typedef Geom<D, TILE> G;
-    constexpr int smem = 2 * G::BUF;
+    constexpr int smem = G::SMEM;
     static bool attr_set = false;      // idempotent; a race only repeats the same call
     auto kern = attn_fwd_kernel<D, TILE, PVT, FMT8>;
     if (!attr_set) {
