@@ -43,14 +43,39 @@ struct AttnArgs {
 template <int PVT> struct PV;
 template <> struct PV<MPSA_BF16> {
     typedef v8bf vec;
-    typedef __bf16 elem;
+    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
     static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ v2 pack(float x, float y) { return (v2){(__bf16)x, (__bf16)y}; }
+    // c + p.x + p.y with the 16-bit values the P.V product will see
+    static __device__ __forceinline__ float add2(v2 p, float c) { return __builtin_amdgcn_fdot2_f32_bf16(p, (v2){(__bf16)1.0f, (__bf16)1.0f}, c, false); }
 };
 template <> struct PV<MPSA_F16> {
     typedef v8h vec;
-    typedef _Float16 elem;
+    typedef _Float16 v2 __attribute__((ext_vector_type(2)));
     static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ v2 pack(float x, float y) { return (v2){(_Float16)x, (_Float16)y}; }
+    static __device__ __forceinline__ float add2(v2 p, float c) { return __builtin_amdgcn_fdot2(p, (v2){(_Float16)1.0f, (_Float16)1.0f}, c, false); }
 };
+
+// Exchange between the two lanes (l, l^32) that share one query.  v_permlane32_swap swaps lanes 32-63 of its first
+// register with lanes 0-31 of its second; fed two copies of x, every lane ends up holding both halves' values.
+// Written as inline assembly because both registers are outputs (the compiler builtin of this toolchain returns
+// the first register for both results); the s_nop's cover the instruction's read/write wait states.
+__device__ __forceinline__ void lane_pair(float x, float& a, float& b) {
+    a = x;
+    b = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float max_lane_pair(float x) {
+    float a, b;
+    lane_pair(x, a, b);
+    return __builtin_fmaxf(a, b);
+}
+__device__ __forceinline__ float sum_lane_pair(float x) {
+    float a, b;
+    lane_pair(x, a, b);
+    return a + b;
+}
 
 template <int FMT8>
 __device__ __forceinline__ v16f score_mfma8(v8i k, v8i q, v16f c, int sel, int ks, int qs) {
@@ -195,8 +220,15 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     for (int d = 0; d < G::NDB; ++d)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[d][e] = 0.0f;
-    float m_run = -__builtin_inff();
+    // Running reference maximum of this lane's query, kept LAZILY: it moves only when a tile's maximum exceeds
+    // it by more than REBASE (so P stays below 2^REBASE), and -m_run rides into the score MFMA as its C operand,
+    // which makes the matrix core deliver S - m_run: the softmax costs no subtract and (almost) no rescale.
+    constexpr float REBASE = 5.0f;
+    float m_run = 0.0f;
     float l_run = 0.0f;
+    v16f negm;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) negm[e] = 0.0f;
 
     const int j_end = a.causal ? i + 1 : a.nt;
     bool cur8 = tile_is8(0);
@@ -205,7 +237,7 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     load_q(cur8);
 
     for (int j = 0; j < j_end; ++j) {
-        // every wave is done with tile j-1: the V buffer and the other K buffer are free; K_j is in flight or landed
+        // every wave is done with tile j-1: the V buffer and the other K buffer are free
         __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): this wave's pieces of K_j (and its scales) have landed
         __syncthreads();
         const bool nxt = j + 1 < j_end;
@@ -221,31 +253,46 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
 
         const uint8_t* kl = kbuf0 + (j & 1) * G::K_BYTES;
 
-        // ---- S^T = K Q^T ----
+        // ---- S^T - m_run = K Q^T + (-m_run) ----
         v16f st[G::KB];
+        if (cur8) {
+            v8i kf[G::KB][G::SST];
 #pragma unroll
-        for (int kb = 0; kb < G::KB; ++kb) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) st[kb][e] = 0.0f;
-            const int krow = 32 * kb + r;
-            if (cur8) {
+            for (int kb = 0; kb < G::KB; ++kb) {
+                const int krow = 32 * kb + r;
                 const int f = (krow >> G::SH8) & (G::CPR8 - 1);
+                const uint8_t* p = kl + krow * G::ROW8;
 #pragma unroll
                 for (int s = 0; s < G::SST; ++s) {
                     // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
-                    const uint8_t* p = kl + krow * G::ROW8;
                     const v4i x0 = *reinterpret_cast<const v4i*>(p + (((4 * s + h) ^ f) * 16));
                     const v4i x1 = *reinterpret_cast<const v4i*>(p + (((4 * s + h + 2) ^ f) * 16));
-                    const v8i kf = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-                    st[kb] = score_mfma8<FMT8>(kf, qf[s], st[kb], s, ksc[kb], qsc);
+                    kf[kb][s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
                 }
-            } else {
+            }
+#pragma unroll
+            for (int kb = 0; kb < G::KB; ++kb) {
+                st[kb] = score_mfma8<FMT8>(kf[kb][0], qf[0], negm, 0, ksc[kb], qsc);
+#pragma unroll
+                for (int s = 1; s < G::SST; ++s) st[kb] = score_mfma8<FMT8>(kf[kb][s], qf[s], st[kb], s, ksc[kb], qsc);
+            }
+        } else {
+            v4i kf[G::KB][G::SST];
+#pragma unroll
+            for (int kb = 0; kb < G::KB; ++kb) {
+                const int krow = 32 * kb + r;
                 const int f = (krow >> G::SH4) & (G::CPR4 - 1);
 #pragma unroll
+                for (int s = 0; s < G::SST; ++s)
+                    kf[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * G::ROW4 + (((2 * s + h) ^ f) * 16));
+            }
+#pragma unroll
+            for (int kb = 0; kb < G::KB; ++kb) {
+#pragma unroll
                 for (int s = 0; s < G::SST; ++s) {
-                    const v4i x = *reinterpret_cast<const v4i*>(kl + krow * G::ROW4 + (((2 * s + h) ^ f) * 16));
-                    const v8i kf = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
-                    st[kb] = score_mfma4(kf, qf[s], st[kb], s, ksc[kb], qsc);
+                    const v4i x = kf[kb][s];
+                    const v8i k8v = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+                    st[kb] = score_mfma4(k8v, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
                 }
             }
         }
@@ -265,58 +312,72 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
                 }
         }
 
-        // ---- online softmax (per lane = per query) ----
+        // ---- online softmax (per lane = per query): st holds S - m_run ----
         float mx = st[0][0];
 #pragma unroll
         for (int kb = 0; kb < G::KB; ++kb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, st[kb][e]);
-        mx = __builtin_fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = __builtin_fmaxf(m_run, mx);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        float psum = 0.0f;
+        mx = max_lane_pair(mx);
+        if (j == 0 || __any(mx > REBASE)) {
+            // move the reference maximum up to this tile's maximum (first tile: set it)
+            const float delta = (j == 0) ? mx : __builtin_fmaxf(mx, 0.0f);
+            const float alpha = (j == 0) ? 1.0f : __builtin_amdgcn_exp2f(-delta);
+            m_run += delta;
 #pragma unroll
-        for (int kb = 0; kb < G::KB; ++kb)
+            for (int e = 0; e < 16; ++e) negm[e] = -m_run;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const float p = __builtin_amdgcn_exp2f(st[kb][e] - m_new);
-                st[kb][e] = p;
-                psum += p;
-            }
-        l_run = l_run * alpha + psum;
-        if (__any(alpha != 1.0f)) {
+            for (int kb = 0; kb < G::KB; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) st[kb][e] -= delta;
+            l_run *= alpha;
 #pragma unroll
             for (int d = 0; d < G::NDB; ++d)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[d][e] *= alpha;
         }
+        // P = exp2(S - m_run), rounded to 16 bits for the P.V product; the row sum adds those 16-bit values
+        typename P::vec pk[G::KB][2];
+        float ps0 = 0.0f, ps1 = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < G::KB; ++kb)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int t = 0; t < 8; t += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(st[kb][8 * c + t]);
+                    const float p1 = __builtin_amdgcn_exp2f(st[kb][8 * c + t + 1]);
+                    const typename P::v2 pp = P::pack(p0, p1);
+                    pk[kb][c][t] = pp[0];
+                    pk[kb][c][t + 1] = pp[1];
+                    if (t & 2) ps1 = P::add2(pp, ps1); else ps0 = P::add2(pp, ps0);
+                }
+        l_run += ps0 + ps1;
 
         // V_j (and K_{j+1}) pieces issued by this wave have landed; after the barrier everybody's have
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
 
-        // ---- O^T += V^T P^T ----
+        // ---- O^T += V^T P^T, V fragments prefetched PRE instructions ahead ----
+        constexpr int NV = G::KB * 2 * G::NDB;          // V fragments (= matrix instructions) per tile
+        constexpr int PRE = 8;
+        typename P::vec vf[PRE];
+        auto vaddr = [&](int idx) { return vbuf + (idx * 64 + lane) * 16; };
 #pragma unroll
-        for (int kb = 0; kb < G::KB; ++kb)
+        for (int x = 0; x < PRE; ++x) vf[x] = *reinterpret_cast<const typename P::vec*>(vaddr(x));
 #pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                typename P::vec pf;
-#pragma unroll
-                for (int t = 0; t < 8; ++t) pf[t] = (typename P::elem)st[kb][8 * c + t];
-#pragma unroll
-                for (int d = 0; d < G::NDB; ++d) {
-                    const typename P::vec vf =
-                        *reinterpret_cast<const typename P::vec*>(vbuf + (((kb * 2 + c) * G::NDB + d) * 64 + lane) * 16);
-                    acc[d] = P::mfma(vf, pf, acc[d]);
-                }
-            }
+        for (int idx = 0; idx < NV; ++idx) {
+            const int d = idx % G::NDB, kc = idx / G::NDB;
+            const typename P::vec cur = vf[idx % PRE];
+            if (idx + PRE < NV) vf[idx % PRE] = *reinterpret_cast<const typename P::vec*>(vaddr(idx + PRE));
+            acc[d] = P::mfma(cur, pk[kc >> 1][kc & 1], acc[d]);
+        }
         if (nxt && nxt8 != cur8) load_q(nxt8);
         cur8 = nxt8;
     }
 
     // ---- epilogue: O = acc / l ; register e of lane (h, r): dim 32*db + 8*(e/4) + 4*h + e%4 of query r ----
-    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float l_tot = sum_lane_pair(l_run);
     const float inv = 1.0f / l_tot;
     const int q_global = i * TILE + q_local;
     if (q_global < a.n) {
