@@ -19,15 +19,19 @@
 //   O^T += V^T P^T on v_mfma_f32_32x32x16_{bf16,f16}: the P^T operand of lane (h, r) is exactly the eight
 //                 scores that lane already holds (keys are contracted in the order the score MFMA left
 //                 them); V is pre-arranged by mpsa_v_tiles to match, one 16-byte LDS read per operand.
-// Staging.  K codes and the V tile travel HBM/L2 -> LDS with direct-to-LDS loads (global_load_lds_dwordx4: each
-// lane names a 16-byte global source, the wave's 64 pieces land contiguously in LDS), so they cost neither
+// Staging.  4-bit K codes and the V tile travel HBM/L2 -> LDS with direct-to-LDS loads (global_load_lds_dwordx4:
+// each lane names a 16-byte global source, the wave's 64 pieces land contiguously in LDS), so they cost neither
 // registers nor LDS-write instructions.  The V tile is already in operand order (a flat copy); K rows keep their
 // row-major order but the 16-byte chunks of a row are XOR-swizzled with the row index, which makes the 128-bit
-// operand reads of 16 consecutive rows hit 16 distinct 4-bank groups.  K is double-buffered (tile j+1 streams in
-// during tile j), V is single-buffered (it streams in during the score MFMAs and the softmax of the same tile);
-// K scales are read straight from global memory one tile ahead.  64 KiB of LDS and at most 256 registers per
-// workgroup let two workgroups share a CU, so one's matrix instructions overlap the other's softmax VALU work.
+// operand reads of 16 consecutive rows hit 16 distinct 4-bank groups.  Both are double-buffered and the loop
+// needs ONE barrier per tile: after the barrier of step t a wave issues the loads of V(t+1) and K(t+2), pulls the
+// K(t+1) fragments from LDS into registers and runs P.V of step t; the next step's score MFMAs then start from
+// registers.  8-bit K tiles (the diagonal tile of "diag" runs, every tile of "mxfp8" runs) bypass LDS: each lane
+// reads its fragments from global memory one step ahead.  K scales are read from global memory one step ahead
+// as well.  80 KiB of LDS and at most 256 registers per workgroup let two workgroups share a CU, so one's matrix
+// instructions overlap the other's softmax VALU work.
 #include "mpsa_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -95,15 +99,14 @@ struct Geom {
     static constexpr int SST = D / 64;            // score matrix instructions along D
     static constexpr int NDB = D / 32;            // 32-wide output dim blocks
     static constexpr int ROW4 = D / 2, ROW8 = D;  // bytes per K row
-    static constexpr int CPR4 = ROW4 / 16, CPR8 = ROW8 / 16;          // 16-byte chunks per K row (2|4, 4|8)
-    static constexpr int SH4 = CPR4 == 2 ? 3 : 2;                     // log2(rows per 256 bytes)
-    static constexpr int SH8 = CPR8 == 4 ? 2 : 1;
-    static constexpr int K_BYTES = TILE * ROW8;   // one K buffer holds a tile in either precision
+    static constexpr int CPR4 = ROW4 / 16;        // 16-byte chunks per 4-bit K row (2 | 4)
+    static constexpr int SH4 = CPR4 == 2 ? 3 : 2; // log2(rows per 256 bytes)
+    static constexpr int K_BYTES = TILE * ROW4;   // one 4-bit K tile
     static constexpr int V_BYTES = TILE * D * 2;
-    static constexpr int SMEM = 2 * K_BYTES + V_BYTES;
-    static constexpr int KI4 = TILE * ROW4 / 1024 / NW;               // direct-load instructions per wave, 4-bit K
-    static constexpr int KI8 = TILE * ROW8 / 1024 / NW;
+    static constexpr int SMEM = 2 * K_BYTES + 2 * V_BYTES;
+    static constexpr int KI4 = K_BYTES / 1024 / NW;                   // direct-load instructions per wave
     static constexpr int VI = V_BYTES / 1024 / NW;
+    static constexpr int NV = KB * 2 * NDB;       // V fragments (= P.V matrix instructions) per tile
 };
 
 // One wave-wide direct-to-LDS load: lane l copies 16 bytes from its own global address to lds_wave_base + 16*l.
@@ -112,7 +115,10 @@ __device__ __forceinline__ void load16_to_lds(const uint8_t* gsrc, uint8_t* lds_
                                      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
-template <int D, int TILE, int PVT, int FMT8>
+// MODE is compile-time: an all-4-bit run carries no 8-bit code, an all-8-bit run keeps the next tile's 8-bit K
+// fragments in registers (read from global memory one step ahead), and a "diag" run pipelines 4-bit tiles through
+// LDS and fetches its single 8-bit tile when it gets there.
+template <int D, int TILE, int PVT, int FMT8, int MODE>
 __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     typedef Geom<D, TILE> G;
     typedef PV<PVT> P;
@@ -141,8 +147,27 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     const int q_local = 32 * w + r;
     const int64_t q_row = qhead_row + (int64_t)i * TILE + q_local;
 
-    // ---- Q fragments of the current tile precision stay in registers; they are re-read from global memory when
-    //      the precision changes (once per workgroup in causal "diag" runs: the diagonal tile comes last) ----
+    uint8_t* const kbuf0 = smem;
+    uint8_t* const vbuf0 = smem + 2 * G::K_BYTES;
+    // Visiting order.  The order of key tiles does not matter to the softmax, so the tiles that need special
+    // treatment go LAST: first every plain tile (main precision, no mask) in one tight loop, then the tile that
+    // holds the sequence tail (masked) if there is one, then the diagonal tile i (causal mask and / or 8-bit).
+    constexpr bool HAS4 = MODE != MPSA_MODE_MXFP8;        // 4-bit tiles exist (LDS pipeline in use)
+    constexpr bool PRE8 = MODE == MPSA_MODE_MXFP8;        // 8-bit K fragments are prefetched one step ahead
+    const bool tail = a.n < a.n_pad;
+    const bool diag_special = a.causal || MODE == MPSA_MODE_DIAG;
+    const bool tail_special = tail && !a.causal && !(MODE == MPSA_MODE_DIAG && i == a.nt - 1);
+    const int nsteps = a.causal ? i + 1 : a.nt;
+    const int n_plain = nsteps - (diag_special ? 1 : 0) - (tail_special ? 1 : 0);
+    const int skip = (MODE == MPSA_MODE_DIAG && !a.causal) ? i : 0x7fffffff;   // plain steps jump over tile i
+    auto tile_at = [&](int t) {
+        if (t < n_plain) return t + (t >= skip ? 1 : 0);
+        if (tail_special && t == n_plain) return a.nt - 1;
+        return i;
+    };
+    auto step_is8 = [&](int t) { return MODE == MPSA_MODE_MXFP8 || (MODE == MPSA_MODE_DIAG && t == nsteps - 1); };
+
+    // ---- Q fragments of the current precision stay in registers; re-read when the precision changes ----
     v8i qf[G::SST];
     int qsc = 0;
     auto load_q = [&](bool is8) __attribute__((always_inline)) {
@@ -166,53 +191,63 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         qsc = (int)(sw >> (8 * h));
     };
 
-    // ---- staging: direct-to-LDS loads of K (swizzled rows, double-buffered) and V (flat, single buffer) ----
-    uint8_t* const kbuf0 = smem;
-    uint8_t* const vbuf = smem + 2 * G::K_BYTES;
-    auto tile_is8 = [&](int j) { return a.mode == MPSA_MODE_MXFP8 || (a.mode == MPSA_MODE_DIAG && j == i); };
-    auto issue_k = [&](int j, bool is8) __attribute__((always_inline)) {
-        const int64_t krow0 = khead_row + (int64_t)j * TILE;
-        uint8_t* dst = kbuf0 + (j & 1) * G::K_BYTES;
-        if (is8) {
-            const uint8_t* src = a.k8 + krow0 * G::ROW8;
+    // ---- staging ----
+    auto issue_k4 = [&](int t) __attribute__((always_inline)) {           // 4-bit K tile of step t -> kbuf[t & 1], swizzled rows
+        const uint8_t* src = a.k4 + (khead_row + (int64_t)tile_at(t) * TILE) * G::ROW4;
+        uint8_t* dst = kbuf0 + (t & 1) * G::K_BYTES;
 #pragma unroll
-            for (int c = 0; c < G::KI8; ++c) {
-                const int ci = w * G::KI8 + c;
-                const int p = ci * 64 + lane;
-                const int row = p / G::CPR8, slot = p % G::CPR8;
-                const int cb = slot ^ ((row >> G::SH8) & (G::CPR8 - 1));
-                load16_to_lds(src + row * G::ROW8 + cb * 16, dst + ci * 1024);
-            }
-        } else {
-            const uint8_t* src = a.k4 + krow0 * G::ROW4;
-#pragma unroll
-            for (int c = 0; c < G::KI4; ++c) {
-                const int ci = w * G::KI4 + c;
-                const int p = ci * 64 + lane;
-                const int row = p / G::CPR4, slot = p % G::CPR4;
-                const int cb = slot ^ ((row >> G::SH4) & (G::CPR4 - 1));
-                load16_to_lds(src + row * G::ROW4 + cb * 16, dst + ci * 1024);
-            }
+        for (int c = 0; c < G::KI4; ++c) {
+            const int ci = w * G::KI4 + c;
+            const int p = ci * 64 + lane;
+            const int row = p / G::CPR4, slot = p % G::CPR4;
+            const int cb = slot ^ ((row >> G::SH4) & (G::CPR4 - 1));
+            load16_to_lds(src + row * G::ROW4 + cb * 16, dst + ci * 1024);
         }
     };
-    auto issue_v = [&](int j) __attribute__((always_inline)) {
-        const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)j * TILE) * (D * 2);
+    auto issue_v = [&](int t) __attribute__((always_inline)) {            // V tile of step t -> vbuf[t & 1], flat
+        const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)tile_at(t) * TILE) * (D * 2);
+        uint8_t* dst = vbuf0 + (t & 1) * G::V_BYTES;
 #pragma unroll
         for (int c = 0; c < G::VI; ++c) {
             const int ci = w * G::VI + c;
-            load16_to_lds(src + ci * 1024 + lane * 16, vbuf + ci * 1024);
+            load16_to_lds(src + ci * 1024 + lane * 16, dst + ci * 1024);
         }
     };
-    // E8M0 bytes of this lane's key rows (32*kb + r), shifted so that byte 0 / byte 2 belong to MX block h / 2+h
-    int ksc_next[G::KB];
-    auto load_kscales = [&](int j, bool is8) __attribute__((always_inline)) {
-        const uint8_t* sp = (is8 ? a.ks8 : a.ks4) + (khead_row + (int64_t)j * TILE + r) * (D / 32);
+    // K operand of the coming step, in registers: 4-bit fragments come from LDS, 8-bit ones straight from global
+    v4i kf4[HAS4 ? G::KB : 1][G::SST];
+    v8i kf8[PRE8 ? G::KB : 1][G::SST];
+    int ksc[G::KB];             // E8M0 bytes of this lane's key rows, shifted so bytes 0 / 2 belong to MX block h / 2+h
+    auto load_kscales = [&](int t, bool is8) __attribute__((always_inline)) {
+        const uint8_t* sp = (is8 ? a.ks8 : a.ks4) + (khead_row + (int64_t)tile_at(t) * TILE + r) * (D / 32);
 #pragma unroll
         for (int kb = 0; kb < G::KB; ++kb) {
             const uint32_t sw = (D == 128) ? *reinterpret_cast<const uint32_t*>(sp + kb * 32 * (D / 32))
                                            : (uint32_t)*reinterpret_cast<const uint16_t*>(sp + kb * 32 * (D / 32));
-            ksc_next[kb] = (int)(sw >> (8 * h));
+            ksc[kb] = (int)(sw >> (8 * h));
         }
+    };
+    auto read_kf4 = [&](int t) __attribute__((always_inline)) {
+        const uint8_t* kl = kbuf0 + (t & 1) * G::K_BYTES;
+#pragma unroll
+        for (int kb = 0; kb < G::KB; ++kb) {
+            const int krow = 32 * kb + r;
+            const int f = (krow >> G::SH4) & (G::CPR4 - 1);
+#pragma unroll
+            for (int s = 0; s < G::SST; ++s)
+                kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * G::ROW4 + (((2 * s + h) ^ f) * 16));
+        }
+    };
+    auto load_kf8 = [&](int t, v8i (&dstf)[G::KB][G::SST]) __attribute__((always_inline)) {
+        const uint8_t* src = a.k8 + (khead_row + (int64_t)tile_at(t) * TILE + r) * G::ROW8 + h * 16;
+#pragma unroll
+        for (int kb = 0; kb < G::KB; ++kb)
+#pragma unroll
+            for (int s = 0; s < G::SST; ++s) {
+                // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
+                const v4i x0 = *reinterpret_cast<const v4i*>(src + kb * 32 * G::ROW8 + s * 64);
+                const v4i x1 = *reinterpret_cast<const v4i*>(src + kb * 32 * G::ROW8 + s * 64 + 32);
+                dstf[kb][s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+            }
     };
 
     v16f acc[G::NDB];
@@ -230,67 +265,51 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) negm[e] = 0.0f;
 
-    const int j_end = a.causal ? i + 1 : a.nt;
-    bool cur8 = tile_is8(0);
-    issue_k(0, cur8);
-    load_kscales(0, cur8);
-    load_q(cur8);
+    // ---- prologue: V(0), K(0), K(1) on their way; operands of step 0 into registers ----
+    const bool first8 = step_is8(0);
+    issue_v(0);
+    if constexpr (HAS4) {
+        issue_k4(0);
+        if (nsteps > 1) issue_k4(1);
+    }
+    load_kscales(0, first8);
+    load_q(first8);
+    if constexpr (PRE8) load_kf8(0, kf8);
+    __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0)
+    __syncthreads();
+    if constexpr (HAS4) read_kf4(0);
 
-    for (int j = 0; j < j_end; ++j) {
-        // every wave is done with tile j-1: the V buffer and the other K buffer are free
-        __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): this wave's pieces of K_j (and its scales) have landed
-        __syncthreads();
-        const bool nxt = j + 1 < j_end;
-        const bool nxt8 = nxt ? tile_is8(j + 1) : false;
-        int ksc[G::KB];
-#pragma unroll
-        for (int kb = 0; kb < G::KB; ++kb) ksc[kb] = ksc_next[kb];
-        issue_v(j);
-        if (nxt) {
-            issue_k(j + 1, nxt8);
-            load_kscales(j + 1, nxt8);
-        }
-
-        const uint8_t* kl = kbuf0 + (j & 1) * G::K_BYTES;
+    // One step = one key tile.  IS8 / MASKED are compile-time so the common step (4-bit, unmasked) carries no
+    // branches or mask arithmetic.
+    //   PREP: also pull the next step's K operand (same precision as the run's plain tiles) into registers.
+    auto step = [&](int t, auto is8_c, auto masked_c, auto prep_c) __attribute__((always_inline)) {
+        constexpr bool IS8 = decltype(is8_c)::value;
+        constexpr bool MASKED = decltype(masked_c)::value;
+        constexpr bool PREP = decltype(prep_c)::value;
+        const int j = tile_at(t);                          // key tile of this step
 
         // ---- S^T - m_run = K Q^T + (-m_run) ----
         v16f st[G::KB];
-        if (cur8) {
-            v8i kf[G::KB][G::SST];
 #pragma unroll
-            for (int kb = 0; kb < G::KB; ++kb) {
-                const int krow = 32 * kb + r;
-                const int f = (krow >> G::SH8) & (G::CPR8 - 1);
-                const uint8_t* p = kl + krow * G::ROW8;
+        for (int kb = 0; kb < G::KB; ++kb) {
+            if constexpr (IS8 && PRE8) {
+                st[kb] = score_mfma8<FMT8>(kf8[kb][0], qf[0], negm, 0, ksc[kb], qsc);
+#pragma unroll
+                for (int s = 1; s < G::SST; ++s) st[kb] = score_mfma8<FMT8>(kf8[kb][s], qf[s], st[kb], s, ksc[kb], qsc);
+            } else if constexpr (IS8) {
+                // "diag" run: the single 8-bit tile's fragments come straight from global memory, block by block
+                const uint8_t* src = a.k8 + (khead_row + (int64_t)j * TILE + 32 * kb + r) * G::ROW8 + h * 16;
 #pragma unroll
                 for (int s = 0; s < G::SST; ++s) {
-                    // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
-                    const v4i x0 = *reinterpret_cast<const v4i*>(p + (((4 * s + h) ^ f) * 16));
-                    const v4i x1 = *reinterpret_cast<const v4i*>(p + (((4 * s + h + 2) ^ f) * 16));
-                    kf[kb][s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+                    const v4i x0 = *reinterpret_cast<const v4i*>(src + s * 64);
+                    const v4i x1 = *reinterpret_cast<const v4i*>(src + s * 64 + 32);
+                    const v8i kd = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+                    st[kb] = score_mfma8<FMT8>(kd, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
                 }
-            }
-#pragma unroll
-            for (int kb = 0; kb < G::KB; ++kb) {
-                st[kb] = score_mfma8<FMT8>(kf[kb][0], qf[0], negm, 0, ksc[kb], qsc);
-#pragma unroll
-                for (int s = 1; s < G::SST; ++s) st[kb] = score_mfma8<FMT8>(kf[kb][s], qf[s], st[kb], s, ksc[kb], qsc);
-            }
-        } else {
-            v4i kf[G::KB][G::SST];
-#pragma unroll
-            for (int kb = 0; kb < G::KB; ++kb) {
-                const int krow = 32 * kb + r;
-                const int f = (krow >> G::SH4) & (G::CPR4 - 1);
-#pragma unroll
-                for (int s = 0; s < G::SST; ++s)
-                    kf[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * G::ROW4 + (((2 * s + h) ^ f) * 16));
-            }
-#pragma unroll
-            for (int kb = 0; kb < G::KB; ++kb) {
+            } else {
 #pragma unroll
                 for (int s = 0; s < G::SST; ++s) {
-                    const v4i x = kf[kb][s];
+                    const v4i x = kf4[kb][s];
                     const v8i k8v = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
                     st[kb] = score_mfma4(k8v, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
                 }
@@ -298,10 +317,9 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         }
 
         // ---- masks: causal on the diagonal tile, key tail on the last tile ----
-        const bool diag_mask = a.causal && j == i;
-        const bool tail_mask = (j == a.nt - 1) && (a.n < a.n_pad);
-        if (diag_mask || tail_mask) {
-            const int kmax = tail_mask ? a.n - j * TILE : TILE;        // keys >= kmax are padding
+        if constexpr (MASKED) {
+            const bool diag_mask = a.causal && j == i;
+            const int kmax = (j == a.nt - 1) ? a.n - j * TILE : TILE;   // keys >= kmax are padding
 #pragma unroll
             for (int kb = 0; kb < G::KB; ++kb)
 #pragma unroll
@@ -319,10 +337,10 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, st[kb][e]);
         mx = max_lane_pair(mx);
-        if (j == 0 || __any(mx > REBASE)) {
+        if (t == 0 || __any(mx > REBASE)) {
             // move the reference maximum up to this tile's maximum (first tile: set it)
-            const float delta = (j == 0) ? mx : __builtin_fmaxf(mx, 0.0f);
-            const float alpha = (j == 0) ? 1.0f : __builtin_amdgcn_exp2f(-delta);
+            const float delta = (t == 0) ? mx : __builtin_fmaxf(mx, 0.0f);
+            const float alpha = (t == 0) ? 1.0f : __builtin_amdgcn_exp2f(-delta);
             m_run += delta;
 #pragma unroll
             for (int e = 0; e < 16; ++e) negm[e] = -m_run;
@@ -337,44 +355,72 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
                 for (int e = 0; e < 16; ++e) acc[d][e] *= alpha;
         }
         // P = exp2(S - m_run), rounded to 16 bits for the P.V product; the row sum adds those 16-bit values
-        typename P::vec pk[G::KB][2];
+        v4i pk[G::KB][2];                               // 8 packed 16-bit values = one P^T operand
         float ps0 = 0.0f, ps1 = 0.0f;
 #pragma unroll
         for (int kb = 0; kb < G::KB; ++kb)
 #pragma unroll
             for (int c = 0; c < 2; ++c)
 #pragma unroll
-                for (int t = 0; t < 8; t += 2) {
-                    const float p0 = __builtin_amdgcn_exp2f(st[kb][8 * c + t]);
-                    const float p1 = __builtin_amdgcn_exp2f(st[kb][8 * c + t + 1]);
+                for (int e = 0; e < 8; e += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(st[kb][8 * c + e]);
+                    const float p1 = __builtin_amdgcn_exp2f(st[kb][8 * c + e + 1]);
                     const typename P::v2 pp = P::pack(p0, p1);
-                    pk[kb][c][t] = pp[0];
-                    pk[kb][c][t + 1] = pp[1];
-                    if (t & 2) ps1 = P::add2(pp, ps1); else ps0 = P::add2(pp, ps0);
+                    pk[kb][c][e >> 1] = __builtin_bit_cast(int, pp);
+                    if (e & 2) ps1 = P::add2(pp, ps1); else ps0 = P::add2(pp, ps0);
                 }
         l_run += ps0 + ps1;
 
-        // V_j (and K_{j+1}) pieces issued by this wave have landed; after the barrier everybody's have
+        // this wave's pieces of V(t) and K(t+1) have landed; after the barrier everybody's have, and everybody
+        // is done reading V(t-1) and the K(t) fragments
+        __builtin_amdgcn_sched_barrier(0);             // keep the softmax above and the loads below: register lifetimes
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+
+        if (t + 1 < nsteps) issue_v(t + 1);
+        if constexpr (HAS4) {
+            if (t + 2 < nsteps) issue_k4(t + 2);
+        }
 
         // ---- O^T += V^T P^T, V fragments prefetched PRE instructions ahead ----
-        constexpr int NV = G::KB * 2 * G::NDB;          // V fragments (= matrix instructions) per tile
         constexpr int PRE = 8;
+        const uint8_t* vl = vbuf0 + (t & 1) * G::V_BYTES + lane * 16;
         typename P::vec vf[PRE];
-        auto vaddr = [&](int idx) { return vbuf + (idx * 64 + lane) * 16; };
 #pragma unroll
-        for (int x = 0; x < PRE; ++x) vf[x] = *reinterpret_cast<const typename P::vec*>(vaddr(x));
+        for (int x = 0; x < PRE; ++x) vf[x] = *reinterpret_cast<const typename P::vec*>(vl + x * 1024);
+        // operands of the next step: scales (and 8-bit K) from global memory, 4-bit K from LDS.  Past the last
+        // step this reads a valid but unused tile.
+        if constexpr (PREP) {
+            load_kscales(t + 1, PRE8);
+            if constexpr (PRE8) load_kf8(t + 1, kf8);
+            if constexpr (HAS4) read_kf4(t + 1);
+        }
 #pragma unroll
-        for (int idx = 0; idx < NV; ++idx) {
+        for (int idx = 0; idx < G::NV; ++idx) {
             const int d = idx % G::NDB, kc = idx / G::NDB;
             const typename P::vec cur = vf[idx % PRE];
-            if (idx + PRE < NV) vf[idx % PRE] = *reinterpret_cast<const typename P::vec*>(vaddr(idx + PRE));
-            acc[d] = P::mfma(cur, pk[kc >> 1][kc & 1], acc[d]);
+            if (idx + PRE < G::NV) vf[idx % PRE] = *reinterpret_cast<const typename P::vec*>(vl + (idx + PRE) * 1024);
+            acc[d] = P::mfma(cur, __builtin_bit_cast(typename P::vec, pk[kc >> 1][kc & 1]), acc[d]);
         }
-        if (nxt && nxt8 != cur8) load_q(nxt8);
-        cur8 = nxt8;
+    };
+
+    // ---- plain tiles: one tight single-variant loop ----
+    for (int t = 0; t < n_plain; ++t) step(t, std::integral_constant<bool, PRE8>{}, std::false_type{}, std::true_type{});
+    // ---- the (at most two) special tiles: the sequence-tail tile, then the diagonal tile; both run the masked
+    //      variant (a mask that hides nothing is harmless).  The step before has already fetched their K operand
+    //      unless the precision changes. ----
+    if constexpr (MODE == MPSA_MODE_DIAG) {
+        if (tail_special) step(n_plain, std::false_type{}, std::true_type{}, std::true_type{});
+        if (nsteps > 1) {                              // otherwise the prologue already loaded 8-bit Q and scales
+            load_kscales(nsteps - 1, true);
+            load_q(true);
+        }
+        step(nsteps - 1, std::true_type{}, std::true_type{}, std::false_type{});
+    } else {
+        for (int t = n_plain; t < nsteps; ++t) step(t, std::integral_constant<bool, PRE8>{}, std::true_type{}, std::true_type{});
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
 
     // ---- epilogue: O = acc / l ; register e of lane (h, r): dim 32*db + 8*(e/4) + 4*h + e%4 of query r ----
     const float l_tot = sum_lane_pair(l_run);
@@ -392,26 +438,26 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
                 const float o2 = acc[d][4 * g4 + 2] * inv, o3 = acc[d][4 * g4 + 3] * inv;
                 if (a.o_dtype == MPSA_BF16) {
                     typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
-                    const v4bf pk = {(__bf16)o0, (__bf16)o1, (__bf16)o2, (__bf16)o3};
-                    *reinterpret_cast<v4bf*>(orow + (off + dim) * 2) = pk;
+                    const v4bf pk4 = {(__bf16)o0, (__bf16)o1, (__bf16)o2, (__bf16)o3};
+                    *reinterpret_cast<v4bf*>(orow + (off + dim) * 2) = pk4;
                 } else if (a.o_dtype == MPSA_F16) {
                     typedef _Float16 v4hh __attribute__((ext_vector_type(4)));
-                    const v4hh pk = {(_Float16)o0, (_Float16)o1, (_Float16)o2, (_Float16)o3};
-                    *reinterpret_cast<v4hh*>(orow + (off + dim) * 2) = pk;
+                    const v4hh pk4 = {(_Float16)o0, (_Float16)o1, (_Float16)o2, (_Float16)o3};
+                    *reinterpret_cast<v4hh*>(orow + (off + dim) * 2) = pk4;
                 } else {
-                    const v4f pk = {o0, o1, o2, o3};
-                    *reinterpret_cast<v4f*>(orow + (off + dim) * 4) = pk;
+                    const v4f pk4 = {o0, o1, o2, o3};
+                    *reinterpret_cast<v4f*>(orow + (off + dim) * 4) = pk4;
                 }
             }
     }
 }
 
-template <int D, int TILE, int PVT, int FMT8>
+template <int D, int TILE, int PVT, int FMT8, int MODE>
 int launch_one(const AttnArgs& a, hipStream_t st) {
     typedef Geom<D, TILE> G;
     constexpr int smem = G::SMEM;
     static bool attr_set = false;      // idempotent; a race only repeats the same call
-    auto kern = attn_fwd_kernel<D, TILE, PVT, FMT8>;
+    auto kern = attn_fwd_kernel<D, TILE, PVT, FMT8, MODE>;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "attn: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
@@ -423,11 +469,20 @@ int launch_one(const AttnArgs& a, hipStream_t st) {
     return MPSA_OK;
 }
 
+template <int D, int TILE, int PVT>
+int launch_mode(const AttnArgs& a, hipStream_t st) {
+    if (a.mode == MPSA_MODE_MXFP4) return launch_one<D, TILE, PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP4>(a, st);
+    if (a.mode == MPSA_MODE_MXFP8)
+        return a.fmt8 == MPSA_FMT_E5M2 ? launch_one<D, TILE, PVT, MPSA_FMT_E5M2, MPSA_MODE_MXFP8>(a, st)
+                                       : launch_one<D, TILE, PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP8>(a, st);
+    return a.fmt8 == MPSA_FMT_E5M2 ? launch_one<D, TILE, PVT, MPSA_FMT_E5M2, MPSA_MODE_DIAG>(a, st)
+                                   : launch_one<D, TILE, PVT, MPSA_FMT_E4M3, MPSA_MODE_DIAG>(a, st);
+}
+
 template <int D, int TILE>
 int launch_dt(const AttnArgs& a, int pv_dtype, hipStream_t st) {
-    if (pv_dtype == MPSA_BF16)
-        return a.fmt8 == MPSA_FMT_E5M2 ? launch_one<D, TILE, MPSA_BF16, MPSA_FMT_E5M2>(a, st) : launch_one<D, TILE, MPSA_BF16, MPSA_FMT_E4M3>(a, st);
-    return a.fmt8 == MPSA_FMT_E5M2 ? launch_one<D, TILE, MPSA_F16, MPSA_FMT_E5M2>(a, st) : launch_one<D, TILE, MPSA_F16, MPSA_FMT_E4M3>(a, st);
+    if (pv_dtype == MPSA_BF16) return launch_mode<D, TILE, MPSA_BF16>(a, st);
+    return launch_mode<D, TILE, MPSA_F16>(a, st);
 }
 
 }  // namespace
@@ -461,8 +516,14 @@ extern "C" int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_
     a.B = (int)B; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.n = (int)n; a.nt = (int)nt; a.n_pad = (int)(nt * tile);
     a.causal = causal ? 1 : 0; a.mode = mode; a.fmt8 = fmt8; a.o_dtype = o_dtype;
     hipStream_t st = (hipStream_t)stream;
+#ifdef MPSA_ATTN_ONLY_128
+    if (D == 128 && tile == 128 && pv_dtype == MPSA_BF16 && fmt8 == MPSA_FMT_E4M3 && mode == MPSA_MODE_DIAG)
+        return launch_one<128, 128, MPSA_BF16, MPSA_FMT_E4M3, MPSA_MODE_DIAG>(a, st);
+    return mpsa_fail(MPSA_EUNSUPPORTED, "attn: development build with a single variant");
+#else
     if (D == 128 && tile == 128) return launch_dt<128, 128>(a, pv_dtype, st);
     if (D == 64 && tile == 64)   return launch_dt<64, 64>(a, pv_dtype, st);
     if (D == 128 && tile == 64)  return launch_dt<128, 64>(a, pv_dtype, st);
     return launch_dt<64, 128>(a, pv_dtype, st);
+#endif
 }
