@@ -1,0 +1,75 @@
+// Pieces shared by the attention kernels (device helpers, argument block).
+#pragma once
+#include "mpsa_common.h"
+#include <type_traits>
+
+struct AttnArgs {
+    const uint8_t *q4, *qs4, *q8, *qs8, *k4, *ks4, *k8, *ks8;
+    const void* v;
+    void* o;
+    int64_t o_sb, o_sh, o_sn;
+    int B, Hq, Hkv, n, n_pad, nt;
+    int causal, mode, fmt8, o_dtype;
+    int d, tile;
+};
+
+template <int PVT> struct PV;
+template <> struct PV<MPSA_BF16> {
+    typedef v8bf vec;
+    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ v2 pack(float x, float y) { return (v2){(__bf16)x, (__bf16)y}; }
+    // c + p.x + p.y with the 16-bit values the P.V product will see
+    static __device__ __forceinline__ float add2(v2 p, float c) { return __builtin_amdgcn_fdot2_f32_bf16(p, (v2){(__bf16)1.0f, (__bf16)1.0f}, c, false); }
+    // P = exp2(S - m_run) may grow to 2^REBASE before the running maximum is moved: bf16 has float32's range
+    static constexpr float REBASE = 60.0f;
+};
+template <> struct PV<MPSA_F16> {
+    typedef v8h vec;
+    typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ v2 pack(float x, float y) { return (v2){(_Float16)x, (_Float16)y}; }
+    static __device__ __forceinline__ float add2(v2 p, float c) { return __builtin_amdgcn_fdot2(p, (v2){(_Float16)1.0f, (_Float16)1.0f}, c, false); }
+    static constexpr float REBASE = 12.0f;      // fp16 P must stay below 65504
+};
+
+// Exchange between the two lanes (l, l^32) that share one query.  v_permlane32_swap swaps lanes 32-63 of its first
+// register with lanes 0-31 of its second; fed two copies of x, every lane ends up holding both halves' values.
+// Written as inline assembly because both registers are outputs (the compiler builtin of this toolchain returns
+// the first register for both results); the s_nop's cover the instruction's read/write wait states.
+__device__ __forceinline__ void lane_pair(float x, float& a, float& b) {
+    a = x;
+    b = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float max_lane_pair(float x) {
+    float a, b;
+    lane_pair(x, a, b);
+    return __builtin_fmaxf(a, b);
+}
+__device__ __forceinline__ float sum_lane_pair(float x) {
+    float a, b;
+    lane_pair(x, a, b);
+    return a + b;
+}
+
+template <int FMT8>
+__device__ __forceinline__ v16f score_mfma8(v8i k, v8i q, v16f c, int sel, int ks, int qs) {
+    if (sel == 0) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, FMT8, FMT8, 0, ks, 0, qs);
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, FMT8, FMT8, 2, ks, 2, qs);
+}
+__device__ __forceinline__ v16f score_mfma4(v8i k, v8i q, v16f c, int sel, int ks, int qs) {
+    if (sel == 0) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, 4, 4, 0, ks, 0, qs);
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, 4, 4, 2, ks, 2, qs);
+}
+
+// One wave-wide direct-to-LDS load: lane l copies 16 bytes from its own global address to lds_wave_base + 16*l.
+__device__ __forceinline__ void load16_to_lds(const uint8_t* gsrc, uint8_t* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
+
+// Paired-tile ("ping-pong") kernel for causal runs with D = 128, tile = 128 and whole tile pairs: attn_fwd_pp.hip
+bool attn_pp_supported(const AttnArgs& a, int pv_dtype);
+int attn_pp_launch(const AttnArgs& a, int pv_dtype, hipStream_t st);

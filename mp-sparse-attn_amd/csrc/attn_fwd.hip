@@ -30,66 +30,9 @@
 // reads its fragments from global memory one step ahead.  K scales are read from global memory one step ahead
 // as well.  80 KiB of LDS and at most 256 registers per workgroup let two workgroups share a CU, so one's matrix
 // instructions overlap the other's softmax VALU work.
-#include "mpsa_common.h"
-#include <type_traits>
+#include "attn_common.h"
 
 namespace {
-
-struct AttnArgs {
-    const uint8_t *q4, *qs4, *q8, *qs8, *k4, *ks4, *k8, *ks8;
-    const void* v;
-    void* o;
-    int64_t o_sb, o_sh, o_sn;
-    int B, Hq, Hkv, n, n_pad, nt;
-    int causal, mode, fmt8, o_dtype;
-};
-
-template <int PVT> struct PV;
-template <> struct PV<MPSA_BF16> {
-    typedef v8bf vec;
-    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
-    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-    static __device__ __forceinline__ v2 pack(float x, float y) { return (v2){(__bf16)x, (__bf16)y}; }
-    // c + p.x + p.y with the 16-bit values the P.V product will see
-    static __device__ __forceinline__ float add2(v2 p, float c) { return __builtin_amdgcn_fdot2_f32_bf16(p, (v2){(__bf16)1.0f, (__bf16)1.0f}, c, false); }
-};
-template <> struct PV<MPSA_F16> {
-    typedef v8h vec;
-    typedef _Float16 v2 __attribute__((ext_vector_type(2)));
-    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-    static __device__ __forceinline__ v2 pack(float x, float y) { return (v2){(_Float16)x, (_Float16)y}; }
-    static __device__ __forceinline__ float add2(v2 p, float c) { return __builtin_amdgcn_fdot2(p, (v2){(_Float16)1.0f, (_Float16)1.0f}, c, false); }
-};
-
-// Exchange between the two lanes (l, l^32) that share one query.  v_permlane32_swap swaps lanes 32-63 of its first
-// register with lanes 0-31 of its second; fed two copies of x, every lane ends up holding both halves' values.
-// Written as inline assembly because both registers are outputs (the compiler builtin of this toolchain returns
-// the first register for both results); the s_nop's cover the instruction's read/write wait states.
-__device__ __forceinline__ void lane_pair(float x, float& a, float& b) {
-    a = x;
-    b = x;
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-}
-__device__ __forceinline__ float max_lane_pair(float x) {
-    float a, b;
-    lane_pair(x, a, b);
-    return __builtin_fmaxf(a, b);
-}
-__device__ __forceinline__ float sum_lane_pair(float x) {
-    float a, b;
-    lane_pair(x, a, b);
-    return a + b;
-}
-
-template <int FMT8>
-__device__ __forceinline__ v16f score_mfma8(v8i k, v8i q, v16f c, int sel, int ks, int qs) {
-    if (sel == 0) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, FMT8, FMT8, 0, ks, 0, qs);
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, FMT8, FMT8, 2, ks, 2, qs);
-}
-__device__ __forceinline__ v16f score_mfma4(v8i k, v8i q, v16f c, int sel, int ks, int qs) {
-    if (sel == 0) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, 4, 4, 0, ks, 0, qs);
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, 4, 4, 2, ks, 2, qs);
-}
 
 template <int D, int TILE>
 struct Geom {
@@ -108,12 +51,6 @@ struct Geom {
     static constexpr int VI = V_BYTES / 1024 / NW;
     static constexpr int NV = KB * 2 * NDB;       // V fragments (= P.V matrix instructions) per tile
 };
-
-// One wave-wide direct-to-LDS load: lane l copies 16 bytes from its own global address to lds_wave_base + 16*l.
-__device__ __forceinline__ void load16_to_lds(const uint8_t* gsrc, uint8_t* lds_wave_base) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
-                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
-}
 
 // MODE is compile-time: an all-4-bit run carries no 8-bit code, an all-8-bit run keeps the next tile's 8-bit K
 // fragments in registers (read from global memory one step ahead), and a "diag" run pipelines 4-bit tiles through
@@ -256,9 +193,10 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[d][e] = 0.0f;
     // Running reference maximum of this lane's query, kept LAZILY: it moves only when a tile's maximum exceeds
-    // it by more than REBASE (so P stays below 2^REBASE), and -m_run rides into the score MFMA as its C operand,
+    // it by more than REBASE (so P stays below 2^REBASE, far inside the range of P's 16-bit type and of the float32
+    // accumulators), and -m_run rides into the score MFMA as its C operand,
     // which makes the matrix core deliver S - m_run: the softmax costs no subtract and (almost) no rescale.
-    constexpr float REBASE = 5.0f;
+    constexpr float REBASE = P::REBASE;
     float m_run = 0.0f;
     float l_run = 0.0f;
     v16f negm;
@@ -515,7 +453,9 @@ extern "C" int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_
     a.o_sb = o_strides[0]; a.o_sh = o_strides[1]; a.o_sn = o_strides[2];
     a.B = (int)B; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.n = (int)n; a.nt = (int)nt; a.n_pad = (int)(nt * tile);
     a.causal = causal ? 1 : 0; a.mode = mode; a.fmt8 = fmt8; a.o_dtype = o_dtype;
+    a.d = (int)D; a.tile = tile;
     hipStream_t st = (hipStream_t)stream;
+    if (attn_pp_supported(a, pv_dtype)) return attn_pp_launch(a, pv_dtype, st);
 #ifdef MPSA_ATTN_ONLY_128
     if (D == 128 && tile == 128 && pv_dtype == MPSA_BF16 && fmt8 == MPSA_FMT_E4M3 && mode == MPSA_MODE_DIAG)
         return launch_one<128, 128, MPSA_BF16, MPSA_FMT_E4M3, MPSA_MODE_DIAG>(a, st);

@@ -1,0 +1,382 @@
+// Paired-tile ("ping-pong") fused MXFP attention forward for gfx950: causal, D = 128, 128x128 tiles.
+//
+// Same arithmetic as attn_fwd.hip (see there for the operand layouts and the reference citations:
+// ours/mxfp_attn_kernel.py:216-359 for the loop, ours/online_routing.py:68-77, :113-118, :160-171 for the causal
+// tile structure and the grouped-query head mapping).  What differs is the schedule.  A SIMD has one matrix pipe
+// and one vector ALU; a wave alternates between a matrix-heavy phase (P.V of one key tile, then Q.K^T of the next)
+// and a vector-heavy phase (softmax).  Here a workgroup of EIGHT waves owns TWO adjacent query tiles:
+// waves 0-3 ("X", tile 2I+1) and waves 4-7 ("Y", tile 2I); wave w and wave w+4 sit on the same SIMD.  Between two
+// consecutive workgroup barriers X runs  P.V(t) -> S(t+1) -> softmax(t+1)  while Y runs  softmax(t) -> P.V(t) -> S(t+1):
+// whenever one of the two co-resident waves is in its matrix phase the other is in its vector phase, so the matrix
+// pipe and the vector ALU overlap by construction instead of by luck.  Both groups read the same K and V tiles
+// from LDS, which also halves the L2 -> LDS traffic per query.
+//
+// Staging is the one of attn_fwd.hip: 4-bit K tiles (XOR-swizzled rows) and V tiles (operand order) arrive by
+// direct-to-LDS loads, double-buffered, one barrier per key tile; the K fragments of the next tile are pulled into
+// registers before the P.V instructions are issued; the single 8-bit (diagonal) tile of a "diag" run is read straight
+// from global memory.  The running maximum is lazy and rides in the score MFMA's C operand.
+#include "attn_common.h"
+
+namespace {
+
+constexpr int D = 128, TILE = 128;
+constexpr int KB = TILE / 32, SST = D / 64, NDB = D / 32;
+constexpr int ROW4 = D / 2, ROW8 = D;
+constexpr int CPR4 = ROW4 / 16, SH4 = 2;
+constexpr int K_BYTES = TILE * ROW4, V_BYTES = TILE * D * 2;
+constexpr int SMEM = 2 * K_BYTES + 2 * V_BYTES;
+constexpr int NWAVES = 8;
+constexpr int VI = V_BYTES / 1024 / NWAVES;     // direct-load instructions per wave for one V tile (4)
+constexpr int NV = KB * 2 * NDB;                // P.V matrix instructions per tile (32)
+static_assert(K_BYTES / 1024 == NWAVES, "one K direct-load instruction per wave");
+
+template <int PVT, int FMT8, int MODE>
+__global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
+    typedef PV<PVT> P;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, w = tid >> 6;
+    const int h = lane >> 5, r = lane & 31;
+    const int role = w >> 2;                     // 0 = X (matrix phase first), 1 = Y (vector phase first)
+    const int wq = w & 3;
+
+    // ---- which (batch, kv head, query head, query-tile pair) -- XCD-aware, heavy pairs first ----
+    const int npairs = a.nt >> 1;
+    const int group = a.Hq / a.Hkv;
+    const int total = a.B * a.Hq * npairs;
+    int L = blockIdx.x;
+    if ((total & 7) == 0) L = (L & 7) * (total >> 3) + (L >> 3);
+    const int per_unit = group * npairs;
+    const int unit = L / per_unit;
+    const int rem = L - unit * per_unit;
+    const int rank = rem / group;
+    const int hq = (unit % a.Hkv) * group + (rem - rank * group);
+    const int b = unit / a.Hkv;
+    const int kvh = unit % a.Hkv;
+    const int pair = npairs - 1 - rank;
+    const int i = 2 * pair + (1 - role);         // this wave's query tile
+    const int nsteps = 2 * pair + 2;             // key tiles 0 .. 2*pair+1, step t visits tile t
+
+    const int64_t qhead_row = ((int64_t)b * a.Hq + hq) * a.n_pad;
+    const int64_t khead_row = ((int64_t)b * a.Hkv + kvh) * a.n_pad;
+    const int q_local = 32 * wq + r;
+    const int64_t q_row = qhead_row + (int64_t)i * TILE + q_local;
+
+    uint8_t* const kbuf0 = smem;
+    uint8_t* const vbuf0 = smem + 2 * K_BYTES;
+
+    // ---- operands in registers ----
+    v8i qf[SST];
+    int qsc = 0;
+    v4i kf4[KB][SST];
+    int ksc[KB];
+    auto load_q = [&](bool is8) __attribute__((always_inline)) {
+        if (is8) {
+#pragma unroll
+            for (int s = 0; s < SST; ++s) {
+                // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
+                const v4i x0 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + s * 64 + h * 16);
+                const v4i x1 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + s * 64 + h * 16 + 32);
+                qf[s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < SST; ++s) {
+                const v4i x = *reinterpret_cast<const v4i*>(a.q4 + q_row * (D / 2) + (2 * s + h) * 16);
+                qf[s] = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+            }
+        }
+        const uint8_t* qs = (is8 ? a.qs8 : a.qs4) + q_row * (D / 32);
+        qsc = (int)(*reinterpret_cast<const uint32_t*>(qs) >> (8 * h));
+    };
+    auto load_kscales = [&](int t, bool is8) __attribute__((always_inline)) {
+        const uint8_t* sp = (is8 ? a.ks8 : a.ks4) + (khead_row + (int64_t)t * TILE + r) * (D / 32);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+            ksc[kb] = (int)(*reinterpret_cast<const uint32_t*>(sp + kb * 32 * (D / 32)) >> (8 * h));
+    };
+    auto read_kf4 = [&](int t) __attribute__((always_inline)) {
+        const uint8_t* kl = kbuf0 + (t & 1) * K_BYTES;
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            const int krow = 32 * kb + r;
+            const int f = (krow >> SH4) & (CPR4 - 1);
+#pragma unroll
+            for (int s = 0; s < SST; ++s)
+                kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * ROW4 + (((2 * s + h) ^ f) * 16));
+        }
+    };
+
+    // ---- staging: every wave issues its share of each tile ----
+    auto issue_k4 = [&](int t) __attribute__((always_inline)) {
+        const uint8_t* src = a.k4 + (khead_row + (int64_t)t * TILE) * ROW4;
+        const int p = w * 64 + lane;
+        const int row = p / CPR4, slot = p % CPR4;
+        const int cb = slot ^ ((row >> SH4) & (CPR4 - 1));
+        load16_to_lds(src + row * ROW4 + cb * 16, kbuf0 + (t & 1) * K_BYTES + w * 1024);
+    };
+    auto issue_v = [&](int t) __attribute__((always_inline)) {
+        const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)t * TILE) * (D * 2);
+        uint8_t* dst = vbuf0 + (t & 1) * V_BYTES;
+#pragma unroll
+        for (int c = 0; c < VI; ++c) {
+            const int ci = w * VI + c;
+            load16_to_lds(src + ci * 1024 + lane * 16, dst + ci * 1024);
+        }
+    };
+    // barrier of step t: this wave's pieces of V(t) and K(t+1) have landed, after it everybody's have and everybody
+    // is done with V(t-1) and the K(t) fragments; then the next loads go out
+    auto sync_issue = [&](int t) __attribute__((always_inline)) {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < nsteps) issue_v(t + 1);
+        if (t + 2 < nsteps) issue_k4(t + 2);
+    };
+
+    // ---- per-query state ----
+    v16f acc[NDB];
+#pragma unroll
+    for (int d = 0; d < NDB; ++d)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[d][e] = 0.0f;
+    constexpr float REBASE = P::REBASE;          // lazy running maximum, see attn_fwd.hip
+    float m_run = 0.0f, l_run = 0.0f;
+    v16f negm;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) negm[e] = 0.0f;
+    v16f st[KB];
+    v4i pk[KB][2];
+
+    auto prep_plain = [&](int t) __attribute__((always_inline)) {
+        load_kscales(t, false);
+        read_kf4(t);
+    };
+    auto prep_special = [&](int t) __attribute__((always_inline)) {      // this wave's diagonal tile
+        if constexpr (MODE == MPSA_MODE_DIAG) {
+            load_kscales(t, true);
+            load_q(true);
+        } else {
+            prep_plain(t);
+        }
+    };
+    auto s_plain = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int s = 0; s < SST; ++s) {
+                const v4i x = kf4[kb][s];
+                const v8i k8v = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+                st[kb] = score_mfma4(k8v, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
+            }
+    };
+    auto s_special = [&](int t) __attribute__((always_inline)) {
+        if constexpr (MODE == MPSA_MODE_DIAG) {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                const uint8_t* src = a.k8 + (khead_row + (int64_t)t * TILE + 32 * kb + r) * ROW8 + h * 16;
+#pragma unroll
+                for (int s = 0; s < SST; ++s) {
+                    const v4i x0 = *reinterpret_cast<const v4i*>(src + s * 64);
+                    const v4i x1 = *reinterpret_cast<const v4i*>(src + s * 64 + 32);
+                    const v8i kd = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+                    st[kb] = score_mfma8<FMT8>(kd, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
+                }
+            }
+        } else {
+            s_plain();
+        }
+    };
+    auto softmax = [&](bool first, auto masked_c) __attribute__((always_inline)) {
+        if constexpr (decltype(masked_c)::value) {      // diagonal tile: keys after the query are dead
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int key = 32 * kb + 8 * (e >> 2) + 4 * h + (e & 3);
+                    if (key > q_local) st[kb][e] = -__builtin_inff();
+                }
+        }
+        float mx = st[0][0];
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, st[kb][e]);
+        mx = max_lane_pair(mx);
+        if (first || __any(mx > REBASE)) {
+            const float delta = first ? mx : __builtin_fmaxf(mx, 0.0f);
+            const float alpha = first ? 1.0f : __builtin_amdgcn_exp2f(-delta);
+            m_run += delta;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) negm[e] = -m_run;
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) st[kb][e] -= delta;
+            l_run *= alpha;
+#pragma unroll
+            for (int d = 0; d < NDB; ++d)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[d][e] *= alpha;
+        }
+        float ps0 = 0.0f, ps1 = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(st[kb][8 * c + e]);
+                    const float p1 = __builtin_amdgcn_exp2f(st[kb][8 * c + e + 1]);
+                    const typename P::v2 pp = P::pack(p0, p1);
+                    pk[kb][c][e >> 1] = __builtin_bit_cast(int, pp);
+                    if (e & 2) ps1 = P::add2(pp, ps1); else ps0 = P::add2(pp, ps0);
+                }
+        l_run += ps0 + ps1;
+    };
+    auto pv = [&](int t) __attribute__((always_inline)) {
+        constexpr int PRE = 8;
+        const uint8_t* vl = vbuf0 + (t & 1) * V_BYTES + lane * 16;
+        typename P::vec vf[PRE];
+#pragma unroll
+        for (int x = 0; x < PRE; ++x) vf[x] = *reinterpret_cast<const typename P::vec*>(vl + x * 1024);
+#pragma unroll
+        for (int idx = 0; idx < NV; ++idx) {
+            const int d = idx % NDB, kc = idx / NDB;
+            const typename P::vec cur = vf[idx % PRE];
+            if (idx + PRE < NV) vf[idx % PRE] = *reinterpret_cast<const typename P::vec*>(vl + (idx + PRE) * 1024);
+            acc[d] = P::mfma(cur, __builtin_bit_cast(typename P::vec, pk[kc >> 1][kc & 1]), acc[d]);
+        }
+    };
+
+    // ---- prologue (all waves): V(0), K(0), K(1) on their way; step-0 operands into registers ----
+    issue_v(0);
+    issue_k4(0);
+    issue_k4(1);
+    load_kscales(0, false);
+    load_q(false);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    read_kf4(0);
+
+    if (role == 0) {
+        // ===== X: tile i = 2*pair+1 >= 1; between barriers: P.V(t) -> S(t+1) -> softmax(t+1) =====
+        s_plain();
+        softmax(true, std::false_type{});
+        for (int t = 0; t < nsteps - 2; ++t) {
+            sync_issue(t);
+            prep_plain(t + 1);
+            pv(t);
+            s_plain();
+            softmax(false, std::false_type{});
+        }
+        {
+            const int t = nsteps - 2;
+            sync_issue(t);
+            prep_special(t + 1);
+            pv(t);
+            s_special(t + 1);
+            softmax(false, std::true_type{});
+        }
+        sync_issue(nsteps - 1);
+        pv(nsteps - 1);
+    } else {
+        // ===== Y: tile i = 2*pair; between barriers: softmax(t) -> P.V(t) -> S(t+1); idle in the last step =====
+        if (i == 0) {
+            prep_special(0);
+            s_special(0);
+        } else {
+            s_plain();
+        }
+        for (int t = 0; t < i - 1; ++t) {
+            sync_issue(t);
+            softmax(t == 0, std::false_type{});
+            prep_plain(t + 1);
+            pv(t);
+            s_plain();
+        }
+        if (i >= 1) {
+            const int t = i - 1;
+            sync_issue(t);
+            softmax(t == 0, std::false_type{});
+            prep_special(t + 1);
+            pv(t);
+            s_special(t + 1);
+        }
+        sync_issue(i);
+        softmax(i == 0, std::true_type{});
+        pv(i);
+        sync_issue(i + 1);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
+
+    // ---- epilogue: O = acc / l ; register e of lane (h, r): dim 32*db + 8*(e/4) + 4*h + e%4 of query r ----
+    const float l_tot = sum_lane_pair(l_run);
+    const float inv = 1.0f / l_tot;
+    const int q_global = i * TILE + q_local;
+    uint8_t* orow = static_cast<uint8_t*>(a.o);
+    const int64_t off = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh + (int64_t)q_global * a.o_sn;
+#pragma unroll
+    for (int d = 0; d < NDB; ++d)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            const int dim = 32 * d + 8 * g4 + 4 * h;
+            const float o0 = acc[d][4 * g4 + 0] * inv, o1 = acc[d][4 * g4 + 1] * inv;
+            const float o2 = acc[d][4 * g4 + 2] * inv, o3 = acc[d][4 * g4 + 3] * inv;
+            if (a.o_dtype == MPSA_BF16) {
+                typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+                const v4bf pk4 = {(__bf16)o0, (__bf16)o1, (__bf16)o2, (__bf16)o3};
+                *reinterpret_cast<v4bf*>(orow + (off + dim) * 2) = pk4;
+            } else if (a.o_dtype == MPSA_F16) {
+                typedef _Float16 v4hh __attribute__((ext_vector_type(4)));
+                const v4hh pk4 = {(_Float16)o0, (_Float16)o1, (_Float16)o2, (_Float16)o3};
+                *reinterpret_cast<v4hh*>(orow + (off + dim) * 2) = pk4;
+            } else {
+                const v4f pk4 = {o0, o1, o2, o3};
+                *reinterpret_cast<v4f*>(orow + (off + dim) * 4) = pk4;
+            }
+        }
+}
+
+template <int PVT, int FMT8, int MODE>
+int launch_pp(const AttnArgs& a, hipStream_t st) {
+    static bool attr_set = false;      // idempotent; a race only repeats the same call
+    auto kern = attn_pp_kernel<PVT, FMT8, MODE>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+        if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "attn: cannot reserve %d bytes of LDS: %s", SMEM, hipGetErrorString(e));
+        attr_set = true;
+    }
+    dim3 grid((unsigned)(a.B * a.Hq * (a.nt / 2)));
+    hipLaunchKernelGGL(kern, grid, dim3(512), SMEM, st, a);
+    MPSA_CHECK_LAUNCH("attn(pp)");
+    return MPSA_OK;
+}
+
+template <int PVT>
+int launch_pp_mode(const AttnArgs& a, hipStream_t st) {
+    if (a.mode == MPSA_MODE_MXFP4) return launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP4>(a, st);
+    return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_DIAG>(a, st)
+                                   : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_DIAG>(a, st);
+}
+
+}  // namespace
+
+// The paired-tile kernel covers causal runs over whole pairs of full 128-query tiles with D = 128.
+// MPSA_ATTN_PP=0 in the environment switches it off (the general kernel then runs everything).
+bool attn_pp_supported(const AttnArgs& a, int pv_dtype) {
+    static const bool enabled = [] {
+        const char* v = getenv("MPSA_ATTN_PP");
+        return !(v && v[0] == '0');
+    }();
+    (void)pv_dtype;
+    return enabled && a.causal && a.d == 128 && a.tile == 128 && a.n == a.n_pad && (a.nt % 2) == 0 &&
+           (a.mode == MPSA_MODE_DIAG || a.mode == MPSA_MODE_MXFP4);
+}
+
+int attn_pp_launch(const AttnArgs& a, int pv_dtype, hipStream_t st) {
+    if (pv_dtype == MPSA_BF16) return launch_pp_mode<MPSA_BF16>(a, st);
+    return launch_pp_mode<MPSA_F16>(a, st);
+}

@@ -29,6 +29,16 @@ def _run(q, k, v, **kw):
 
 
 @pytest.mark.parametrize("mode", ["diag", "mxfp4", "mxfp8"])
+@pytest.mark.parametrize("N", [1024, 128, 256])
+def test_modes_d128_tile128_causal(mode, N):
+    """Every precision mode on the benchmark's kernel shape, including a single tile and a single tile pair."""
+    q, k, v = make_qkv(1, 4, 2, N, 128, seed=70 + N)
+    got = _run(q, k, v, is_causal=True, block_scale_type=mode, tile=128, output_dtype=torch.bfloat16)
+    want = O.attn_mx(q, k, v, tile=128, causal=True, mode=mode)
+    _compare(got, want, f"{mode} N={N}")
+
+
+@pytest.mark.parametrize("mode", ["diag", "mxfp4", "mxfp8"])
 def test_c1_cpu_plumbing_config(mode):
     """B=1 H=8 N=1024 D=64, seed 0, causal, 64x64 tiles."""
     q, k, v = make_qkv(1, 8, 8, 1024, 64, seed=0)
@@ -37,10 +47,11 @@ def test_c1_cpu_plumbing_config(mode):
     _compare(got, want, f"C1 {mode}")
 
 
-@pytest.mark.parametrize("D,tile", [(128, 128), (64, 128), (128, 64), (64, 64)])
+@pytest.mark.parametrize("N", [512, 384])      # 4 and 3 tiles of 128: causal D=128/tile=128 runs the paired-tile
+@pytest.mark.parametrize("D,tile", [(128, 128), (64, 128), (128, 64), (64, 64)])   # kernel for 512, the general one for 384
 @pytest.mark.parametrize("causal", [True, False])
-def test_all_kernel_variants_gqa(D, tile, causal):
-    q, k, v = make_qkv(2, 4, 2, 512, D, seed=10 + D + tile)
+def test_all_kernel_variants_gqa(D, tile, causal, N):
+    q, k, v = make_qkv(2, 4, 2, N, D, seed=10 + D + tile)
     got = _run(q, k, v, is_causal=causal, block_scale_type="diag", tile=tile, output_dtype=torch.float32)
     want = O.attn_mx(q, k, v, tile=tile, causal=causal, mode="diag", out_dtype=torch.float32)
     _compare(got, want, f"D={D} tile={tile} causal={causal}")
