@@ -14,7 +14,7 @@ FMT_E4M3, FMT_E5M2, FMT_E2M1 = 0, 1, 4
 MODE_MXFP4, MODE_MXFP8, MODE_DIAG = 0, 1, 2
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libmpsa.so")
+LIB_PATH = os.environ.get("MPSA_LIB_PATH") or os.path.join(os.path.dirname(_HERE), "lib", "libmpsa.so")
 
 _i64, _int, _vp, _f32 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_float
 _p64 = ctypes.POINTER(ctypes.c_int64)
