@@ -30,6 +30,11 @@ PEAK_FP8_TFLOPS = 5000.0
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 
+# HBM-side bytes per launch of the fused attention kernel (L2 <-> fabric), from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of `bench.py --only attn`, each scaled by the same counter's reading for a 1 GiB copy
+# (`bench.py --only copy`): FETCH_SIZE x 2.0 KiB, WRITE_SIZE x 1.0 KiB.  Summary: profiles/attn_c3_hbm_traffic.txt
+MEASURED_ATTN_TRAFFIC_BYTES = {"c3": 110.2e6 + 67.1e6}
+
 WORKLOADS = {
     # name: (B, Hq, Hkv, N, D, tile, seed, description)
     "c1": (1, 8, 8, 1024, 64, 64, 0, "C1 B1 H8 N1024 D64 causal tile64 diag"),
@@ -127,6 +132,47 @@ def secondary(device, quick):
     return out
 
 
+def run_only(args, device):
+    """Launch one kernel repeatedly (for rocprofv3 --pmc / --kernel-trace runs)."""
+    from ours import _lib
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands
+    from ours.quant_mxint8 import quantize_mx, quantize_mx_dual
+    from ours.block_scaled_matmul import block_scaled_matmul, make_configs
+    if args.only == "copy":
+        src = torch.ones(1 << 29, dtype=torch.bfloat16, device=device)          # 1 GiB
+        dst = torch.empty_like(src)
+        fn = lambda: dst.copy_(src)
+        info = {"kernel": "torch copy", "bytes_read": src.numel() * 2, "bytes_written": src.numel() * 2}
+    elif args.only == "attn":
+        B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
+        q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device)
+        out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
+        ops = prepare_operands(q, k, v, tile, "diag")
+        fn = lambda: attention_from_operands(ops, out, True)
+        info = {"kernel": "attention", "workload": desc}
+    elif args.only == "quant":
+        B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
+        q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device)
+        fn = lambda: quantize_mx_dual(q, 0.1275)
+        info = {"kernel": "quantize dual (Q of the workload)", "elements": q.numel(), "algorithmic_bytes": q.numel() * 3.5625}
+    else:
+        M = N = K = 8192
+        g = torch.Generator(device=device).manual_seed(1)
+        a = torch.randn(M, K, generator=g, device=device).to(torch.bfloat16)[None, None]
+        b = torch.randn(N, K, generator=g, device=device).to(torch.bfloat16)[None, None]
+        bst, fmt = ("mxfp4", _lib.FMT_E2M1) if args.only == "gemm4" else ("mxfp8", _lib.FMT_E4M3)
+        ac, asc = quantize_mx(a, 1.0, fmt)
+        bc, bsc = quantize_mx(b, 1.0, fmt)
+        cfg = make_configs(bst)
+        fn = lambda: block_scaled_matmul(ac[0, 0], asc[0, 0], bc[0, 0], bsc[0, 0], torch.bfloat16, M, N, K, cfg)
+        info = {"kernel": "gemm " + bst, "flops": 2.0 * M * N * K}
+    fn()
+    torch.cuda.synchronize()
+    ms = time_events(fn, args.steps)
+    info["ms"] = round(ms, 4)
+    print(json.dumps(info))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -135,6 +181,9 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--only", default=None, choices=["attn", "copy", "quant", "gemm4", "gemm8"],
+                    help="profiling aid: launch just this kernel --steps times and exit (copy = 1 GiB torch copy, "
+                         "the calibration kernel for HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the kernel is measured on one GPU's "
@@ -148,6 +197,9 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.only:
+        run_only(args, device)
+        return
     B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
     q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device)
     out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
@@ -179,8 +231,9 @@ def main():
     nt = (N + tile - 1) // tile
     comp = composite_peak_tflops(nt)
     roofline = {
-        "bound": "mfma", "kernel": "attn_fwd_kernel", "achieved": round(achieved, 2), "peak": PEAK_FP4_TFLOPS,
-        "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP4_TFLOPS, 5), "traffic": None,
+        "bound": "mfma", "kernel": "attn_pp_kernel (fused attention)", "achieved": round(achieved, 2), "peak": PEAK_FP4_TFLOPS,
+        "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP4_TFLOPS, 5),
+        "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get(args.workload),
         "kernel_ms": round(attn_ms, 4), "prepare_ms": round(prep_ms, 4),
         "composite_peak": round(comp, 1), "frac_composite": round(achieved / comp, 5),
         "flops_per_launch": flops,

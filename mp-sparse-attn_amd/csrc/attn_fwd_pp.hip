@@ -2,14 +2,14 @@
 //
 // Same arithmetic as attn_fwd.hip (see there for the operand layouts and the reference citations:
 // ours/mxfp_attn_kernel.py:216-359 for the loop, ours/online_routing.py:68-77, :113-118, :160-171 for the causal
-// tile structure and the grouped-query head mapping).  What differs is the schedule.  A SIMD has one matrix pipe
-// and one vector ALU; a wave alternates between a matrix-heavy phase (P.V of one key tile, then Q.K^T of the next)
-// and a vector-heavy phase (softmax).  Here a workgroup of EIGHT waves owns TWO adjacent query tiles:
-// waves 0-3 ("X", tile 2I+1) and waves 4-7 ("Y", tile 2I); wave w and wave w+4 sit on the same SIMD.  Between two
-// consecutive workgroup barriers X runs  P.V(t) -> S(t+1) -> softmax(t+1)  while Y runs  softmax(t) -> P.V(t) -> S(t+1):
-// whenever one of the two co-resident waves is in its matrix phase the other is in its vector phase, so the matrix
-// pipe and the vector ALU overlap by construction instead of by luck.  Both groups read the same K and V tiles
-// from LDS, which also halves the L2 -> LDS traffic per query.
+// tile structure and the grouped-query head mapping).  What differs is the work split.  A workgroup of EIGHT waves
+// owns TWO adjacent query tiles: waves 0-3 ("X", tile 2I+1) and waves 4-7 ("Y", tile 2I); wave w and wave w+4 sit
+// on the same SIMD.  Both groups read the same K and V tiles from LDS, which halves the L2 -> LDS traffic per query
+// and the number of direct-to-LDS loads per CU.  Between two consecutive workgroup barriers X runs
+// P.V(t) -> S(t+1) -> softmax(t+1) while Y runs softmax(t) -> P.V(t) -> S(t+1), i.e. the two waves of a SIMD are in
+// opposite phases.  (Measured on MI355X this phase offset buys little: while one wave streams back-to-back matrix
+// instructions the other wave of the SIMD gets almost no vector issue slots, so matrix and vector phases of the two
+// waves still add up; the shared staging is what makes this kernel faster than the one-tile kernel.)
 //
 // Staging is the one of attn_fwd.hip: 4-bit K tiles (XOR-swizzled rows) and V tiles (operand order) arrive by
 // direct-to-LDS loads, double-buffered, one barrier per key tile; the K fragments of the next tile are pulled into
