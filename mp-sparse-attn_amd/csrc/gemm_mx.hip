@@ -13,16 +13,24 @@
 // with 8-bit elements registers 0-3 of the two lane halves together are block 0 and registers 4-7 block 1
 // (each half holds 16 bytes of either block).  Either way fragments are plain 16-byte pieces of the
 // row-major HBM layout.  K advances 64 bytes of codes per row per stage (128 E2M1 or 64 8-bit elements).
-// Stages are double-buffered in LDS with rows padded from 64 to 80 bytes: the 16 lanes of a 128-bit
-// LDS access phase then fall into 16 distinct 4-bank groups.  Wave tiles of 128x128 keep LDS reads at
-// 8 operand fragments per 16 matrix instructions.
+//
+// Staging.  Codes and scale bytes go HBM/L2 -> LDS with direct-to-LDS loads (no registers, no LDS-write
+// instructions) into a ring of four stages, three of them in flight while one is being multiplied: with one
+// workgroup per CU nothing else hides the memory latency.  The 16-byte chunks of a row are XOR-swizzled with
+// the row index so that the 128-bit operand reads of 16 consecutive rows hit 16 distinct 4-bank groups.  One
+// barrier per stage.  Wave tiles of 128x128 keep LDS reads at 8 operand fragments per 16 matrix instructions.
 #include "mpsa_common.h"
 
 namespace {
 
 constexpr int BM = 256, BN = 256;       // workgroup tile
 constexpr int ROWB = 64;                // code bytes per row per stage
-constexpr int PITCH = 80;               // LDS row pitch
+constexpr int NSTAGE = 4;               // LDS ring depth
+constexpr int OP_BYTES = BM * ROWB;     // one operand's codes per stage (16 KiB)
+constexpr int SC_BYTES = BM * 4;        // one operand's scale bytes per stage (4 per row)
+constexpr int STAGE_BYTES = 2 * OP_BYTES + 2 * SC_BYTES;
+constexpr int SMEM_BYTES = NSTAGE * STAGE_BYTES;
+constexpr int LOADS_PER_STAGE = 2 * (OP_BYTES / 1024 / 4) + 2;   // direct-to-LDS instructions per wave per stage (10)
 
 struct GemmArgs {
     const uint8_t *a, *sa, *b, *sb;
@@ -36,66 +44,80 @@ template <> __device__ __forceinline__ float cvt_out<float>(float v) { return v;
 template <> __device__ __forceinline__ __bf16 cvt_out<__bf16>(float v) { return (__bf16)v; }
 template <> __device__ __forceinline__ _Float16 cvt_out<_Float16>(float v) { return (_Float16)v; }
 
+// Direct-to-LDS load written as inline assembly: lane L's BYTES bytes at gsrc land at lds_wave_base + L*BYTES
+// (M0 carries the wave-uniform LDS base).  The compiler's own builtin for this instruction makes it wait for
+// every outstanding load (vmcnt(0)) before the next barrier or LDS read, which would drain the ring each stage;
+// as assembly the loads are invisible to that bookkeeping and the kernel's explicit partial waits stand.
+template <int BYTES>
+__device__ __forceinline__ void load_to_lds(const uint8_t* gsrc, uint8_t* lds_wave_base) {
+    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds_wave_base);
+    if constexpr (BYTES == 16)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(gsrc) : "memory", "m0");
+    else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(gsrc) : "memory", "m0");
+}
+
 template <int FMT, typename OutT>
 __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     constexpr bool FP4 = (FMT == MPSA_FMT_E2M1);
-    constexpr int STEPS = FP4 ? 2 : 1;                 // matrix instructions along K per stage
-    constexpr int SCB = FP4 ? 4 : 2;                   // scale bytes per row per stage
     const int row_bytes = FP4 ? g.K / 2 : g.K;         // code bytes per matrix row
     const int srow_bytes = g.K / 32;
     const int KT = row_bytes / ROWB;
 
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][BM * PITCH];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_b[2][BN * PITCH];
-    __shared__ uint32_t lds_sa[2][BM];
-    __shared__ uint32_t lds_sb[2][BN];
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int h = lane >> 5, r = lane & 31;
 
-    // XCD-aware tile order: consecutive workgroup ids go to different XCDs (8 of them), so give each
-    // XCD a contiguous band of tile rows; tiles of one band share their A rows in that XCD's L2.
-    const int tiles_n = g.N / BN;
-    const int ntiles = (g.M / BM) * tiles_n;
-    int wg = blockIdx.x;
-    if (ntiles % 8 == 0) wg = (wg & 7) * (ntiles >> 3) + (wg >> 3);
-    const int m0 = (wg / tiles_n) * BM;
-    const int n0 = (wg % tiles_n) * BN;
+    // XCD-aware tile order.  Consecutive workgroup ids go to different XCDs (8 of them, each with its own L2) and
+    // an XCD starts its workgroups in id order.  Give XCD x one block of a 2 x 4 split of the tile grid and walk
+    // that block in panels four tile rows high, column by column: the workgroups running together on an XCD
+    // then cover a few tile rows by a few tile columns and share both operands' K-slices in that L2.
+    const int tiles_m = g.M / BM, tiles_n = g.N / BN;
+    int tm, tn;
+    if (tiles_m % 2 == 0 && tiles_n % 4 == 0) {
+        const int x = blockIdx.x & 7, j = blockIdx.x >> 3;
+        const int rm = tiles_m / 2, rn = tiles_n / 4;
+        const int ph = rm % 4 == 0 ? 4 : (rm % 2 == 0 ? 2 : 1);
+        const int panel = j / (ph * rn), jj = j % (ph * rn);
+        tm = (x >> 2) * rm + panel * ph + jj % ph;
+        tn = (x & 3) * rn + jj / ph;
+    } else {
+        tm = blockIdx.x / tiles_n;
+        tn = blockIdx.x % tiles_n;
+    }
+    const int m0 = tm * BM;
+    const int n0 = tn * BN;
 
-    // global -> register staging: thread t moves 16-byte chunk (row t/4 + 64 i, column chunk t%4)
-    const int crow = tid >> 2, ccol = tid & 3;
-    const uint8_t* ga = g.a + (int64_t)(m0 + crow) * row_bytes + ccol * 16;
-    const uint8_t* gb = g.b + (int64_t)(n0 + crow) * row_bytes + ccol * 16;
-    const uint8_t* gsa = g.sa + (int64_t)(m0 + tid) * srow_bytes;
-    const uint8_t* gsb = g.sb + (int64_t)(n0 + tid) * srow_bytes;
-    const int64_t rstep = (int64_t)64 * row_bytes;
-
-    uint4 ra[4], rb[4];
-    uint32_t rsa, rsb;
-    auto load_stage = [&](int kt) {
+    // ---- direct-to-LDS staging: wave w moves chunks [4w, 4w+4) x 1 KiB of either operand and the scale bytes
+    //      of rows [64w, 64w+64); chunk position p = row*4 + slot holds row's 16-byte piece slot ^ ((row>>2)&3)
+    const uint8_t* ga[4];
+    const uint8_t* gb[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            ra[i] = *reinterpret_cast<const uint4*>(ga + i * rstep + (int64_t)kt * ROWB);
-            rb[i] = *reinterpret_cast<const uint4*>(gb + i * rstep + (int64_t)kt * ROWB);
-        }
-        if constexpr (FP4) {
-            rsa = *reinterpret_cast<const uint32_t*>(gsa + kt * SCB);
-            rsb = *reinterpret_cast<const uint32_t*>(gsb + kt * SCB);
-        } else {
-            rsa = *reinterpret_cast<const uint16_t*>(gsa + kt * SCB);
-            rsb = *reinterpret_cast<const uint16_t*>(gsb + kt * SCB);
-        }
-    };
-    auto store_stage = [&](int buf) {
+    for (int c = 0; c < 4; ++c) {
+        const int p = (wave * 4 + c) * 64 + lane;
+        const int row = p >> 2, slot = p & 3;
+        const int cb = slot ^ ((row >> 2) & 3);
+        ga[c] = g.a + (int64_t)(m0 + row) * row_bytes + cb * 16;
+        gb[c] = g.b + (int64_t)(n0 + row) * row_bytes + cb * 16;
+    }
+    const uint8_t* gsa = g.sa + (int64_t)(m0 + wave * 64 + lane) * srow_bytes;
+    const uint8_t* gsb = g.sb + (int64_t)(n0 + wave * 64 + lane) * srow_bytes;
+    auto issue_stage = [&](int kt) __attribute__((always_inline)) {
+        const int kc = kt < KT ? kt : KT - 1;             // past the end: re-load the last stage (keeps the count uniform)
+        uint8_t* st = smem + (kt % NSTAGE) * STAGE_BYTES;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<uint4*>(&lds_a[buf][(crow + 64 * i) * PITCH + ccol * 16]) = ra[i];
-            *reinterpret_cast<uint4*>(&lds_b[buf][(crow + 64 * i) * PITCH + ccol * 16]) = rb[i];
+        for (int c = 0; c < 4; ++c) {
+            load_to_lds<16>(ga[c] + (int64_t)kc * ROWB, st + (wave * 4 + c) * 1024);
+            load_to_lds<16>(gb[c] + (int64_t)kc * ROWB, st + OP_BYTES + (wave * 4 + c) * 1024);
         }
-        lds_sa[buf][tid] = rsa;
-        lds_sb[buf][tid] = rsb;
+        // four scale bytes per row: the stage's own with 4-bit codes; with 8-bit codes the aligned word that
+        // holds this stage's two bytes (the stage count is even, so the word is inside the row)
+        const int sco = FP4 ? kc * 4 : (kc >> 1) * 4;
+        load_to_lds<4>(gsa + sco, st + 2 * OP_BYTES + wave * 256);
+        load_to_lds<4>(gsb + sco, st + 2 * OP_BYTES + SC_BYTES + wave * 256);
     };
 
     v16f acc[4][4];
@@ -106,56 +128,105 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    load_stage(0);
-    store_stage(0);
-    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < NSTAGE; ++s) issue_stage(s);
 
-    for (int kt = 0; kt < KT; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < KT) load_stage(kt + 1);
+    // LDS offsets of this lane's operand rows (row-major 64-byte rows, swizzled chunks)
+    int offa[4], offb[4], swz_a[4], swz_b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ra_ = wm * 128 + i * 32 + r, rb_ = wn * 128 + i * 32 + r;
+        offa[i] = ra_ * ROWB; swz_a[i] = (ra_ >> 2) & 3;
+        offb[i] = rb_ * ROWB; swz_b[i] = (rb_ >> 2) & 3;
+    }
 
-        int sca[4], scb[4];
+    // One matrix-instruction step's operands: 4 + 4 fragments and their scale words.  Two sets alternate: while
+    // the 16 instructions of one set run, the LDS reads of the next set are in flight.
+    struct Frag { v8i a[4], b[4]; int sa[4], sb[4]; };
+
+    // reads the operands of step s of stage kt out of the ring
+    auto read_frags = [&](Frag& f, int kt, int s) __attribute__((always_inline)) {
+        const uint8_t* st = smem + (kt % NSTAGE) * STAGE_BYTES;
+        const uint8_t* la = st;
+        const uint8_t* lb = st + OP_BYTES;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            sca[i] = (int)(lds_sa[buf][wm * 128 + i * 32 + r] >> (8 * h));
-            scb[i] = (int)(lds_sb[buf][wn * 128 + i * 32 + r] >> (8 * h));
-        }
-#pragma unroll
-        for (int s = 0; s < STEPS; ++s) {
-            v8i fa[4], fb[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint8_t* pa = &lds_a[buf][(wm * 128 + i * 32 + r) * PITCH];
-                const uint8_t* pb = &lds_b[buf][(wn * 128 + i * 32 + r) * PITCH];
-                if constexpr (FP4) {
-                    const v4i xa = *reinterpret_cast<const v4i*>(pa + (2 * s + h) * 16);
-                    const v4i xb = *reinterpret_cast<const v4i*>(pb + (2 * s + h) * 16);
-                    fa[i] = (v8i){xa[0], xa[1], xa[2], xa[3], 0, 0, 0, 0};
-                    fb[i] = (v8i){xb[0], xb[1], xb[2], xb[3], 0, 0, 0, 0};
-                } else {
-                    // 8-bit operands: registers 0-3 of both lane halves form MX block 0 (scaled by the byte
-                    // lane half 0 supplies), registers 4-7 form block 1 (scaled by lane half 1's byte)
-                    const v4i xa0 = *reinterpret_cast<const v4i*>(pa + h * 16);
-                    const v4i xa1 = *reinterpret_cast<const v4i*>(pa + h * 16 + 32);
-                    const v4i xb0 = *reinterpret_cast<const v4i*>(pb + h * 16);
-                    const v4i xb1 = *reinterpret_cast<const v4i*>(pb + h * 16 + 32);
-                    fa[i] = (v8i){xa0[0], xa0[1], xa0[2], xa0[3], xa1[0], xa1[1], xa1[2], xa1[3]};
-                    fb[i] = (v8i){xb0[0], xb0[1], xb0[2], xb0[3], xb1[0], xb1[1], xb1[2], xb1[3]};
-                }
+            const int ra_ = wm * 128 + i * 32 + r, rb_ = wn * 128 + i * 32 + r;
+            if constexpr (FP4) {
+                f.sa[i] = st[2 * OP_BYTES + ra_ * 4 + 2 * s + h];
+                f.sb[i] = st[2 * OP_BYTES + SC_BYTES + rb_ * 4 + 2 * s + h];
+                const v4i xa = *reinterpret_cast<const v4i*>(la + offa[i] + (((2 * s + h) ^ swz_a[i]) * 16));
+                const v4i xb = *reinterpret_cast<const v4i*>(lb + offb[i] + (((2 * s + h) ^ swz_b[i]) * 16));
+                f.a[i] = (v8i){xa[0], xa[1], xa[2], xa[3], 0, 0, 0, 0};
+                f.b[i] = (v8i){xb[0], xb[1], xb[2], xb[3], 0, 0, 0, 0};
+            } else {
+                // 8-bit operands: registers 0-3 of both lane halves form MX block 0 (scaled by the byte
+                // lane half 0 supplies), registers 4-7 form block 1 (scaled by lane half 1's byte)
+                f.sa[i] = st[2 * OP_BYTES + ra_ * 4 + 2 * (kt & 1) + h];
+                f.sb[i] = st[2 * OP_BYTES + SC_BYTES + rb_ * 4 + 2 * (kt & 1) + h];
+                const v4i xa0 = *reinterpret_cast<const v4i*>(la + offa[i] + ((h ^ swz_a[i]) * 16));
+                const v4i xa1 = *reinterpret_cast<const v4i*>(la + offa[i] + (((h + 2) ^ swz_a[i]) * 16));
+                const v4i xb0 = *reinterpret_cast<const v4i*>(lb + offb[i] + ((h ^ swz_b[i]) * 16));
+                const v4i xb1 = *reinterpret_cast<const v4i*>(lb + offb[i] + (((h + 2) ^ swz_b[i]) * 16));
+                f.a[i] = (v8i){xa0[0], xa0[1], xa0[2], xa0[3], xa1[0], xa1[1], xa1[2], xa1[3]};
+                f.b[i] = (v8i){xb0[0], xb0[1], xb0[2], xb0[3], xb1[0], xb1[1], xb1[2], xb1[3]};
             }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    if (s == 0)
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], FMT, FMT, 0, sca[i], 0, scb[j]);
-                    else
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], FMT, FMT, 2, sca[i], 2, scb[j]);
-                }
         }
-        if (kt + 1 < KT) store_stage(buf ^ 1);
+    };
+    auto multiply = [&](const Frag& f) __attribute__((always_inline)) {
+        constexpr int OPSEL = 0;                         // the lane's scale byte was read into bits 7:0
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMT, OPSEL, f.sa[i], OPSEL, f.sb[j]);
+    };
+    // Stage kt has been read into registers by every wave: wait until stage kt+1 has landed (the loads of
+    // stages kt+2 and kt+3 may stay in flight), then refill stage kt's buffer with stage kt+NSTAGE.
+    auto advance = [&](int kt) __attribute__((always_inline)) {
+        constexpr int keep = (NSTAGE - 2) * LOADS_PER_STAGE;
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0070 | (keep & 15) | ((keep >> 4) << 14));     // vmcnt(keep), lgkmcnt(0)
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        issue_stage(kt + NSTAGE);
+    };
+
+    Frag f0, f1;
+    {
+        constexpr int keep = (NSTAGE - 1) * LOADS_PER_STAGE;
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0070 | (keep & 15) | ((keep >> 4) << 14));
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
     }
+    read_frags(f0, 0, 0);
+    if constexpr (FP4) {
+        // a stage is two steps: the second step's operands load under the first step's instructions, and the
+        // next stage's first operands (after the barrier that publishes it) under the second step's
+        for (int kt = 0; kt < KT; ++kt) {
+            read_frags(f1, kt, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(f0);
+            advance(kt);
+            read_frags(f0, kt + 1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(f1);
+        }
+    } else {
+        // a stage is one step; two stages per trip so that the two operand sets keep their registers
+        for (int kt = 0; kt < KT; kt += 2) {
+            advance(kt);
+            read_frags(f1, kt + 1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(f0);
+            advance(kt + 1);
+            read_frags(f0, kt + 2, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(f1);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
 
     // epilogue: accumulator register e of lane (h, r) is C[8*(e/4) + 4*h + e%4][r] of its 32x32 block
     OutT* c = static_cast<OutT*>(g.c);
@@ -172,11 +243,22 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         }
 }
 
+template <int FMT, typename OutT>
+void launch_one(const GemmArgs& g, dim3 grid, hipStream_t st) {
+    static bool attr_set = false;      // idempotent; a race only repeats the same call
+    auto kern = gemm_mx_kernel<FMT, OutT>;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(256), SMEM_BYTES, st, g);
+}
+
 template <int FMT>
 void launch_fmt(const GemmArgs& g, int c_dtype, dim3 grid, hipStream_t st) {
-    if (c_dtype == MPSA_BF16)      hipLaunchKernelGGL((gemm_mx_kernel<FMT, __bf16>), grid, dim3(256), 0, st, g);
-    else if (c_dtype == MPSA_F16)  hipLaunchKernelGGL((gemm_mx_kernel<FMT, _Float16>), grid, dim3(256), 0, st, g);
-    else                           hipLaunchKernelGGL((gemm_mx_kernel<FMT, float>), grid, dim3(256), 0, st, g);
+    if (c_dtype == MPSA_BF16)      launch_one<FMT, __bf16>(g, grid, st);
+    else if (c_dtype == MPSA_F16)  launch_one<FMT, _Float16>(g, grid, st);
+    else                           launch_one<FMT, float>(g, grid, st);
 }
 
 }  // namespace
