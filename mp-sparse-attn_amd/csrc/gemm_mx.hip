@@ -14,11 +14,17 @@
 // (each half holds 16 bytes of either block).  Either way fragments are plain 16-byte pieces of the
 // row-major HBM layout.  K advances 64 bytes of codes per row per stage (128 E2M1 or 64 8-bit elements).
 //
-// Staging.  Codes and scale bytes go HBM/L2 -> LDS with direct-to-LDS loads (no registers, no LDS-write
-// instructions) into a ring of four stages, three of them in flight while one is being multiplied: with one
-// workgroup per CU nothing else hides the memory latency.  The 16-byte chunks of a row are XOR-swizzled with
-// the row index so that the 128-bit operand reads of 16 consecutive rows hit 16 distinct 4-bank groups.  One
-// barrier per stage.  Wave tiles of 128x128 keep LDS reads at 8 operand fragments per 16 matrix instructions.
+// Staging.  Codes go HBM/L2 -> LDS with direct-to-LDS loads (no registers, no LDS-write instructions) into a
+// ring of four stages, three of them in flight while one is being multiplied: with one workgroup per CU nothing
+// else hides the memory latency.  The 16-byte chunks of a row are XOR-swizzled with the row index so that the
+// 128-bit operand reads of 16 consecutive rows hit 16 distinct 4-bank groups.  One barrier per stage.  Wave
+// tiles of 128x128 keep LDS reads at 8 operand fragments per 16 matrix instructions.
+//
+// Scale bytes.  A row's scale bytes for one stage are 4 (or 2) bytes in a line of their own, so fetching them
+// stage by stage costs the vector memory path one cache-line access per row per stage - as many accesses as
+// the codes themselves.  When K is a multiple of 512 the kernel instead fetches 16 scale bytes per row at a
+// time (a "group" of 4 stages of 4-bit codes, 8 stages of 8-bit codes) into a double-buffered LDS area, one
+// group ahead.  Other K fall back to one 4-byte scale load per row per stage.
 #include "mpsa_common.h"
 
 namespace {
@@ -27,10 +33,15 @@ constexpr int BM = 256, BN = 256;       // workgroup tile
 constexpr int ROWB = 64;                // code bytes per row per stage
 constexpr int NSTAGE = 4;               // LDS ring depth
 constexpr int OP_BYTES = BM * ROWB;     // one operand's codes per stage (16 KiB)
-constexpr int SC_BYTES = BM * 4;        // one operand's scale bytes per stage (4 per row)
-constexpr int STAGE_BYTES = 2 * OP_BYTES + 2 * SC_BYTES;
-constexpr int SMEM_BYTES = NSTAGE * STAGE_BYTES;
-constexpr int LOADS_PER_STAGE = 2 * (OP_BYTES / 1024 / 4) + 2;   // direct-to-LDS instructions per wave per stage (10)
+constexpr int SC_BYTES = BM * 4;        // narrow path: one operand's scale bytes per stage (4 per row)
+constexpr int SCG_BYTES = BM * 16;      // wide path: one operand's scale bytes per group (16 per row)
+constexpr int CODE_LOADS = 2 * (OP_BYTES / 1024 / 4);   // direct-to-LDS code instructions per wave per stage (8)
+
+template <bool WIDE> constexpr int stage_bytes() { return WIDE ? 2 * OP_BYTES : 2 * OP_BYTES + 2 * SC_BYTES; }
+template <bool WIDE> constexpr int smem_bytes() { return NSTAGE * stage_bytes<WIDE>() + (WIDE ? 4 * SCG_BYTES : 0); }
+
+// s_waitcnt immediate: vmcnt(vm), lgkmcnt(0), expcnt untouched
+constexpr int wait_imm(int vm) { return 0x0070 | (vm & 15) | ((vm >> 4) << 14); }
 
 struct GemmArgs {
     const uint8_t *a, *sa, *b, *sb;
@@ -57,14 +68,17 @@ __device__ __forceinline__ void load_to_lds(const uint8_t* gsrc, uint8_t* lds_wa
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(gsrc) : "memory", "m0");
 }
 
-template <int FMT, typename OutT>
+template <int FMT, typename OutT, bool WIDE>
 __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     constexpr bool FP4 = (FMT == MPSA_FMT_E2M1);
+    constexpr int STAGE_BYTES = stage_bytes<WIDE>();
+    constexpr int GROUP = FP4 ? 4 : 8;                 // stages covered by 16 scale bytes of a row
     const int row_bytes = FP4 ? g.K / 2 : g.K;         // code bytes per matrix row
     const int srow_bytes = g.K / 32;
     const int KT = row_bytes / ROWB;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint8_t* const scg = smem + NSTAGE * STAGE_BYTES;  // wide path: [group parity][operand][row][16]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -113,11 +127,21 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
             load_to_lds<16>(ga[c] + (int64_t)kc * ROWB, st + (wave * 4 + c) * 1024);
             load_to_lds<16>(gb[c] + (int64_t)kc * ROWB, st + OP_BYTES + (wave * 4 + c) * 1024);
         }
-        // four scale bytes per row: the stage's own with 4-bit codes; with 8-bit codes the aligned word that
-        // holds this stage's two bytes (the stage count is even, so the word is inside the row)
-        const int sco = FP4 ? kc * 4 : (kc >> 1) * 4;
-        load_to_lds<4>(gsa + sco, st + 2 * OP_BYTES + wave * 256);
-        load_to_lds<4>(gsb + sco, st + 2 * OP_BYTES + SC_BYTES + wave * 256);
+        if constexpr (!WIDE) {
+            // four scale bytes per row: the stage's own with 4-bit codes; with 8-bit codes the aligned word that
+            // holds this stage's two bytes (the stage count is even, so the word is inside the row)
+            const int sco = FP4 ? kc * 4 : (kc >> 1) * 4;
+            load_to_lds<4>(gsa + sco, st + 2 * OP_BYTES + wave * 256);
+            load_to_lds<4>(gsb + sco, st + 2 * OP_BYTES + SC_BYTES + wave * 256);
+        }
+    };
+    // wide path: the 16 scale bytes per row of group grp (two instructions per wave)
+    auto issue_scales = [&](int grp) __attribute__((always_inline)) {
+        const int ng = KT / GROUP;
+        const int gc = grp < ng ? grp : ng - 1;
+        uint8_t* dst = scg + (grp & 1) * 2 * SCG_BYTES + wave * 1024;
+        load_to_lds<16>(gsa + gc * 16, dst);
+        load_to_lds<16>(gsb + gc * 16, dst + SCG_BYTES);
     };
 
     v16f acc[4][4];
@@ -128,6 +152,7 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
+    if constexpr (WIDE) issue_scales(0);
 #pragma unroll
     for (int s = 0; s < NSTAGE; ++s) issue_stage(s);
 
@@ -140,7 +165,7 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         offb[i] = rb_ * ROWB; swz_b[i] = (rb_ >> 2) & 3;
     }
 
-    // One matrix-instruction step's operands: 4 + 4 fragments and their scale words.  Two sets alternate: while
+    // One matrix-instruction step's operands: 4 + 4 fragments and their scale bytes.  Two sets alternate: while
     // the 16 instructions of one set run, the LDS reads of the next set are in flight.
     struct Frag { v8i a[4], b[4]; int sa[4], sb[4]; };
 
@@ -149,12 +174,23 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         const uint8_t* st = smem + (kt % NSTAGE) * STAGE_BYTES;
         const uint8_t* la = st;
         const uint8_t* lb = st + OP_BYTES;
+        // the lane's scale byte of this step: byte 2s+h of the stage's four (4-bit codes), byte h of its two (8-bit)
+        const uint8_t* sca;
+        int sstride;
+        if constexpr (WIDE) {
+            sca = scg + ((kt / GROUP) & 1) * 2 * SCG_BYTES + (FP4 ? 4 * (kt % GROUP) + 2 * s + h : 2 * (kt % GROUP) + h);
+            sstride = 16;
+        } else {
+            sca = st + 2 * OP_BYTES + (FP4 ? 2 * s + h : 2 * (kt & 1) + h);
+            sstride = 4;
+        }
+        const uint8_t* scb = sca + (WIDE ? SCG_BYTES : SC_BYTES);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int ra_ = wm * 128 + i * 32 + r, rb_ = wn * 128 + i * 32 + r;
+            f.sa[i] = sca[ra_ * sstride];
+            f.sb[i] = scb[rb_ * sstride];
             if constexpr (FP4) {
-                f.sa[i] = st[2 * OP_BYTES + ra_ * 4 + 2 * s + h];
-                f.sb[i] = st[2 * OP_BYTES + SC_BYTES + rb_ * 4 + 2 * s + h];
                 const v4i xa = *reinterpret_cast<const v4i*>(la + offa[i] + (((2 * s + h) ^ swz_a[i]) * 16));
                 const v4i xb = *reinterpret_cast<const v4i*>(lb + offb[i] + (((2 * s + h) ^ swz_b[i]) * 16));
                 f.a[i] = (v8i){xa[0], xa[1], xa[2], xa[3], 0, 0, 0, 0};
@@ -162,8 +198,6 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
             } else {
                 // 8-bit operands: registers 0-3 of both lane halves form MX block 0 (scaled by the byte
                 // lane half 0 supplies), registers 4-7 form block 1 (scaled by lane half 1's byte)
-                f.sa[i] = st[2 * OP_BYTES + ra_ * 4 + 2 * (kt & 1) + h];
-                f.sb[i] = st[2 * OP_BYTES + SC_BYTES + rb_ * 4 + 2 * (kt & 1) + h];
                 const v4i xa0 = *reinterpret_cast<const v4i*>(la + offa[i] + ((h ^ swz_a[i]) * 16));
                 const v4i xa1 = *reinterpret_cast<const v4i*>(la + offa[i] + (((h + 2) ^ swz_a[i]) * 16));
                 const v4i xb0 = *reinterpret_cast<const v4i*>(lb + offb[i] + ((h ^ swz_b[i]) * 16));
@@ -174,29 +208,49 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         }
     };
     auto multiply = [&](const Frag& f) __attribute__((always_inline)) {
-        constexpr int OPSEL = 0;                         // the lane's scale byte was read into bits 7:0
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMT, OPSEL, f.sa[i], OPSEL, f.sb[j]);
+            for (int j = 0; j < 4; ++j)   // op_sel 0: the lane's scale byte was read into bits 7:0
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMT, 0, f.sa[i], 0, f.sb[j]);
     };
-    // Stage kt has been read into registers by every wave: wait until stage kt+1 has landed (the loads of
-    // stages kt+2 and kt+3 may stay in flight), then refill stage kt's buffer with stage kt+NSTAGE.
+    // Stage kt has been read into registers by every wave.  Wait until stage kt+1 has landed - everything but
+    // the loads of the two trips before this one - then refill stage kt's buffer with stage kt+NSTAGE.  On the
+    // wide path the first trip of a group also fetches the next group's scale bytes; they land, like that
+    // trip's codes, three trips later, before the next group's first stage is read.  (The wait leaves 16
+    // loads in flight on the wide path although the two trips after a scale fetch have issued 18: waiting
+    // for two loads more than needed is harmless and keeps the count a constant.)
     auto advance = [&](int kt) __attribute__((always_inline)) {
-        constexpr int keep = (NSTAGE - 2) * LOADS_PER_STAGE;
+        constexpr int KEEP = 2 * (WIDE ? CODE_LOADS : CODE_LOADS + 2);
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0x0070 | (keep & 15) | ((keep >> 4) << 14));     // vmcnt(keep), lgkmcnt(0)
+        __builtin_amdgcn_s_waitcnt(wait_imm(KEEP));
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         issue_stage(kt + NSTAGE);
+        if constexpr (WIDE) {
+            if (kt % GROUP == 0) issue_scales(kt / GROUP + 1);
+        }
+    };
+
+    // Issue order of one step: the LDS reads of the other operand set go out between the matrix instructions
+    // of this one (front-loaded), so that the matrix pipe keeps running while the reads are issued.
+    auto interleave = [&]() __attribute__((always_inline)) {
+        constexpr int READS = FP4 ? 16 : 24;               // 8 fragment reads (16 with 8-bit codes) + 8 scale bytes
+        constexpr int PER = READS / 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one matrix instruction
+            __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);    // PER LDS reads
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+        __builtin_amdgcn_sched_barrier(0);
     };
 
     Frag f0, f1;
     {
-        constexpr int keep = (NSTAGE - 1) * LOADS_PER_STAGE;
+        constexpr int KEEP = (NSTAGE - 1) * (WIDE ? CODE_LOADS : CODE_LOADS + 2);
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0x0070 | (keep & 15) | ((keep >> 4) << 14));
+        __builtin_amdgcn_s_waitcnt(wait_imm(KEEP));
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -206,24 +260,24 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         // next stage's first operands (after the barrier that publishes it) under the second step's
         for (int kt = 0; kt < KT; ++kt) {
             read_frags(f1, kt, 1);
-            __builtin_amdgcn_sched_barrier(0);
             multiply(f0);
+            interleave();
             advance(kt);
             read_frags(f0, kt + 1, 0);
-            __builtin_amdgcn_sched_barrier(0);
             multiply(f1);
+            interleave();
         }
     } else {
         // a stage is one step; two stages per trip so that the two operand sets keep their registers
         for (int kt = 0; kt < KT; kt += 2) {
             advance(kt);
             read_frags(f1, kt + 1, 0);
-            __builtin_amdgcn_sched_barrier(0);
             multiply(f0);
+            interleave();
             advance(kt + 1);
             read_frags(f0, kt + 2, 0);
-            __builtin_amdgcn_sched_barrier(0);
             multiply(f1);
+            interleave();
         }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
@@ -243,15 +297,21 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         }
 }
 
-template <int FMT, typename OutT>
-void launch_one(const GemmArgs& g, dim3 grid, hipStream_t st) {
+template <int FMT, typename OutT, bool WIDE>
+void launch_kernel(const GemmArgs& g, dim3 grid, hipStream_t st) {
     static bool attr_set = false;      // idempotent; a race only repeats the same call
-    auto kern = gemm_mx_kernel<FMT, OutT>;
+    auto kern = gemm_mx_kernel<FMT, OutT, WIDE>;
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes<WIDE>());
         attr_set = true;
     }
-    hipLaunchKernelGGL(kern, grid, dim3(256), SMEM_BYTES, st, g);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem_bytes<WIDE>(), st, g);
+}
+
+template <int FMT, typename OutT>
+void launch_one(const GemmArgs& g, dim3 grid, hipStream_t st) {
+    if (g.K % 512 == 0) launch_kernel<FMT, OutT, true>(g, grid, st);
+    else                launch_kernel<FMT, OutT, false>(g, grid, st);
 }
 
 template <int FMT>

@@ -48,7 +48,7 @@ def _operands(M, N, K, bst, seed):
 
 
 @pytest.mark.parametrize("bst", ["mxfp4", "mxfp8", "mxfp8e5"])
-@pytest.mark.parametrize("shape", [(256, 256, 128), (512, 768, 1024), (256, 1024, 4096)])
+@pytest.mark.parametrize("shape", [(256, 256, 128), (512, 768, 1024), (256, 1024, 4096), (256, 512, 640), (512, 256, 1536)])
 def test_quantize_then_matmul_matches_oracle(bst, shape):
     M, N, K = shape
     a, b, (ac, asc, bc, bsc, cfg) = _operands(M, N, K, bst, seed=M + K)
