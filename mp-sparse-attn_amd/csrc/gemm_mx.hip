@@ -119,21 +119,26 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     }
     const uint8_t* gsa = g.sa + (int64_t)(m0 + wave * 64 + lane) * srow_bytes;
     const uint8_t* gsb = g.sb + (int64_t)(n0 + wave * 64 + lane) * srow_bytes;
-    auto issue_stage = [&](int kt) __attribute__((always_inline)) {
+    // a stage's loads go out in four parts (two code instructions each, the narrow path's scale words with the
+    // last) so that they can be spread between the matrix instructions of a step
+    auto issue_part = [&](int kt, int part) __attribute__((always_inline)) {
         const int kc = kt < KT ? kt : KT - 1;             // past the end: re-load the last stage (keeps the count uniform)
         uint8_t* st = smem + (kt % NSTAGE) * STAGE_BYTES;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            load_to_lds<16>(ga[c] + (int64_t)kc * ROWB, st + (wave * 4 + c) * 1024);
-            load_to_lds<16>(gb[c] + (int64_t)kc * ROWB, st + OP_BYTES + (wave * 4 + c) * 1024);
-        }
+        load_to_lds<16>(ga[part] + (int64_t)kc * ROWB, st + (wave * 4 + part) * 1024);
+        load_to_lds<16>(gb[part] + (int64_t)kc * ROWB, st + OP_BYTES + (wave * 4 + part) * 1024);
         if constexpr (!WIDE) {
-            // four scale bytes per row: the stage's own with 4-bit codes; with 8-bit codes the aligned word that
-            // holds this stage's two bytes (the stage count is even, so the word is inside the row)
-            const int sco = FP4 ? kc * 4 : (kc >> 1) * 4;
-            load_to_lds<4>(gsa + sco, st + 2 * OP_BYTES + wave * 256);
-            load_to_lds<4>(gsb + sco, st + 2 * OP_BYTES + SC_BYTES + wave * 256);
+            if (part == 3) {
+                // four scale bytes per row: the stage's own with 4-bit codes; with 8-bit codes the aligned word
+                // that holds this stage's two bytes (the stage count is even, so the word is inside the row)
+                const int sco = FP4 ? kc * 4 : (kc >> 1) * 4;
+                load_to_lds<4>(gsa + sco, st + 2 * OP_BYTES + wave * 256);
+                load_to_lds<4>(gsb + sco, st + 2 * OP_BYTES + SC_BYTES + wave * 256);
+            }
         }
+    };
+    auto issue_stage = [&](int kt) __attribute__((always_inline)) {
+#pragma unroll
+        for (int part = 0; part < 4; ++part) issue_part(kt, part);
     };
     // wide path: the 16 scale bytes per row of group grp (two instructions per wave)
     auto issue_scales = [&](int grp) __attribute__((always_inline)) {
@@ -169,80 +174,86 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     // the 16 instructions of one set run, the LDS reads of the next set are in flight.
     struct Frag { v8i a[4], b[4]; int sa[4], sb[4]; };
 
-    // reads the operands of step s of stage kt out of the ring
-    auto read_frags = [&](Frag& f, int kt, int s) __attribute__((always_inline)) {
+    // reads operands of step s of stage kt out of the ring: part 0 the B fragments and their scale bytes,
+    // part 1 the A fragments and theirs
+    auto read_part = [&](Frag& f, int kt, int s, int part) __attribute__((always_inline)) {
         const uint8_t* st = smem + (kt % NSTAGE) * STAGE_BYTES;
-        const uint8_t* la = st;
-        const uint8_t* lb = st + OP_BYTES;
         // the lane's scale byte of this step: byte 2s+h of the stage's four (4-bit codes), byte h of its two (8-bit)
-        const uint8_t* sca;
+        const uint8_t* sc;
         int sstride;
         if constexpr (WIDE) {
-            sca = scg + ((kt / GROUP) & 1) * 2 * SCG_BYTES + (FP4 ? 4 * (kt % GROUP) + 2 * s + h : 2 * (kt % GROUP) + h);
+            sc = scg + ((kt / GROUP) & 1) * 2 * SCG_BYTES + (FP4 ? 4 * (kt % GROUP) + 2 * s + h : 2 * (kt % GROUP) + h);
             sstride = 16;
         } else {
-            sca = st + 2 * OP_BYTES + (FP4 ? 2 * s + h : 2 * (kt & 1) + h);
+            sc = st + 2 * OP_BYTES + (FP4 ? 2 * s + h : 2 * (kt & 1) + h);
             sstride = 4;
         }
-        const uint8_t* scb = sca + (WIDE ? SCG_BYTES : SC_BYTES);
+        const bool isb = part == 0;
+        const uint8_t* lx = isb ? st + OP_BYTES : st;
+        if (isb) sc += WIDE ? SCG_BYTES : SC_BYTES;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int ra_ = wm * 128 + i * 32 + r, rb_ = wn * 128 + i * 32 + r;
-            f.sa[i] = sca[ra_ * sstride];
-            f.sb[i] = scb[rb_ * sstride];
+            const int row = (isb ? wn : wm) * 128 + i * 32 + r;
+            const int off = isb ? offb[i] : offa[i], swz = isb ? swz_b[i] : swz_a[i];
+            int& fs = isb ? f.sb[i] : f.sa[i];
+            v8i& fx = isb ? f.b[i] : f.a[i];
+            fs = sc[row * sstride];
             if constexpr (FP4) {
-                const v4i xa = *reinterpret_cast<const v4i*>(la + offa[i] + (((2 * s + h) ^ swz_a[i]) * 16));
-                const v4i xb = *reinterpret_cast<const v4i*>(lb + offb[i] + (((2 * s + h) ^ swz_b[i]) * 16));
-                f.a[i] = (v8i){xa[0], xa[1], xa[2], xa[3], 0, 0, 0, 0};
-                f.b[i] = (v8i){xb[0], xb[1], xb[2], xb[3], 0, 0, 0, 0};
+                const v4i x = *reinterpret_cast<const v4i*>(lx + off + (((2 * s + h) ^ swz) * 16));
+                fx = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
             } else {
                 // 8-bit operands: registers 0-3 of both lane halves form MX block 0 (scaled by the byte
                 // lane half 0 supplies), registers 4-7 form block 1 (scaled by lane half 1's byte)
-                const v4i xa0 = *reinterpret_cast<const v4i*>(la + offa[i] + ((h ^ swz_a[i]) * 16));
-                const v4i xa1 = *reinterpret_cast<const v4i*>(la + offa[i] + (((h + 2) ^ swz_a[i]) * 16));
-                const v4i xb0 = *reinterpret_cast<const v4i*>(lb + offb[i] + ((h ^ swz_b[i]) * 16));
-                const v4i xb1 = *reinterpret_cast<const v4i*>(lb + offb[i] + (((h + 2) ^ swz_b[i]) * 16));
-                f.a[i] = (v8i){xa0[0], xa0[1], xa0[2], xa0[3], xa1[0], xa1[1], xa1[2], xa1[3]};
-                f.b[i] = (v8i){xb0[0], xb0[1], xb0[2], xb0[3], xb1[0], xb1[1], xb1[2], xb1[3]};
+                const v4i x0 = *reinterpret_cast<const v4i*>(lx + off + ((h ^ swz) * 16));
+                const v4i x1 = *reinterpret_cast<const v4i*>(lx + off + (((h + 2) ^ swz) * 16));
+                fx = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
             }
         }
     };
-    auto multiply = [&](const Frag& f) __attribute__((always_inline)) {
+    // the four matrix instructions of accumulator row i
+    auto multiply_row = [&](const Frag& f, int i) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)   // op_sel 0: the lane's scale byte was read into bits 7:0
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMT, 0, f.sa[i], 0, f.sb[j]);
+        for (int j = 0; j < 4; ++j)   // op_sel 0: the lane's scale byte was read into bits 7:0
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMT, 0, f.sa[i], 0, f.sb[j]);
     };
-    // Stage kt has been read into registers by every wave.  Wait until stage kt+1 has landed - everything but
-    // the loads of the two trips before this one - then refill stage kt's buffer with stage kt+NSTAGE.  On the
-    // wide path the first trip of a group also fetches the next group's scale bytes; they land, like that
-    // trip's codes, three trips later, before the next group's first stage is read.  (The wait leaves 16
-    // loads in flight on the wide path although the two trips after a scale fetch have issued 18: waiting
-    // for two loads more than needed is harmless and keeps the count a constant.)
-    auto advance = [&](int kt) __attribute__((always_inline)) {
+    // One step: the 16 matrix instructions on operand set `cur`, in four rows.  Between them go the LDS reads
+    // that fill the other set `nxt` with step ns of stage nkt (rows 0 and 1) and, when `refill` is set, the
+    // loads of stage lkt into the buffer of stage lkt-NSTAGE (two per row; on the wide path the first stage of
+    // a group also brings the next group's scale bytes), so that the matrix pipe keeps running while they issue.
+    auto step = [&](const Frag& cur, Frag& nxt, int nkt, int ns, bool refill, int lkt) __attribute__((always_inline)) {
+        constexpr int PER = FP4 ? 2 : 3;                   // LDS reads issued behind each matrix instruction
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (refill) {
+                issue_part(lkt, i);
+                if constexpr (WIDE) {
+                    if (i == 3 && (lkt - NSTAGE) % GROUP == 0) issue_scales((lkt - NSTAGE) / GROUP + 1);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (i < 2) read_part(nxt, nkt, ns, i);
+            multiply_row(cur, i);
+            if (i < 2) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one matrix instruction
+                    __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);    // PER LDS reads
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // Every wave has read stage kt into registers.  Wait until stage kt+1 has landed - everything but the loads
+    // of the two stages issued last - and meet the other waves; after that stage kt's buffer may be refilled.
+    // The next group's scale bytes, fetched with the first stage of a group, land like that stage's codes three
+    // stages later, before the next group's first stage is read.  (The wait leaves 16 loads in flight on the
+    // wide path although the two stages after a scale fetch amount to 18: waiting for two loads more than
+    // needed is harmless and keeps the count a constant.)
+    auto publish = [&]() __attribute__((always_inline)) {
         constexpr int KEEP = 2 * (WIDE ? CODE_LOADS : CODE_LOADS + 2);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(wait_imm(KEEP));
         __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
-        issue_stage(kt + NSTAGE);
-        if constexpr (WIDE) {
-            if (kt % GROUP == 0) issue_scales(kt / GROUP + 1);
-        }
-    };
-
-    // Issue order of one step: the LDS reads of the other operand set go out between the matrix instructions
-    // of this one (front-loaded), so that the matrix pipe keeps running while the reads are issued.
-    auto interleave = [&]() __attribute__((always_inline)) {
-        constexpr int READS = FP4 ? 16 : 24;               // 8 fragment reads (16 with 8-bit codes) + 8 scale bytes
-        constexpr int PER = READS / 8;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one matrix instruction
-            __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);    // PER LDS reads
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
 
@@ -254,30 +265,23 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
     }
-    read_frags(f0, 0, 0);
+    read_part(f0, 0, 0, 0);
+    read_part(f0, 0, 0, 1);
     if constexpr (FP4) {
         // a stage is two steps: the second step's operands load under the first step's instructions, and the
         // next stage's first operands (after the barrier that publishes it) under the second step's
         for (int kt = 0; kt < KT; ++kt) {
-            read_frags(f1, kt, 1);
-            multiply(f0);
-            interleave();
-            advance(kt);
-            read_frags(f0, kt + 1, 0);
-            multiply(f1);
-            interleave();
+            step(f0, f1, kt, 1, false, 0);
+            publish();
+            step(f1, f0, kt + 1, 0, true, kt + NSTAGE);
         }
     } else {
         // a stage is one step; two stages per trip so that the two operand sets keep their registers
         for (int kt = 0; kt < KT; kt += 2) {
-            advance(kt);
-            read_frags(f1, kt + 1, 0);
-            multiply(f0);
-            interleave();
-            advance(kt + 1);
-            read_frags(f0, kt + 2, 0);
-            multiply(f1);
-            interleave();
+            publish();
+            step(f0, f1, kt + 1, 0, true, kt + NSTAGE);
+            publish();
+            step(f1, f0, kt + 2, 0, true, kt + 1 + NSTAGE);
         }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
