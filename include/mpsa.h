@@ -69,6 +69,9 @@ int mpsa_e8m0_decode(const uint8_t* codes, int64_t n, float* out, mpsa_stream_t 
  *
  *   x          [B,H,N,D] of x_dtype (MPSA_BF16 | MPSA_F16), element strides x_strides[4],
  *              last dim contiguous, D % 32 == 0, rows 16-byte aligned
+ *   sub        NULL, or [B,H,D] of x_dtype (contiguous, 16-byte aligned): x := round_to_x_dtype(x - sub) row by
+ *              row before anything else - the smooth-K step k - k.mean(dim=-2) of ours/mxfp_attn.py:44-45 and
+ *              ours/mxfp_attn_kernel.py:33-34 with the mean from mpsa_seq_mean
  *   pre_scale  float32 factor multiplied in before quantizing (sm_scale*log2(e) for Q, 1 for K)
  *   fmt        MPSA_FMT_E2M1 | MPSA_FMT_E4M3 | MPSA_FMT_E5M2
  *   emax_elem  shared exponent = floor(log2(amax)) - emax_elem (reference: 3 for E2M1, 7 for 8-bit)
@@ -78,7 +81,7 @@ int mpsa_e8m0_decode(const uint8_t* codes, int64_t n, float* out, mpsa_stream_t 
  *   out_rows   rows per (b,h) in the outputs, >= N; rows N..out_rows-1 are written as zero
  */
 int mpsa_quantize_mx(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
-                     const int64_t x_strides[4], float pre_scale, int fmt, int emax_elem,
+                     const int64_t x_strides[4], const void* sub, float pre_scale, int fmt, int emax_elem,
                      uint8_t* codes, uint8_t* scales, int64_t out_rows, mpsa_stream_t stream);
 
 /*
@@ -87,9 +90,24 @@ int mpsa_quantize_mx(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N
  * (fmt8, emax8); x is read once.  Replaces the same reference functions as above.
  */
 int mpsa_quantize_mx_dual(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
-                          const int64_t x_strides[4], float pre_scale, int emax4, int fmt8, int emax8,
+                          const int64_t x_strides[4], const void* sub, float pre_scale, int emax4, int fmt8, int emax8,
                           uint8_t* codes4, uint8_t* scales4, uint8_t* codes8, uint8_t* scales8,
                           int64_t out_rows, mpsa_stream_t stream);
+
+/*
+ * Mean over the sequence dim, per (batch, head, channel): mean[b,h,d] = round_to_x_dtype(float32 sum over n of
+ * x[b,h,n,d] * float32(1/N)).  Replaces the k.mean(dim=-2, keepdim=True) of the smooth-K prologue
+ * (ours/mxfp_attn.py:44-45, ours/mxfp_attn_kernel.py:33-34); the subtraction itself happens inside the quantizer
+ * (its sub argument).  The float32 additions run in a fixed order (256-row partial sums, then those in order), so the
+ * result is reproducible; it can differ from another summation order in the last bit of the 16-bit mean.
+ *
+ *   x          as for mpsa_quantize_mx, D in {64,128}
+ *   workspace  mpsa_seq_mean_workspace(B,H,N,D) bytes of device memory (float32 partial sums), caller-owned
+ *   mean       [B,H,D] of x_dtype
+ */
+int64_t mpsa_seq_mean_workspace(int64_t B, int64_t H, int64_t N, int64_t D);
+int mpsa_seq_mean(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                  const int64_t x_strides[4], float* workspace, void* mean, mpsa_stream_t stream);
 
 /*
  * Block-scaled matmul  C[M,N] = (A o 2^(sa-127)) (B o 2^(sb-127))^T.  Replaces block_scaled_matmul

@@ -7,6 +7,11 @@
 // (ours/mxfp.py:84-170) bit for bit, including its float32 1e-6 tie-break bias; codes leave the
 // kernel already nibble-packed (ours/mxfp.py:196-205: even element in the low nibble).
 //
+// Smooth-K (ours/mxfp_attn.py:44-45, ours/mxfp_attn_kernel.py:33-34: k = k - k.mean(dim=-2, keepdim=True) in k's
+// 16-bit dtype) is folded in: seq_mean_kernel + seq_mean_finish_kernel produce the per-(batch, head, channel) mean
+// over the sequence, rounded to the input dtype, and the quantizer subtracts it - rounding the difference to the
+// input dtype again, as the elementwise torch op would - before it does anything else.
+//
 // Work mapping: one lane owns 8 consecutive elements (one 128-bit load), four neighbouring lanes
 // own one MX block, so the block maximum is two DPP quad exchanges.  The kernel is HBM-bound:
 // 2 B/element in, 0.5 (+1) B/element of codes and 1/32 (x2) B/element of scales out.
@@ -17,6 +22,7 @@ namespace {
 
 struct QuantArgs {
     const void* x;
+    const void* sub;           // optional [B,H,D] of x's dtype, subtracted (and the difference rounded to that dtype) first
     int64_t sb, sh, sn;        // element strides of x
     int n, d;                  // valid rows, row length
     int out_rows;              // rows per (b,h) in the outputs
@@ -66,6 +72,17 @@ __device__ __forceinline__ void load8(const void* p, float (&x)[8]) {
     }
 }
 
+// round a float32 to the 16-bit dtype XDT (nearest even) and back
+template <int XDT>
+__device__ __forceinline__ float round16(float v) {
+    if constexpr (XDT == MPSA_BF16) {
+        const uint32_t u = mpsa_f2u(v);
+        return mpsa_u2f((u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u);
+    } else {
+        return (float)(_Float16)v;
+    }
+}
+
 template <int XDT, bool DO4, bool DO8, int FMT8, bool SW8>
 __global__ __launch_bounds__(256) void quantize_kernel(QuantArgs a) {
     const uint32_t cpr = (uint32_t)a.d >> 3;                              // 16-byte chunks per row
@@ -81,6 +98,12 @@ __global__ __launch_bounds__(256) void quantize_kernel(QuantArgs a) {
         const char* base = static_cast<const char*>(a.x) +
                            2 * ((int64_t)blockIdx.z * a.sb + (int64_t)blockIdx.y * a.sh + (int64_t)row * a.sn + 8 * (int64_t)col8);
         load8<XDT>(base, x);
+        if (a.sub) {
+            float m[8];
+            load8<XDT>(static_cast<const char*>(a.sub) + 2 * (head * a.d + 8 * (int64_t)col8), m);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] = round16<XDT>(x[i] - m[i]);
+        }
     } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i) x[i] = 0.0f;
@@ -130,6 +153,66 @@ __global__ __launch_bounds__(256) void quantize_kernel(QuantArgs a) {
     }
 }
 
+// ---- mean over the sequence, per (batch, head, channel) ----
+constexpr int MEAN_ROWS = 256;     // rows per partial sum
+
+struct MeanArgs {
+    const void* x;
+    int64_t sb, sh, sn;
+    int n, d, nchunk;
+    float* partial;            // [B,H,nchunk,D]
+    void* mean;                // [B,H,D] of x's dtype
+    float inv_n;
+};
+
+// One workgroup sums MEAN_ROWS rows of one head: a thread owns 8 channels of every (256*8/D)-th row; the row
+// groups are then added in a fixed order through LDS, so the result does not depend on timing.
+template <int XDT>
+__global__ __launch_bounds__(256) void seq_mean_kernel(MeanArgs a) {
+    __shared__ float part[256][9];
+    const int cpr = a.d >> 3;                    // 8-channel groups per row (8 or 16)
+    const int rthreads = 256 / cpr;
+    const int cg = threadIdx.x % cpr, rt = threadIdx.x / cpr;
+    const int chunk = blockIdx.x;
+    const int row0 = chunk * MEAN_ROWS;
+    const int row1 = min(row0 + MEAN_ROWS, a.n);
+    const char* base = static_cast<const char*>(a.x) + 2 * ((int64_t)blockIdx.z * a.sb + (int64_t)blockIdx.y * a.sh + 8 * (int64_t)cg);
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int row = row0 + rt; row < row1; row += rthreads) {
+        float x[8];
+        load8<XDT>(base + 2 * (int64_t)row * a.sn, x);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] += x[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) part[threadIdx.x][i] = acc[i];
+    __syncthreads();
+    if (threadIdx.x < a.d) {
+        const int c = threadIdx.x;               // channel
+        float s = 0.0f;
+        for (int t = 0; t < rthreads; ++t) s += part[t * cpr + (c >> 3)][c & 7];
+        const int64_t head = (int64_t)blockIdx.z * gridDim.y + blockIdx.y;
+        a.partial[(head * a.nchunk + chunk) * a.d + c] = s;
+    }
+}
+
+// adds a head's partial sums in chunk order, multiplies by 1/N (float32) and rounds to the 16-bit dtype
+template <int XDT>
+__global__ __launch_bounds__(128) void seq_mean_finish_kernel(MeanArgs a) {
+    const int c = threadIdx.x;
+    if (c >= a.d) return;
+    const int64_t head = blockIdx.x;
+    float s = 0.0f;
+    for (int k = 0; k < a.nchunk; ++k) s += a.partial[(head * a.nchunk + k) * a.d + c];
+    const float m = s * a.inv_n;
+    if constexpr (XDT == MPSA_BF16) {
+        const uint32_t u = mpsa_f2u(m);
+        static_cast<uint16_t*>(a.mean)[head * a.d + c] = (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+    } else {
+        static_cast<_Float16*>(a.mean)[head * a.d + c] = (_Float16)m;
+    }
+}
+
 bool use_sw_fp8() {
     static const bool sw = [] {
         const char* v = getenv("MPSA_FP8_ENCODE");
@@ -151,7 +234,7 @@ void launch(const QuantArgs& a, int fmt8, dim3 grid, hipStream_t st) {
 }
 
 int quantize_common(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D, const int64_t* xs,
-                    float pre, bool do4, int emax4, bool do8, int fmt8, int emax8,
+                    const void* sub, float pre, bool do4, int emax4, bool do8, int fmt8, int emax8,
                     uint8_t* c4, uint8_t* s4, uint8_t* c8, uint8_t* s8, int64_t out_rows, hipStream_t st) {
     if (!x || !xs) return mpsa_fail(MPSA_EINVAL, "quantize: null input");
     if ((do4 && (!c4 || !s4)) || (do8 && (!c8 || !s8))) return mpsa_fail(MPSA_EINVAL, "quantize: null output");
@@ -162,11 +245,12 @@ int quantize_common(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N,
     if (xs[3] != 1) return mpsa_fail(MPSA_EINVAL, "quantize: last dim of x must be contiguous");
     if (!mpsa_aligned16(x) || (xs[0] % 8) || (xs[1] % 8) || (xs[2] % 8)) return mpsa_fail(MPSA_EALIGN, "quantize: x rows must be 16-byte aligned");
     if ((do4 && !mpsa_aligned16(c4)) || (do8 && !mpsa_aligned16(c8))) return mpsa_fail(MPSA_EALIGN, "quantize: outputs must be 16-byte aligned");
+    if (sub && !mpsa_aligned16(sub)) return mpsa_fail(MPSA_EALIGN, "quantize: sub must be 16-byte aligned");
     if (B == 0 || H == 0 || out_rows == 0) return MPSA_OK;
     const int64_t chunks = out_rows * (D / 8);
     if (chunks >= (int64_t(1) << 31) || H > 65535 || B > 65535) return mpsa_fail(MPSA_EUNSUPPORTED, "quantize: a head has too many elements, or too many heads");
     QuantArgs a;
-    a.x = x; a.sb = xs[0]; a.sh = xs[1]; a.sn = xs[2];
+    a.x = x; a.sub = sub; a.sb = xs[0]; a.sh = xs[1]; a.sn = xs[2];
     a.n = (int)N; a.d = (int)D; a.out_rows = (int)out_rows; a.pre = pre;
     a.emax4 = emax4; a.emax8 = emax8;
     a.codes4 = c4; a.scales4 = s4; a.codes8 = c8; a.scales8 = s8;
@@ -187,21 +271,52 @@ int quantize_common(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N,
 }  // namespace
 
 extern "C" int mpsa_quantize_mx(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
-                                const int64_t x_strides[4], float pre_scale, int fmt, int emax_elem,
+                                const int64_t x_strides[4], const void* sub, float pre_scale, int fmt, int emax_elem,
                                 uint8_t* codes, uint8_t* scales, int64_t out_rows, mpsa_stream_t stream) {
     if (fmt == MPSA_FMT_E2M1)
-        return quantize_common(x, x_dtype, B, H, N, D, x_strides, pre_scale, true, emax_elem, false, 0, 0,
+        return quantize_common(x, x_dtype, B, H, N, D, x_strides, sub, pre_scale, true, emax_elem, false, 0, 0,
                                codes, scales, nullptr, nullptr, out_rows, (hipStream_t)stream);
     if (fmt == MPSA_FMT_E4M3 || fmt == MPSA_FMT_E5M2)
-        return quantize_common(x, x_dtype, B, H, N, D, x_strides, pre_scale, false, 0, true, fmt, emax_elem,
+        return quantize_common(x, x_dtype, B, H, N, D, x_strides, sub, pre_scale, false, 0, true, fmt, emax_elem,
                                nullptr, nullptr, codes, scales, out_rows, (hipStream_t)stream);
     return mpsa_fail(MPSA_EINVAL, "quantize: unknown format %d", fmt);
 }
 
 extern "C" int mpsa_quantize_mx_dual(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
-                                     const int64_t x_strides[4], float pre_scale, int emax4, int fmt8, int emax8,
+                                     const int64_t x_strides[4], const void* sub, float pre_scale, int emax4, int fmt8, int emax8,
                                      uint8_t* codes4, uint8_t* scales4, uint8_t* codes8, uint8_t* scales8,
                                      int64_t out_rows, mpsa_stream_t stream) {
-    return quantize_common(x, x_dtype, B, H, N, D, x_strides, pre_scale, true, emax4, true, fmt8, emax8,
+    return quantize_common(x, x_dtype, B, H, N, D, x_strides, sub, pre_scale, true, emax4, true, fmt8, emax8,
                            codes4, scales4, codes8, scales8, out_rows, (hipStream_t)stream);
+}
+
+extern "C" int64_t mpsa_seq_mean_workspace(int64_t B, int64_t H, int64_t N, int64_t D) {
+    if (B < 0 || H < 0 || N < 0 || D < 0) return 0;
+    return B * H * ((N + MEAN_ROWS - 1) / MEAN_ROWS) * D * (int64_t)sizeof(float);
+}
+
+extern "C" int mpsa_seq_mean(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                             const int64_t x_strides[4], float* workspace, void* mean, mpsa_stream_t stream) {
+    if (!x || !x_strides || !workspace || !mean) return mpsa_fail(MPSA_EINVAL, "seq_mean: null pointer");
+    if (x_dtype != MPSA_BF16 && x_dtype != MPSA_F16) return mpsa_fail(MPSA_EINVAL, "seq_mean: x_dtype must be bf16 or f16");
+    if (B <= 0 || H <= 0 || N <= 0) return mpsa_fail(MPSA_EINVAL, "seq_mean: bad shape");
+    if (D != 64 && D != 128) return mpsa_fail(MPSA_EUNSUPPORTED, "seq_mean: D must be 64 or 128 (got %lld)", (long long)D);
+    if (x_strides[3] != 1) return mpsa_fail(MPSA_EINVAL, "seq_mean: last dim of x must be contiguous");
+    if (!mpsa_aligned16(x) || (x_strides[0] % 8) || (x_strides[1] % 8) || (x_strides[2] % 8)) return mpsa_fail(MPSA_EALIGN, "seq_mean: x rows must be 16-byte aligned");
+    if (H > 65535 || B > 65535 || N >= (int64_t(1) << 31)) return mpsa_fail(MPSA_EUNSUPPORTED, "seq_mean: shape too large");
+    MeanArgs a;
+    a.x = x; a.sb = x_strides[0]; a.sh = x_strides[1]; a.sn = x_strides[2];
+    a.n = (int)N; a.d = (int)D; a.nchunk = (int)((N + MEAN_ROWS - 1) / MEAN_ROWS);
+    a.partial = workspace; a.mean = mean; a.inv_n = 1.0f / (float)N;
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid((unsigned)a.nchunk, (unsigned)H, (unsigned)B);
+    if (x_dtype == MPSA_BF16) {
+        hipLaunchKernelGGL(seq_mean_kernel<MPSA_BF16>, grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(seq_mean_finish_kernel<MPSA_BF16>, dim3((unsigned)(B * H)), dim3(128), 0, st, a);
+    } else {
+        hipLaunchKernelGGL(seq_mean_kernel<MPSA_F16>, grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(seq_mean_finish_kernel<MPSA_F16>, dim3((unsigned)(B * H)), dim3(128), 0, st, a);
+    }
+    MPSA_CHECK_LAUNCH("seq_mean");
+    return MPSA_OK;
 }

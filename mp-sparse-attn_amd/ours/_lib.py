@@ -27,8 +27,10 @@ SIGNATURES = {
     "mpsa_e2m1_decode": (_int, [_vp, _i64, _vp, _vp]),
     "mpsa_e8m0_encode": (_int, [_vp, _i64, _vp, _vp]),
     "mpsa_e8m0_decode": (_int, [_vp, _i64, _vp, _vp]),
-    "mpsa_quantize_mx": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _f32, _int, _int, _vp, _vp, _i64, _vp]),
-    "mpsa_quantize_mx_dual": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _f32, _int, _int, _int,
+    "mpsa_quantize_mx": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _vp, _f32, _int, _int, _vp, _vp, _i64, _vp]),
+    "mpsa_seq_mean_workspace": (_i64, [_i64, _i64, _i64, _i64]),
+    "mpsa_seq_mean": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _vp, _vp, _vp]),
+    "mpsa_quantize_mx_dual": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _vp, _f32, _int, _int, _int,
                                      _vp, _vp, _vp, _vp, _i64, _vp]),
     "mpsa_gemm_mx": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
     "mpsa_v_tiles": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _int, _vp, _vp]),

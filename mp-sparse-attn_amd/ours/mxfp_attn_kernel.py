@@ -9,14 +9,14 @@ Pipeline per call (all on torch's current stream, no host synchronisation):
 import torch
 
 from . import _lib
-from .quant_mxint8 import quantize_mx, quantize_mx_dual, pre_scale_q, _as_bhnd
+from .quant_mxint8 import quantize_mx, quantize_mx_dual, seq_mean, pre_scale_q, _as_bhnd
 
 _MODES = {"mxfp4": _lib.MODE_MXFP4, "mxfp8": _lib.MODE_MXFP8, "mxfp8e5": _lib.MODE_MXFP8, "diag": _lib.MODE_DIAG,
           "diag_e5": _lib.MODE_DIAG}
 
 
-def prepare_operands(q, k, v, tile, block_scale_type, scale=None):
-    """Quantize Q/K and repack V for one attention call.  q ``[B,Hq,N,D]``, k/v ``[B,Hkv,N,D]`` of one
+def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False):
+    """Quantize Q/K (K minus its mean over the sequence if ``smooth_k``) and repack V for one attention call.  q ``[B,Hq,N,D]``, k/v ``[B,Hkv,N,D]`` of one
     16-bit dtype.  Returns a dict of device tensors (rows padded to whole tiles) the launcher consumes."""
     if block_scale_type not in _MODES:
         raise ValueError(f"Invalid block scale type: {block_scale_type}")
@@ -29,15 +29,17 @@ def prepare_operands(q, k, v, tile, block_scale_type, scale=None):
     pre = pre_scale_q(D, scale)
     ops = {"mode": mode, "fmt8": fmt8, "tile": tile, "n": N, "q4": None, "qs4": None, "q8": None, "qs8": None,
            "k4": None, "ks4": None, "k8": None, "ks8": None}
+    # smooth-K (ours/mxfp_attn_kernel.py:33-34): the mean over the sequence is subtracted inside the K quantizer
+    kmean = seq_mean(k) if smooth_k else None
     if mode == _lib.MODE_DIAG:
         ops["q4"], ops["qs4"], ops["q8"], ops["qs8"] = quantize_mx_dual(q, pre, fmt8, n_pad)
-        ops["k4"], ops["ks4"], ops["k8"], ops["ks8"] = quantize_mx_dual(k, 1.0, fmt8, n_pad)
+        ops["k4"], ops["ks4"], ops["k8"], ops["ks8"] = quantize_mx_dual(k, 1.0, fmt8, n_pad, sub=kmean)
     elif mode == _lib.MODE_MXFP4:
         ops["q4"], ops["qs4"] = quantize_mx(q, pre, _lib.FMT_E2M1, out_rows=n_pad)
-        ops["k4"], ops["ks4"] = quantize_mx(k, 1.0, _lib.FMT_E2M1, out_rows=n_pad)
+        ops["k4"], ops["ks4"] = quantize_mx(k, 1.0, _lib.FMT_E2M1, out_rows=n_pad, sub=kmean)
     else:
         ops["q8"], ops["qs8"] = quantize_mx(q, pre, fmt8, out_rows=n_pad)
-        ops["k8"], ops["ks8"] = quantize_mx(k, 1.0, fmt8, out_rows=n_pad)
+        ops["k8"], ops["ks8"] = quantize_mx(k, 1.0, fmt8, out_rows=n_pad, sub=kmean)
     v_tiles = torch.empty((B, Hkv, nt, tile * D), dtype=v.dtype, device=v.device)
     with torch.cuda.device(v.device):
         _lib.check(_lib.lib().mpsa_v_tiles(_lib.ptr(v), _lib.dtype_id(v.dtype), B, Hkv, N, D, _lib.strides4(v), tile,
@@ -92,8 +94,6 @@ def mxfp_attn_kernel(q, k, v, attn_mask=None, dropout_p=0.0,
     torch.cuda.set_device(v.device)
     q, k, v = _normalise(q, k, v)
     q, k, v = _as_bhnd(q, tensor_layout), _as_bhnd(k, tensor_layout), _as_bhnd(v, tensor_layout)
-    if smooth_k:
-        k = k - k.mean(dim=-2, keepdim=True)                        # ours/mxfp_attn_kernel.py:33-34
     B, Hq, N, D = q.shape
     assert D in [64, 128], "headdim should be in [64, 128]."
     assert k.shape[2] == N and v.shape[2] == N, "q, k and v must have the same sequence length"
@@ -103,7 +103,7 @@ def mxfp_attn_kernel(q, k, v, attn_mask=None, dropout_p=0.0,
         raise ValueError(f"Unsupported dtype: {output_dtype}")       # ours/mxfp_attn_kernel.py:389
     if v.stride(-1) != 1:
         v = v.contiguous()
-    ops = prepare_operands(q, k, v, tile, block_scale_type, scale)
+    ops = prepare_operands(q, k, v, tile, block_scale_type, scale, smooth_k=smooth_k)
     if tensor_layout == "HND":
         out = torch.empty((B, Hq, N, D), dtype=output_dtype, device=q.device)
         attention_from_operands(ops, out, is_causal)

@@ -50,10 +50,34 @@ def pre_scale_q(head_dim, sm_scale=None):
     return float(torch.tensor(sm_scale * LOG2E, dtype=torch.float32).item())
 
 
-def quantize_mx(x, pre_scale, fmt, emax_elem=None, out_rows=None):
+def seq_mean(x):
+    """``x.mean(dim=-2)`` of a ``[B,H,L,D]`` bf16/fp16 tensor -> ``[B,H,D]`` in x's dtype, through ``mpsa_seq_mean``
+    (float32 sum in a fixed order, times float32 ``1/L``, rounded once).  The mean the smooth-K prologue subtracts
+    (ours/mxfp_attn.py:44-45); pass it as ``sub`` to the quantizers."""
+    x = _check_input(x)
+    B, H, L, D = x.shape
+    mean = torch.empty((B, H, D), dtype=x.dtype, device=x.device)
+    nbytes = _lib.lib().mpsa_seq_mean_workspace(B, H, L, D)
+    work = torch.empty((max(nbytes // 4, 1),), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().mpsa_seq_mean(_lib.ptr(x), _lib.dtype_id(x.dtype), B, H, L, D, _lib.strides4(x),
+                                            _lib.ptr(work), _lib.ptr(mean), _lib.stream_ptr(x.device)))
+    return mean
+
+
+def _sub_ptr(sub, x):
+    if sub is None:
+        return None
+    B, H, _, D = x.shape
+    assert sub.shape == (B, H, D) and sub.dtype == x.dtype and sub.device == x.device, "sub must be [B,H,D] of x's dtype"
+    return _lib.ptr(sub.contiguous())
+
+
+def quantize_mx(x, pre_scale, fmt, emax_elem=None, out_rows=None, sub=None):
     """One tensor ``[B,H,L,D]`` -> (codes, scales) through ``mpsa_quantize_mx``.
 
-    ``out_rows`` >= L pads every head with zero rows (the attention kernel wants whole tiles)."""
+    ``out_rows`` >= L pads every head with zero rows (the attention kernel wants whole tiles).
+    ``sub`` (``[B,H,D]``, x's dtype): quantize ``x - sub[:, :, None]`` (difference rounded to x's dtype)."""
     x = _check_input(x)
     B, H, L, D = x.shape
     rows = L if out_rows is None else int(out_rows)
@@ -64,13 +88,14 @@ def quantize_mx(x, pre_scale, fmt, emax_elem=None, out_rows=None):
     scales = torch.empty((B, H, rows, D // 32), dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
         _lib.check(_lib.lib().mpsa_quantize_mx(
-            _lib.ptr(x), _lib.dtype_id(x.dtype), B, H, L, D, _lib.strides4(x), pre_scale, fmt, emax_elem,
+            _lib.ptr(x), _lib.dtype_id(x.dtype), B, H, L, D, _lib.strides4(x), _sub_ptr(sub, x), pre_scale, fmt, emax_elem,
             _lib.ptr(codes), _lib.ptr(scales), rows, _lib.stream_ptr(x.device)))
     return codes, scales
 
 
-def quantize_mx_dual(x, pre_scale, fmt8=_lib.FMT_E4M3, out_rows=None):
-    """E2M1 and an 8-bit format in one pass over x -> (codes4, scales4, codes8, scales8)."""
+def quantize_mx_dual(x, pre_scale, fmt8=_lib.FMT_E4M3, out_rows=None, sub=None):
+    """E2M1 and an 8-bit format in one pass over x -> (codes4, scales4, codes8, scales8).  ``sub`` as in
+    :func:`quantize_mx`."""
     x = _check_input(x)
     B, H, L, D = x.shape
     rows = L if out_rows is None else int(out_rows)
@@ -81,7 +106,7 @@ def quantize_mx_dual(x, pre_scale, fmt8=_lib.FMT_E4M3, out_rows=None):
     s8 = torch.empty((B, H, rows, D // 32), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().mpsa_quantize_mx_dual(
-            _lib.ptr(x), _lib.dtype_id(x.dtype), B, H, L, D, _lib.strides4(x), pre_scale,
+            _lib.ptr(x), _lib.dtype_id(x.dtype), B, H, L, D, _lib.strides4(x), _sub_ptr(sub, x), pre_scale,
             EMAX_E2M1, fmt8, EMAX_8BIT, _lib.ptr(c4), _lib.ptr(s4), _lib.ptr(c8), _lib.ptr(s8), rows,
             _lib.stream_ptr(dev)))
     return c4, s4, c8, s8

@@ -37,7 +37,7 @@ from .mx_formats import (  # noqa: F401
     encode_e8m0, decode_e8m0, encode_e4m3, decode_e4m3, encode_e5m2, decode_e5m2,
 )
 from .mx_quantize import (  # noqa: F401
-    FMT_E2M1, FMT_E4M3, FMT_E5M2, EMAX_ELEM, q_pre_scale, quantize_mx, dequantize_mx, smooth_k,
+    FMT_E2M1, FMT_E4M3, FMT_E5M2, EMAX_ELEM, q_pre_scale, quantize_mx, dequantize_mx, smooth_k, seq_mean,
 )
 from .mx_gemm import gemm_mx  # noqa: F401
 from .mx_attention import attn_mx, attn_dense_f64, precision_metric, v_fragment_order  # noqa: F401

@@ -45,13 +45,14 @@ def _prepare(q, k, mode, scale, fmt8):
 
 
 def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=False,
-            fmt8=FMT_E4M3, out_dtype=None, heads=None) -> torch.Tensor:
+            fmt8=FMT_E4M3, out_dtype=None, heads=None, q_tiles=None) -> torch.Tensor:
     """Tile-by-tile MXFP attention.  q ``[B,Hq,N,D]``, k/v ``[B,Hkv,N,D]`` in bf16 or fp16.
 
     P is rounded to v's dtype before P.V and the product of a tile is accumulated in float32
     (ours/mxfp_attn_kernel.py:339-340).  ``heads`` restricts the computation to a list of query
     heads (the output then has ``len(heads)`` heads).  N need not be a multiple of ``tile``:
-    the last key tile is cut at N."""
+    the last key tile is cut at N.  ``q_tiles`` restricts the computation to a list of query tiles (all
+    keys are still visited); the output then holds only those tiles' rows, concatenated in list order."""
     B, Hq, N, D = q.shape
     Hkv = k.shape[1]
     assert Hq % Hkv == 0
@@ -65,11 +66,16 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
     ops = _prepare(q[:, head_list], k, mode, scale, fmt8)
     vf = v.to(torch.float32)
     nt = (N + tile - 1) // tile
-    out = torch.empty((B, len(head_list), N, D), dtype=out_dtype)
+    tile_list = list(range(nt)) if q_tiles is None else list(q_tiles)
+    starts, n_out = {}, 0
+    for i in tile_list:
+        starts[i] = n_out
+        n_out += min((i + 1) * tile, N) - i * tile
+    out = torch.empty((B, len(head_list), n_out, D), dtype=out_dtype)
     for b in range(B):
         for hi_, h in enumerate(head_list):
             kvh = h // group
-            for i in range(nt):
+            for i in tile_list:
                 r0, r1 = i * tile, min((i + 1) * tile, N)
                 rows = r1 - r0
                 m = torch.full((rows,), float("-inf"))
@@ -93,7 +99,7 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
                     pv = p.to(lp).to(torch.float32) @ vf[b, kvh, c0:c1]
                     acc = acc * alpha.unsqueeze(1) + pv
                     m = m_new
-                out[b, hi_, r0:r1] = (acc / l.unsqueeze(1)).to(out_dtype)
+                out[b, hi_, starts[i]:starts[i] + rows] = (acc / l.unsqueeze(1)).to(out_dtype)
     return out
 
 

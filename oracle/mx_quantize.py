@@ -92,6 +92,21 @@ def dequantize_mx(codes: torch.Tensor, scales: torch.Tensor, fmt: int, dtype=tor
     return val.to(dtype) * s
 
 
-def smooth_k(k: torch.Tensor) -> torch.Tensor:
-    """``k - mean over the sequence dim`` in k's own dtype.  ours/mxfp_attn.py:44-45."""
-    return k - k.mean(dim=-2, keepdim=True)
+def seq_mean(k: torch.Tensor) -> torch.Tensor:
+    """Mean over the sequence dim in k's 16-bit dtype the way the reference's device computes it: float32
+    accumulation, times float32 ``1/N``, one rounding (torch's CUDA mean; its CPU mean for 16-bit inputs rounds
+    the sum to 16 bits first, which is not what the reference ran).  ours/mxfp_attn.py:44-45."""
+    n = k.shape[-2]
+    inv = torch.tensor(1.0, dtype=torch.float32) / torch.tensor(float(n), dtype=torch.float32)
+    return (k.to(torch.float32).sum(dim=-2, keepdim=True) * inv).to(k.dtype)
+
+
+def smooth_k(k: torch.Tensor, mean: torch.Tensor = None) -> torch.Tensor:
+    """``k - mean over the sequence dim`` in k's own dtype.  ours/mxfp_attn.py:44-45.  ``mean`` (``[..., 1, D]``
+    or ``[..., D]``, k's dtype) replaces the oracle's own mean, for checking the subtraction apart from the
+    summation order of the mean."""
+    if mean is None:
+        mean = seq_mean(k)
+    elif mean.dim() == k.dim() - 1:
+        mean = mean.unsqueeze(-2)
+    return k - mean.to(k.dtype)

@@ -32,14 +32,18 @@ def test_host_side_argument_validation():
     null = ctypes.c_void_p(0)
     one = ctypes.c_void_p(16)           # never dereferenced: validation fails first
     st = (ctypes.c_int64 * 4)(1, 1, 32, 1)
-    assert L.mpsa_quantize_mx(null, 0, 1, 1, 1, 32, st, 1.0, 4, 3, one, one, 1, null) == -1
+    assert L.mpsa_quantize_mx(null, 0, 1, 1, 1, 32, st, null, 1.0, 4, 3, one, one, 1, null) == -1
     assert b"null" in L.mpsa_last_error()
     st_ok = (ctypes.c_int64 * 4)(64, 64, 64, 1)
-    assert L.mpsa_quantize_mx(one, 0, 1, 1, 1, 48, st_ok, 1.0, 4, 3, one, one, 1, null) == -1      # D % 32
-    assert L.mpsa_quantize_mx(one, 2, 1, 1, 1, 64, st_ok, 1.0, 4, 3, one, one, 1, null) == -1      # f32 input
-    assert L.mpsa_quantize_mx(one, 0, 1, 1, 1, 64, st_ok, 1.0, 9, 3, one, one, 1, null) == -1      # bad format
-    assert L.mpsa_quantize_mx(one, 0, 1, 1, 2, 64, st_ok, 1.0, 4, 3, one, one, 1, null) == -1      # out_rows < N
-    assert L.mpsa_quantize_mx(ctypes.c_void_p(24), 0, 1, 1, 1, 64, st_ok, 1.0, 4, 3, one, one, 1, null) == -2
+    assert L.mpsa_quantize_mx(one, 0, 1, 1, 1, 48, st_ok, null, 1.0, 4, 3, one, one, 1, null) == -1      # D % 32
+    assert L.mpsa_quantize_mx(one, 2, 1, 1, 1, 64, st_ok, null, 1.0, 4, 3, one, one, 1, null) == -1      # f32 input
+    assert L.mpsa_quantize_mx(one, 0, 1, 1, 1, 64, st_ok, null, 1.0, 9, 3, one, one, 1, null) == -1      # bad format
+    assert L.mpsa_quantize_mx(one, 0, 1, 1, 2, 64, st_ok, null, 1.0, 4, 3, one, one, 1, null) == -1      # out_rows < N
+    assert L.mpsa_quantize_mx(ctypes.c_void_p(24), 0, 1, 1, 1, 64, st_ok, null, 1.0, 4, 3, one, one, 1, null) == -2
+    assert L.mpsa_quantize_mx(one, 0, 1, 1, 1, 64, st_ok, ctypes.c_void_p(8), 1.0, 4, 3, one, one, 1, null) == -2   # sub alignment
+    assert L.mpsa_seq_mean_workspace(2, 3, 1000, 64) == 2 * 3 * 4 * 64 * 4
+    assert L.mpsa_seq_mean(one, 0, 1, 1, 8, 64, st_ok, null, one, null) == -1                      # no workspace
+    assert L.mpsa_seq_mean(one, 0, 1, 1, 8, 96, st_ok, one, one, null) == -3                       # D = 96
     assert L.mpsa_gemm_mx(one, one, one, one, 4, 100, 256, 128, one, 0, 256, null) == -3           # M % 256
     assert L.mpsa_gemm_mx(one, one, one, one, 4, 256, 256, 128, one, 7, 256, null) == -1           # bad dtype
     assert L.mpsa_v_tiles(one, 0, 1, 1, 128, 96, st_ok, 128, one, null) == -3                      # D = 96

@@ -93,6 +93,30 @@ def test_ragged_length_tail_masking(causal):
     _compare(got, want, f"ragged causal={causal}")
 
 
+def test_c5_dit_shape_non_causal_ragged():
+    """The video-DiT shape: N = 32760 = 255*128 + 120 keys/queries, D = 128, non-causal, sigma 0.5 draws plus a
+    per-frame offset (21 frames of 1560 tokens) on q and k.  Two heads run on the GPU at full length (the
+    40-head problem is the same kernel 20 times over); the oracle checks 512 query rows spread over the
+    sequence, among them the ragged tail, against all 32760 keys."""
+    N, D, frames = 32760, 128, 21
+    g = torch.Generator().manual_seed(4)
+    q = 0.5 * torch.randn(1, 2, N, D, generator=g)
+    k = 0.5 * torch.randn(1, 2, N, D, generator=g)
+    v = 0.5 * torch.randn(1, 2, N, D, generator=g)
+    off = 0.5 * torch.randn(frames, 1, D, generator=g)
+    q = (q.view(1, 2, frames, N // frames, D) + off).view(1, 2, N, D).bfloat16()
+    k = (k.view(1, 2, frames, N // frames, D) + off).view(1, 2, N, D).bfloat16()
+    v = v.bfloat16()
+    got = _run(q, k, v, is_causal=False, block_scale_type="diag", tile=128, output_dtype=torch.bfloat16)
+    assert got.shape == (1, 2, N, D) and torch.isfinite(got.float()).all()
+    # query tiles 0, 100, 200 and the ragged last one (255), 128 rows each: the oracle on those queries only
+    tiles = [0, 100, 200, 255]
+    want = O.attn_mx(q, k, v, tile=128, causal=False, mode="diag", q_tiles=tiles)
+    rows = torch.cat([torch.arange(t * 128, min((t + 1) * 128, N)) for t in tiles])
+    assert want.shape[2] == rows.numel() == 3 * 128 + 120
+    _compare(got[:, :, rows.to(got.device)], want, "C5 query tiles 0, 100, 200, 255")
+
+
 def test_fp16_inputs_nhd_layout_scale_and_public_entry():
     q, k, v = make_qkv(1, 4, 2, 256, 64, seed=44, dtype=torch.float16)
     want = O.attn_mx(q, k, v, tile=128, causal=True, mode="mxfp4", scale=0.2, out_dtype=torch.float16)

@@ -5,7 +5,7 @@ import torch
 import oracle as O
 from conftest import make_qkv
 from ours import _lib
-from ours.quant_mxint8 import quantize_mx, quantize_mx_dual, quant_mxfp4, quant_mxfp8, quant_mxfp8e5, pre_scale_q
+from ours.quant_mxint8 import seq_mean, quantize_mx, quantize_mx_dual, quant_mxfp4, quant_mxfp8, quant_mxfp8e5, pre_scale_q
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"

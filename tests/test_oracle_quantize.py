@@ -106,3 +106,27 @@ def test_smooth_k():
     s = O.smooth_k(k)
     assert s.dtype == torch.bfloat16
     assert s.float().mean(dim=-2).abs().max() < 0.05
+
+
+def test_seq_mean_is_the_once_rounded_mean():
+    """The mean is the float32 sum times float32 1/N rounded once to the 16-bit dtype: checked against float64
+    arithmetic (the two can only differ where the float64 mean sits within float32 error of a rounding
+    boundary), against an exactly representable case, and the subtraction against explicit bf16 arithmetic."""
+    g = torch.Generator().manual_seed(5)
+    for dtype in (torch.bfloat16, torch.float16):
+        k = (torch.randn(2, 3, 1000, 64, generator=g) * 2 + 1).to(dtype)
+        m = O.seq_mean(k)
+        assert m.dtype == dtype and m.shape == (2, 3, 1, 64)
+        ref = k.double().mean(dim=-2, keepdim=True)
+        ulp = torch.finfo(dtype).eps * ref.abs().clamp_min(2.0 ** -14)
+        assert ((m.double() - ref).abs() <= 0.5 * ulp * (1 + 1e-3)).all()
+        assert (m == ref.to(dtype)).float().mean() > 0.995
+    k = torch.tensor([1.0, 2.0, 3.0, 6.0]).view(1, 1, 4, 1).expand(1, 1, 4, 32).bfloat16()
+    assert (O.seq_mean(k) == 3.0).all()
+    s = O.smooth_k(k)
+    assert torch.equal(s[0, 0, :, 0].float(), torch.tensor([-2.0, -1.0, 0.0, 3.0]))
+    # explicit mean argument: the difference is rounded to the 16-bit dtype
+    k2 = torch.tensor([1.0078125, 100.0]).view(1, 1, 2, 1).expand(1, 1, 2, 32).bfloat16()
+    mean = torch.full((1, 1, 32), 0.00390625).bfloat16()
+    d = O.smooth_k(k2, mean)
+    assert d[0, 0, 0, 0].item() == 1.0 and d[0, 0, 1, 0].item() == 100.0     # 1.00390625 and 99.996 round to bf16
