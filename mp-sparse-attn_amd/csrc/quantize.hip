@@ -83,6 +83,41 @@ __device__ __forceinline__ float round16(float v) {
     }
 }
 
+// Eight E2M1 codes (one packed word, element i in nibble i) of x[0..7] / 2^se.
+// Fast path: v_cvt_scalef32_pk_fp4_f32 divides by the power of two and rounds to nearest, ties to even.  The
+// reference's rule (argmin of float32 distances with 1e-6 taken off the even-mantissa candidate, e2m1_index in
+// mx_codec.h) differs from that only for a value within about 1e-6 of the midpoint between two E2M1 values.  Such
+// a value is found by converting the inputs nudged down and up by 2^-17 of themselves: if the two conversions
+// differ anywhere in the word, the lane falls back to the explicit rule.  (2^-17 of a value near a midpoint - the
+// smallest is 0.25 - is at least 1.9e-6.)  Scales too small for a normal float32 take the explicit rule as well.
+template <bool HW4>
+__device__ __forceinline__ uint32_t e2m1_pack8(const float (&x)[8], int se) {
+    if constexpr (HW4) {
+        if (se >= -126) {
+            const float sc = mpsa_u2f((uint32_t)(se + 127) << 23);
+            const float dn = 1.0f - 0x1p-17f, up = 1.0f + 0x1p-17f;
+            uint32_t w = 0, wd = 0, wu = 0;
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[0], x[1], sc, 0);
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[2], x[3], sc, 1);
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[4], x[5], sc, 2);
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[6], x[7], sc, 3);
+            wd = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wd, x[0] * dn, x[1] * dn, sc, 0);
+            wd = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wd, x[2] * dn, x[3] * dn, sc, 1);
+            wd = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wd, x[4] * dn, x[5] * dn, sc, 2);
+            wd = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wd, x[6] * dn, x[7] * dn, sc, 3);
+            wu = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wu, x[0] * up, x[1] * up, sc, 0);
+            wu = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wu, x[2] * up, x[3] * up, sc, 1);
+            wu = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wu, x[4] * up, x[5] * up, sc, 2);
+            wu = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wu, x[6] * up, x[7] * up, sc, 3);
+            if (wd == wu) return w;
+        }
+    }
+    uint32_t word = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) word |= e2m1_encode(ldexpf(x[i], -se)) << (4 * i);
+    return word;
+}
+
 template <int XDT, bool DO4, bool DO8, int FMT8, bool SW8>
 __global__ __launch_bounds__(256) void quantize_kernel(QuantArgs a) {
     const uint32_t cpr = (uint32_t)a.d >> 3;                              // 16-byte chunks per row
@@ -127,11 +162,7 @@ __global__ __launch_bounds__(256) void quantize_kernel(QuantArgs a) {
 
     if constexpr (DO4) {
         const int se = e - a.emax4;
-        uint32_t word = 0;
-        if (!zero) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) word |= e2m1_encode(ldexpf(x[i], -se)) << (4 * i);
-        }
+        const uint32_t word = zero ? 0u : e2m1_pack8<!SW8>(x, se);
         reinterpret_cast<uint32_t*>(a.codes4)[oc] = word;
         const int sbyte = zero ? 0 : min(max(se + 127, 0), 254);
         if (quad_leader) a.scales4[oc >> 2] = (uint8_t)sbyte;
@@ -213,10 +244,13 @@ __global__ __launch_bounds__(128) void seq_mean_finish_kernel(MeanArgs a) {
     }
 }
 
+// MPSA_FP8_ENCODE=sw or MPSA_FP4_ENCODE=sw in the environment selects the kernels that encode with explicit
+// integer/float arithmetic only (no hardware conversion instructions), for cross-checking
 bool use_sw_fp8() {
     static const bool sw = [] {
         const char* v = getenv("MPSA_FP8_ENCODE");
-        return v && v[0] == 's';
+        const char* w = getenv("MPSA_FP4_ENCODE");
+        return (v && v[0] == 's') || (w && w[0] == 's');
     }();
     return sw;
 }

@@ -110,6 +110,74 @@ def test_reference_style_entry_points_and_layouts():
         quant_mxfp4(qd, kd, tensor_layout="DNH")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 8, 8192, 128), (2, 3, 1000, 64), (1, 2, 32760, 128), (1, 1, 7, 64)])
+def test_smooth_k_mean_and_fused_subtraction(shape, dtype):
+    """mpsa_seq_mean against the oracle's once-rounded mean (summation order may move the 16-bit result by one
+    unit in the last place on rare channels: at most 1 ulp anywhere, equal on more than 99 %), and the
+    quantizer's fused ``x - mean`` bit for bit against the oracle quantizing ``smooth_k(k, that mean)``."""
+    B, H, N, D = shape
+    g = torch.Generator().manual_seed(N + D)
+    k = (torch.randn(B, H, N, D, generator=g) + torch.randn(1, H, 1, D, generator=g) * 2).to(dtype)
+    got = seq_mean(k.to(DEV))
+    assert got.shape == (B, H, D) and got.dtype == dtype
+    want = O.seq_mean(k).squeeze(-2)
+    same = (got.cpu() == want)
+    assert same.float().mean().item() > 0.99
+    ulp = torch.finfo(dtype).eps * want.float().abs().clamp_min(2.0 ** -14)
+    assert ((got.cpu().float() - want.float()).abs() <= ulp).all()
+    smoothed = O.smooth_k(k, got.cpu())
+    for fmt in FMTS:
+        codes, scales = quantize_mx(k.to(DEV), 1.0, fmt, sub=got)
+        want_c, want_s = O.quantize_mx(smoothed, 1.0, fmt)
+        assert torch.equal(scales.cpu(), want_s) and torch.equal(codes.cpu(), want_c), f"fmt {fmt}"
+    c4, s4, c8, s8 = quantize_mx_dual(k.to(DEV), 1.0, O.FMT_E4M3, out_rows=N + 9, sub=got)
+    w4, ws4 = O.quantize_mx(smoothed, 1.0, O.FMT_E2M1)
+    w8, ws8 = O.quantize_mx(smoothed, 1.0, O.FMT_E4M3)
+    assert torch.equal(c4[:, :, :N].cpu(), w4) and torch.equal(s4[:, :, :N].cpu(), ws4)
+    assert torch.equal(c8[:, :, :N].cpu(), w8) and torch.equal(s8[:, :, :N].cpu(), ws8)
+    assert not c4[:, :, N:].any() and not c8[:, :, N:].any() and not s4[:, :, N:].any()
+
+
+def test_hardware_e2m1_conversion_agrees_with_the_explicit_rule_near_every_midpoint():
+    """The quantizer's fast path (hardware FP4 conversion) must hand every value near a rounding boundary to
+    the explicit rule: float32-dense sweeps around each of the seven midpoints, reached through a pre-scale
+    that makes the scaled values arbitrary float32 numbers, and blocks whose scale is not a normal float32."""
+    mids = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0])
+    rows = []
+    for m in mids.tolist():
+        base = torch.tensor(m, dtype=torch.float32)
+        steps = torch.arange(-24, 25, dtype=torch.float32)
+        vals = base + steps * 1.25e-7 * max(m, 1.0)            # a few float32 ulps either side, +-3e-6
+        for chunk in vals.split(31):
+            blk = torch.full((32,), 0.0)
+            blk[0] = 6.0                                        # pins the shared exponent: scale 2^(2-3)... = 0.5
+            blk[1:1 + chunk.numel()] = chunk
+            rows.append(blk)
+            rows.append(-blk)
+    x = torch.stack(rows)                                       # [R, 32] float32 targets of x*pre / 2^se with se = -1
+    # choose bf16 inputs and a pre-scale so that f32(x)*pre lands on arbitrary float32 values near the targets
+    pre = 0.7310585975646973
+    xin = (x * 0.5 / pre).bfloat16().view(1, 1, -1, 32)
+    xin = torch.cat([xin, (xin.float() * 2.0 ** -120).bfloat16()], dim=2)       # tiny blocks: scale below 2^-126
+    for p in (pre, 1.0, 0.9999998807907104, 1.0000001192092896):
+        codes, scales = quantize_mx(xin.to(DEV), p, O.FMT_E2M1)
+        want_c, want_s = O.quantize_mx(xin, p, O.FMT_E2M1)
+        assert torch.equal(scales.cpu(), want_s) and torch.equal(codes.cpu(), want_c), f"pre {p}"
+    # a dense float32 sweep through the pre-scale instead of the input: the scaled value walks across each midpoint
+    one = torch.zeros(1, 1, 1, 32); one[..., 0] = 6.0
+    for m in mids.tolist():
+        xb = one.clone(); xb[..., 1:] = m
+        xb = xb.bfloat16()
+        for k in range(-40, 41):
+            p = float(torch.tensor(1.0 + k * 2.0 ** -23, dtype=torch.float32))
+            if (xb.float().abs().max() * p) >= 8.0:
+                continue
+            codes, scales = quantize_mx(xb.to(DEV), p, O.FMT_E2M1)
+            want_c, want_s = O.quantize_mx(xb, p, O.FMT_E2M1)
+            assert torch.equal(codes.cpu(), want_c) and torch.equal(scales.cpu(), want_s), f"mid {m} pre {p}"
+
+
 @pytest.mark.parametrize("fmt", [O.FMT_E2M1, O.FMT_E4M3])
 def test_c2_gemm_operand_full_size(fmt):
     """The 8192 x 8192 GEMM operand of the standalone config, quantized along K: every byte against the oracle."""
