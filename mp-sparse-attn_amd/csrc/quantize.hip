@@ -16,6 +16,7 @@
 // own one MX block, so the block maximum is two DPP quad exchanges.  The kernel is HBM-bound:
 // 2 B/element in, 0.5 (+1) B/element of codes and 1/32 (x2) B/element of scales out.
 #include "mpsa_common.h"
+#include <cstring>
 #include "mx_codec.h"
 
 namespace {
@@ -27,6 +28,7 @@ struct QuantArgs {
     int n, d;                  // valid rows, row length
     int out_rows;              // rows per (b,h) in the outputs
     float pre;
+    int exact16;               // pre is a power of two: scaled values keep the inputs' 16-bit significands
     int emax4, emax8;
     uint8_t *codes4, *scales4, *codes8, *scales8;
 };
@@ -90,8 +92,12 @@ __device__ __forceinline__ float round16(float v) {
 // a value is found by converting the inputs nudged down and up by 2^-17 of themselves: if the two conversions
 // differ anywhere in the word, the lane falls back to the explicit rule.  (2^-17 of a value near a midpoint - the
 // smallest is 0.25 - is at least 1.9e-6.)  Scales too small for a normal float32 take the explicit rule as well.
+// When the pre-scale is a power of two the scaled values are 16-bit inputs times a power of two, at most 11
+// significant bits: such a value is either exactly a midpoint - where the two rules agree (both take the even
+// mantissa) - or at least 2^-12 away from one, so the check is skipped (`exact16`); it would otherwise fire on every
+// exact tie, which 16-bit data hits all the time.
 template <bool HW4>
-__device__ __forceinline__ uint32_t e2m1_pack8(const float (&x)[8], int se) {
+__device__ __forceinline__ uint32_t e2m1_pack8(const float (&x)[8], int se, bool exact16) {
     if constexpr (HW4) {
         if (se >= -126) {
             const float sc = mpsa_u2f((uint32_t)(se + 127) << 23);
@@ -101,6 +107,7 @@ __device__ __forceinline__ uint32_t e2m1_pack8(const float (&x)[8], int se) {
             w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[2], x[3], sc, 1);
             w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[4], x[5], sc, 2);
             w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[6], x[7], sc, 3);
+            if (exact16) return w;
             wd = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wd, x[0] * dn, x[1] * dn, sc, 0);
             wd = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wd, x[2] * dn, x[3] * dn, sc, 1);
             wd = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wd, x[4] * dn, x[5] * dn, sc, 2);
@@ -162,7 +169,7 @@ __global__ __launch_bounds__(256) void quantize_kernel(QuantArgs a) {
 
     if constexpr (DO4) {
         const int se = e - a.emax4;
-        const uint32_t word = zero ? 0u : e2m1_pack8<!SW8>(x, se);
+        const uint32_t word = zero ? 0u : e2m1_pack8<!SW8>(x, se, a.exact16 != 0);
         reinterpret_cast<uint32_t*>(a.codes4)[oc] = word;
         const int sbyte = zero ? 0 : min(max(se + 127, 0), 254);
         if (quad_leader) a.scales4[oc >> 2] = (uint8_t)sbyte;
@@ -286,6 +293,11 @@ int quantize_common(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N,
     QuantArgs a;
     a.x = x; a.sub = sub; a.sb = xs[0]; a.sh = xs[1]; a.sn = xs[2];
     a.n = (int)N; a.d = (int)D; a.out_rows = (int)out_rows; a.pre = pre;
+    {
+        uint32_t pb;
+        memcpy(&pb, &pre, 4);
+        a.exact16 = ((pb & 0x007FFFFFu) == 0u && (pb & 0x7F800000u) != 0u && (pb & 0x7F800000u) != 0x7F800000u) ? 1 : 0;
+    }
     a.emax4 = emax4; a.emax8 = emax8;
     a.codes4 = c4; a.scales4 = s4; a.codes8 = c8; a.scales8 = s8;
     dim3 grid((unsigned)((chunks + 255) / 256), (unsigned)H, (unsigned)B);
