@@ -154,6 +154,23 @@ int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, cons
                   int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
                   mpsa_stream_t stream);
 
+/*
+ * Fused attention forward with the reference's tile-skipping rule (the skip_thresh argument of mxfp_attn /
+ * mxfp_attn_kernel, ours/mxfp_attn.py:32, ours/mxfp_attn_kernel.py:272-297, with the key/value pointers advancing
+ * past a skipped tile, which the reference's loop forgets): for query tile i, the statistic of key tile j is the mean
+ * over the tile's valid query rows of the row maximum of S (after masking); tile 0 is always kept and sets the
+ * reference value; tile j > 0 is kept iff stat(j) >= stat(0) * skip_thresh; a skipped tile contributes nothing.
+ * Arguments as mpsa_attn_fwd, mode MPSA_MODE_MXFP4 or MPSA_MODE_MXFP8 only (the rule's reference tile must be the
+ * first one visited), plus
+ *   skip_thresh   the factor above (scores are in log2 units with sm_scale folded in, as in the reference)
+ *   skipped       NULL, or int32 [B,Hq,ceil(n/tile)]: number of key tiles skipped for each query tile
+ */
+int mpsa_attn_fwd_skip(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
+                       const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
+                       const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
+                       int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                       float skip_thresh, int32_t* skipped, mpsa_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -11,6 +11,8 @@ struct AttnArgs {
     int B, Hq, Hkv, n, n_pad, nt;
     int causal, mode, fmt8, o_dtype;
     int d, tile;
+    float skip_thresh;         // tile-skipping variants only
+    int32_t* skipped;          // optional [B,Hq,nt] count of skipped key tiles per query tile
 };
 
 template <int PVT> struct PV;
@@ -69,6 +71,9 @@ __device__ __forceinline__ void load16_to_lds(const uint8_t* gsrc, uint8_t* lds_
                                      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
+
+// Tile-skipping variants of the general kernel (modes mxfp4 / mxfp8): attn_fwd_skip.hip
+int attn_skip_launch(const AttnArgs& a, int pv_dtype, hipStream_t st);
 
 // Paired-tile ("ping-pong") kernel for causal runs with D = 128, tile = 128 and whole tile pairs: attn_fwd_pp.hip
 bool attn_pp_supported(const AttnArgs& a, int pv_dtype);

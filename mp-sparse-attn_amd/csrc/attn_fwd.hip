@@ -30,382 +30,9 @@
 // reads its fragments from global memory one step ahead.  K scales are read from global memory one step ahead
 // as well.  80 KiB of LDS and at most 256 registers per workgroup let two workgroups share a CU, so one's matrix
 // instructions overlap the other's softmax VALU work.
-#include "attn_common.h"
+#include "attn_fwd_kernel.h"
 
 namespace {
-
-template <int D, int TILE>
-struct Geom {
-    static constexpr int NW = TILE / 32;          // waves per workgroup
-    static constexpr int NT = NW * 64;            // threads
-    static constexpr int KB = TILE / 32;          // 32-key blocks per tile
-    static constexpr int SST = D / 64;            // score matrix instructions along D
-    static constexpr int NDB = D / 32;            // 32-wide output dim blocks
-    static constexpr int ROW4 = D / 2, ROW8 = D;  // bytes per K row
-    static constexpr int CPR4 = ROW4 / 16;        // 16-byte chunks per 4-bit K row (2 | 4)
-    static constexpr int SH4 = CPR4 == 2 ? 3 : 2; // log2(rows per 256 bytes)
-    static constexpr int K_BYTES = TILE * ROW4;   // one 4-bit K tile
-    static constexpr int V_BYTES = TILE * D * 2;
-    static constexpr int SMEM = 2 * K_BYTES + 2 * V_BYTES;
-    static constexpr int KI4 = K_BYTES / 1024 / NW;                   // direct-load instructions per wave
-    static constexpr int VI = V_BYTES / 1024 / NW;
-    static constexpr int NV = KB * 2 * NDB;       // V fragments (= P.V matrix instructions) per tile
-};
-
-// MODE is compile-time: an all-4-bit run carries no 8-bit code, an all-8-bit run keeps the next tile's 8-bit K
-// fragments in registers (read from global memory one step ahead), and a "diag" run pipelines 4-bit tiles through
-// LDS and fetches its single 8-bit tile when it gets there.
-template <int D, int TILE, int PVT, int FMT8, int MODE>
-__global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
-    typedef Geom<D, TILE> G;
-    typedef PV<PVT> P;
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, w = tid >> 6;
-    const int h = lane >> 5, r = lane & 31;
-
-    // ---- which (batch, kv head, query head, query tile) -- XCD-aware, heavy causal tiles first ----
-    const int group = a.Hq / a.Hkv;
-    const int total = a.B * a.Hq * a.nt;
-    int L = blockIdx.x;
-    if ((total & 7) == 0) L = (L & 7) * (total >> 3) + (L >> 3);      // XCD x gets one contiguous logical range
-    const int per_unit = group * a.nt;
-    const int unit = L / per_unit;
-    const int rem = L - unit * per_unit;
-    const int rank = rem / group;
-    const int hq = (unit % a.Hkv) * group + (rem - rank * group);
-    const int b = unit / a.Hkv;
-    const int kvh = unit % a.Hkv;
-    const int i = a.causal ? a.nt - 1 - rank : rank;
-
-    const int64_t qhead_row = ((int64_t)b * a.Hq + hq) * a.n_pad;
-    const int64_t khead_row = ((int64_t)b * a.Hkv + kvh) * a.n_pad;
-    const int q_local = 32 * w + r;
-    const int64_t q_row = qhead_row + (int64_t)i * TILE + q_local;
-
-    uint8_t* const kbuf0 = smem;
-    uint8_t* const vbuf0 = smem + 2 * G::K_BYTES;
-    // Visiting order.  The order of key tiles does not matter to the softmax, so the tiles that need special
-    // treatment go LAST: first every plain tile (main precision, no mask) in one tight loop, then the tile that
-    // holds the sequence tail (masked) if there is one, then the diagonal tile i (causal mask and / or 8-bit).
-    constexpr bool HAS4 = MODE != MPSA_MODE_MXFP8;        // 4-bit tiles exist (LDS pipeline in use)
-    constexpr bool PRE8 = MODE == MPSA_MODE_MXFP8;        // 8-bit K fragments are prefetched one step ahead
-    const bool tail = a.n < a.n_pad;
-    const bool diag_special = a.causal || MODE == MPSA_MODE_DIAG;
-    const bool tail_special = tail && !a.causal && !(MODE == MPSA_MODE_DIAG && i == a.nt - 1);
-    const int nsteps = a.causal ? i + 1 : a.nt;
-    const int n_plain = nsteps - (diag_special ? 1 : 0) - (tail_special ? 1 : 0);
-    const int skip = (MODE == MPSA_MODE_DIAG && !a.causal) ? i : 0x7fffffff;   // plain steps jump over tile i
-    auto tile_at = [&](int t) {
-        if (t < n_plain) return t + (t >= skip ? 1 : 0);
-        if (tail_special && t == n_plain) return a.nt - 1;
-        return i;
-    };
-    auto step_is8 = [&](int t) { return MODE == MPSA_MODE_MXFP8 || (MODE == MPSA_MODE_DIAG && t == nsteps - 1); };
-
-    // ---- Q fragments of the current precision stay in registers; re-read when the precision changes ----
-    v8i qf[G::SST];
-    int qsc = 0;
-    auto load_q = [&](bool is8) __attribute__((always_inline)) {
-        if (is8) {
-#pragma unroll
-            for (int s = 0; s < G::SST; ++s) {
-                // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
-                const v4i x0 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + s * 64 + h * 16);
-                const v4i x1 = *reinterpret_cast<const v4i*>(a.q8 + q_row * D + s * 64 + h * 16 + 32);
-                qf[s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-            }
-        } else {
-#pragma unroll
-            for (int s = 0; s < G::SST; ++s) {
-                const v4i x = *reinterpret_cast<const v4i*>(a.q4 + q_row * (D / 2) + (2 * s + h) * 16);
-                qf[s] = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
-            }
-        }
-        const uint8_t* qs = (is8 ? a.qs8 : a.qs4) + q_row * (D / 32);
-        const uint32_t sw = (D == 128) ? *reinterpret_cast<const uint32_t*>(qs) : (uint32_t)*reinterpret_cast<const uint16_t*>(qs);
-        qsc = (int)(sw >> (8 * h));
-    };
-
-    // ---- staging ----
-    auto issue_k4 = [&](int t) __attribute__((always_inline)) {           // 4-bit K tile of step t -> kbuf[t & 1], swizzled rows
-        const uint8_t* src = a.k4 + (khead_row + (int64_t)tile_at(t) * TILE) * G::ROW4;
-        uint8_t* dst = kbuf0 + (t & 1) * G::K_BYTES;
-#pragma unroll
-        for (int c = 0; c < G::KI4; ++c) {
-            const int ci = w * G::KI4 + c;
-            const int p = ci * 64 + lane;
-            const int row = p / G::CPR4, slot = p % G::CPR4;
-            const int cb = slot ^ ((row >> G::SH4) & (G::CPR4 - 1));
-            load16_to_lds(src + row * G::ROW4 + cb * 16, dst + ci * 1024);
-        }
-    };
-    auto issue_v = [&](int t) __attribute__((always_inline)) {            // V tile of step t -> vbuf[t & 1], flat
-        const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)tile_at(t) * TILE) * (D * 2);
-        uint8_t* dst = vbuf0 + (t & 1) * G::V_BYTES;
-#pragma unroll
-        for (int c = 0; c < G::VI; ++c) {
-            const int ci = w * G::VI + c;
-            load16_to_lds(src + ci * 1024 + lane * 16, dst + ci * 1024);
-        }
-    };
-    // K operand of the coming step, in registers: 4-bit fragments come from LDS, 8-bit ones straight from global
-    v4i kf4[HAS4 ? G::KB : 1][G::SST];
-    v8i kf8[PRE8 ? G::KB : 1][G::SST];
-    int ksc[G::KB];             // E8M0 bytes of this lane's key rows, shifted so bytes 0 / 2 belong to MX block h / 2+h
-    auto load_kscales = [&](int t, bool is8) __attribute__((always_inline)) {
-        const uint8_t* sp = (is8 ? a.ks8 : a.ks4) + (khead_row + (int64_t)tile_at(t) * TILE + r) * (D / 32);
-#pragma unroll
-        for (int kb = 0; kb < G::KB; ++kb) {
-            const uint32_t sw = (D == 128) ? *reinterpret_cast<const uint32_t*>(sp + kb * 32 * (D / 32))
-                                           : (uint32_t)*reinterpret_cast<const uint16_t*>(sp + kb * 32 * (D / 32));
-            ksc[kb] = (int)(sw >> (8 * h));
-        }
-    };
-    auto read_kf4 = [&](int t) __attribute__((always_inline)) {
-        const uint8_t* kl = kbuf0 + (t & 1) * G::K_BYTES;
-#pragma unroll
-        for (int kb = 0; kb < G::KB; ++kb) {
-            const int krow = 32 * kb + r;
-            const int f = (krow >> G::SH4) & (G::CPR4 - 1);
-#pragma unroll
-            for (int s = 0; s < G::SST; ++s)
-                kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * G::ROW4 + (((2 * s + h) ^ f) * 16));
-        }
-    };
-    auto load_kf8 = [&](int t, v8i (&dstf)[G::KB][G::SST]) __attribute__((always_inline)) {
-        const uint8_t* src = a.k8 + (khead_row + (int64_t)tile_at(t) * TILE + r) * G::ROW8 + h * 16;
-#pragma unroll
-        for (int kb = 0; kb < G::KB; ++kb)
-#pragma unroll
-            for (int s = 0; s < G::SST; ++s) {
-                // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
-                const v4i x0 = *reinterpret_cast<const v4i*>(src + kb * 32 * G::ROW8 + s * 64);
-                const v4i x1 = *reinterpret_cast<const v4i*>(src + kb * 32 * G::ROW8 + s * 64 + 32);
-                dstf[kb][s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-            }
-    };
-
-    v16f acc[G::NDB];
-#pragma unroll
-    for (int d = 0; d < G::NDB; ++d)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[d][e] = 0.0f;
-    // Running reference maximum of this lane's query, kept LAZILY: it moves only when a tile's maximum exceeds
-    // it by more than REBASE (so P stays below 2^REBASE, far inside the range of P's 16-bit type and of the float32
-    // accumulators), and -m_run rides into the score MFMA as its C operand,
-    // which makes the matrix core deliver S - m_run: the softmax costs no subtract and (almost) no rescale.
-    constexpr float REBASE = P::REBASE;
-    float m_run = 0.0f;
-    float l_run = 0.0f;
-    v16f negm;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) negm[e] = 0.0f;
-
-    // ---- prologue: V(0), K(0), K(1) on their way; operands of step 0 into registers ----
-    const bool first8 = step_is8(0);
-    issue_v(0);
-    if constexpr (HAS4) {
-        issue_k4(0);
-        if (nsteps > 1) issue_k4(1);
-    }
-    load_kscales(0, first8);
-    load_q(first8);
-    if constexpr (PRE8) load_kf8(0, kf8);
-    __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0)
-    __syncthreads();
-    if constexpr (HAS4) read_kf4(0);
-
-    // One step = one key tile.  IS8 / MASKED are compile-time so the common step (4-bit, unmasked) carries no
-    // branches or mask arithmetic.
-    //   PREP: also pull the next step's K operand (same precision as the run's plain tiles) into registers.
-    auto step = [&](int t, auto is8_c, auto masked_c, auto prep_c) __attribute__((always_inline)) {
-        constexpr bool IS8 = decltype(is8_c)::value;
-        constexpr bool MASKED = decltype(masked_c)::value;
-        constexpr bool PREP = decltype(prep_c)::value;
-        const int j = tile_at(t);                          // key tile of this step
-
-        // ---- S^T - m_run = K Q^T + (-m_run) ----
-        v16f st[G::KB];
-#pragma unroll
-        for (int kb = 0; kb < G::KB; ++kb) {
-            if constexpr (IS8 && PRE8) {
-                st[kb] = score_mfma8<FMT8>(kf8[kb][0], qf[0], negm, 0, ksc[kb], qsc);
-#pragma unroll
-                for (int s = 1; s < G::SST; ++s) st[kb] = score_mfma8<FMT8>(kf8[kb][s], qf[s], st[kb], s, ksc[kb], qsc);
-            } else if constexpr (IS8) {
-                // "diag" run: the single 8-bit tile's fragments come straight from global memory, block by block
-                const uint8_t* src = a.k8 + (khead_row + (int64_t)j * TILE + 32 * kb + r) * G::ROW8 + h * 16;
-#pragma unroll
-                for (int s = 0; s < G::SST; ++s) {
-                    const v4i x0 = *reinterpret_cast<const v4i*>(src + s * 64);
-                    const v4i x1 = *reinterpret_cast<const v4i*>(src + s * 64 + 32);
-                    const v8i kd = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-                    st[kb] = score_mfma8<FMT8>(kd, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
-                }
-            } else {
-#pragma unroll
-                for (int s = 0; s < G::SST; ++s) {
-                    const v4i x = kf4[kb][s];
-                    const v8i k8v = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
-                    st[kb] = score_mfma4(k8v, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
-                }
-            }
-        }
-
-        // ---- masks: causal on the diagonal tile, key tail on the last tile ----
-        if constexpr (MASKED) {
-            const bool diag_mask = a.causal && j == i;
-            const int kmax = (j == a.nt - 1) ? a.n - j * TILE : TILE;   // keys >= kmax are padding
-#pragma unroll
-            for (int kb = 0; kb < G::KB; ++kb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int key = 32 * kb + 8 * (e >> 2) + 4 * h + (e & 3);
-                    const bool dead = (diag_mask && key > q_local) || key >= kmax;
-                    if (dead) st[kb][e] = -__builtin_inff();
-                }
-        }
-
-        // ---- online softmax (per lane = per query): st holds S - m_run ----
-        float mx = st[0][0];
-#pragma unroll
-        for (int kb = 0; kb < G::KB; ++kb)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, st[kb][e]);
-        mx = max_lane_pair(mx);
-        if (t == 0 || __any(mx > REBASE)) {
-            // move the reference maximum up to this tile's maximum (first tile: set it)
-            const float delta = (t == 0) ? mx : __builtin_fmaxf(mx, 0.0f);
-            const float alpha = (t == 0) ? 1.0f : __builtin_amdgcn_exp2f(-delta);
-            m_run += delta;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) negm[e] = -m_run;
-#pragma unroll
-            for (int kb = 0; kb < G::KB; ++kb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) st[kb][e] -= delta;
-            l_run *= alpha;
-#pragma unroll
-            for (int d = 0; d < G::NDB; ++d)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[d][e] *= alpha;
-        }
-        // P = exp2(S - m_run), rounded to 16 bits for the P.V product; the row sum adds those 16-bit values
-        v4i pk[G::KB][2];                               // 8 packed 16-bit values = one P^T operand
-        float ps0 = 0.0f, ps1 = 0.0f;
-#pragma unroll
-        for (int kb = 0; kb < G::KB; ++kb)
-#pragma unroll
-            for (int c = 0; c < 2; ++c)
-#pragma unroll
-                for (int e = 0; e < 8; e += 2) {
-                    const float p0 = __builtin_amdgcn_exp2f(st[kb][8 * c + e]);
-                    const float p1 = __builtin_amdgcn_exp2f(st[kb][8 * c + e + 1]);
-                    const typename P::v2 pp = P::pack(p0, p1);
-                    pk[kb][c][e >> 1] = __builtin_bit_cast(int, pp);
-                    if (e & 2) ps1 = P::add2(pp, ps1); else ps0 = P::add2(pp, ps0);
-                }
-        l_run += ps0 + ps1;
-
-        // this wave's pieces of V(t) and K(t+1) have landed; after the barrier everybody's have, and everybody
-        // is done reading V(t-1) and the K(t) fragments
-        __builtin_amdgcn_sched_barrier(0);             // keep the softmax above and the loads below: register lifetimes
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
-
-        if (t + 1 < nsteps) issue_v(t + 1);
-        if constexpr (HAS4) {
-            if (t + 2 < nsteps) issue_k4(t + 2);
-        }
-
-        // ---- O^T += V^T P^T, V fragments prefetched PRE instructions ahead ----
-        constexpr int PRE = 8;
-        const uint8_t* vl = vbuf0 + (t & 1) * G::V_BYTES + lane * 16;
-        typename P::vec vf[PRE];
-#pragma unroll
-        for (int x = 0; x < PRE; ++x) vf[x] = *reinterpret_cast<const typename P::vec*>(vl + x * 1024);
-        // operands of the next step: scales (and 8-bit K) from global memory, 4-bit K from LDS.  Past the last
-        // step this reads a valid but unused tile.
-        if constexpr (PREP) {
-            load_kscales(t + 1, PRE8);
-            if constexpr (PRE8) load_kf8(t + 1, kf8);
-            if constexpr (HAS4) read_kf4(t + 1);
-        }
-#pragma unroll
-        for (int idx = 0; idx < G::NV; ++idx) {
-            const int d = idx % G::NDB, kc = idx / G::NDB;
-            const typename P::vec cur = vf[idx % PRE];
-            if (idx + PRE < G::NV) vf[idx % PRE] = *reinterpret_cast<const typename P::vec*>(vl + (idx + PRE) * 1024);
-            acc[d] = P::mfma(cur, __builtin_bit_cast(typename P::vec, pk[kc >> 1][kc & 1]), acc[d]);
-        }
-    };
-
-    // ---- plain tiles: one tight single-variant loop ----
-    for (int t = 0; t < n_plain; ++t) step(t, std::integral_constant<bool, PRE8>{}, std::false_type{}, std::true_type{});
-    // ---- the (at most two) special tiles: the sequence-tail tile, then the diagonal tile; both run the masked
-    //      variant (a mask that hides nothing is harmless).  The step before has already fetched their K operand
-    //      unless the precision changes. ----
-    if constexpr (MODE == MPSA_MODE_DIAG) {
-        if (tail_special) step(n_plain, std::false_type{}, std::true_type{}, std::true_type{});
-        if (nsteps > 1) {                              // otherwise the prologue already loaded 8-bit Q and scales
-            load_kscales(nsteps - 1, true);
-            load_q(true);
-        }
-        step(nsteps - 1, std::true_type{}, std::true_type{}, std::false_type{});
-    } else {
-        for (int t = n_plain; t < nsteps; ++t) step(t, std::integral_constant<bool, PRE8>{}, std::true_type{}, std::true_type{});
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
-
-    // ---- epilogue: O = acc / l ; register e of lane (h, r): dim 32*db + 8*(e/4) + 4*h + e%4 of query r ----
-    const float l_tot = sum_lane_pair(l_run);
-    const float inv = 1.0f / l_tot;
-    const int q_global = i * TILE + q_local;
-    if (q_global < a.n) {
-        uint8_t* orow = static_cast<uint8_t*>(a.o);
-        const int64_t off = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh + (int64_t)q_global * a.o_sn;
-#pragma unroll
-        for (int d = 0; d < G::NDB; ++d)
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const int dim = 32 * d + 8 * g4 + 4 * h;
-                const float o0 = acc[d][4 * g4 + 0] * inv, o1 = acc[d][4 * g4 + 1] * inv;
-                const float o2 = acc[d][4 * g4 + 2] * inv, o3 = acc[d][4 * g4 + 3] * inv;
-                if (a.o_dtype == MPSA_BF16) {
-                    typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
-                    const v4bf pk4 = {(__bf16)o0, (__bf16)o1, (__bf16)o2, (__bf16)o3};
-                    *reinterpret_cast<v4bf*>(orow + (off + dim) * 2) = pk4;
-                } else if (a.o_dtype == MPSA_F16) {
-                    typedef _Float16 v4hh __attribute__((ext_vector_type(4)));
-                    const v4hh pk4 = {(_Float16)o0, (_Float16)o1, (_Float16)o2, (_Float16)o3};
-                    *reinterpret_cast<v4hh*>(orow + (off + dim) * 2) = pk4;
-                } else {
-                    const v4f pk4 = {o0, o1, o2, o3};
-                    *reinterpret_cast<v4f*>(orow + (off + dim) * 4) = pk4;
-                }
-            }
-    }
-}
-
-template <int D, int TILE, int PVT, int FMT8, int MODE>
-int launch_one(const AttnArgs& a, hipStream_t st) {
-    typedef Geom<D, TILE> G;
-    constexpr int smem = G::SMEM;
-    static bool attr_set = false;      // idempotent; a race only repeats the same call
-    auto kern = attn_fwd_kernel<D, TILE, PVT, FMT8, MODE>;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "attn: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
-        attr_set = true;
-    }
-    dim3 grid((unsigned)(a.B * a.Hq * a.nt));
-    hipLaunchKernelGGL(kern, grid, dim3(G::NT), smem, st, a);
-    MPSA_CHECK_LAUNCH("attn");
-    return MPSA_OK;
-}
 
 template <int D, int TILE, int PVT>
 int launch_mode(const AttnArgs& a, hipStream_t st) {
@@ -425,11 +52,11 @@ int launch_dt(const AttnArgs& a, int pv_dtype, hipStream_t st) {
 
 }  // namespace
 
-extern "C" int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
-                             const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
-                             const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
-                             int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
-                             mpsa_stream_t stream) {
+static int attn_entry(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
+                      const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
+                      const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
+                      int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                      bool skip, float skip_thresh, int32_t* skipped, mpsa_stream_t stream) {
     if (mode != MPSA_MODE_MXFP4 && mode != MPSA_MODE_MXFP8 && mode != MPSA_MODE_DIAG) return mpsa_fail(MPSA_EINVAL, "attn: unknown mode %d", mode);
     const bool need4 = mode != MPSA_MODE_MXFP8, need8 = mode != MPSA_MODE_MXFP4;
     if (need4 && (!q4 || !qs4 || !k4 || !ks4)) return mpsa_fail(MPSA_EINVAL, "attn: 4-bit operands missing");
@@ -454,7 +81,14 @@ extern "C" int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_
     a.B = (int)B; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.n = (int)n; a.nt = (int)nt; a.n_pad = (int)(nt * tile);
     a.causal = causal ? 1 : 0; a.mode = mode; a.fmt8 = fmt8; a.o_dtype = o_dtype;
     a.d = (int)D; a.tile = tile;
+    a.skip_thresh = skip_thresh; a.skipped = skipped;
     hipStream_t st = (hipStream_t)stream;
+    if (skip) {
+        if (mode == MPSA_MODE_DIAG) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: tile skipping needs a single-precision mode (mxfp4 or mxfp8): the rule's reference tile is the first key tile, which a diag run visits last for query tile 0");
+        if (!(skip_thresh == skip_thresh)) return mpsa_fail(MPSA_EINVAL, "attn: skip_thresh is NaN");
+        if (skipped && (reinterpret_cast<uintptr_t>(skipped) & 3)) return mpsa_fail(MPSA_EALIGN, "attn: skipped must be 4-byte aligned");
+        return attn_skip_launch(a, pv_dtype, st);
+    }
     if (attn_pp_supported(a, pv_dtype)) return attn_pp_launch(a, pv_dtype, st);
 #ifdef MPSA_ATTN_ONLY_128
     if (D == 128 && tile == 128 && pv_dtype == MPSA_BF16 && fmt8 == MPSA_FMT_E4M3 && mode == MPSA_MODE_DIAG)
@@ -466,4 +100,22 @@ extern "C" int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_
     if (D == 128 && tile == 64)  return launch_dt<128, 64>(a, pv_dtype, st);
     return launch_dt<64, 128>(a, pv_dtype, st);
 #endif
+}
+
+extern "C" int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
+                             const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
+                             const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
+                             int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                             mpsa_stream_t stream) {
+    return attn_entry(q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
+                      B, Hq, Hkv, n, D, tile, causal, mode, false, 0.0f, nullptr, stream);
+}
+
+extern "C" int mpsa_attn_fwd_skip(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
+                                  const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
+                                  const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
+                                  int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                                  float skip_thresh, int32_t* skipped, mpsa_stream_t stream) {
+    return attn_entry(q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
+                      B, Hq, Hkv, n, D, tile, causal, mode, true, skip_thresh, skipped, stream);
 }

@@ -49,10 +49,21 @@ def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False
     return ops
 
 
-def attention_from_operands(ops, out, is_causal):
-    """Launch ``mpsa_attn_fwd`` on prepared operands; ``out`` is a ``[B,Hq,N,D]`` view (last dim contiguous)."""
+def attention_from_operands(ops, out, is_causal, skip_thresh=None, skipped=None):
+    """Launch ``mpsa_attn_fwd`` on prepared operands; ``out`` is a ``[B,Hq,N,D]`` view (last dim contiguous).
+    With ``skip_thresh`` the tile-skipping entry point runs instead (``skipped``: optional int32 ``[B,Hq,nt]``
+    that receives the number of skipped key tiles per query tile)."""
     B, Hq, Hkv, N, D = ops["shape"]
     dev = out.device
+    if skip_thresh is not None:
+        with torch.cuda.device(dev):
+            _lib.check(_lib.lib().mpsa_attn_fwd_skip(
+                _lib.ptr(ops["q4"]), _lib.ptr(ops["qs4"]), _lib.ptr(ops["q8"]), _lib.ptr(ops["qs8"]),
+                _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]), _lib.ptr(ops["ks8"]), ops["fmt8"],
+                _lib.ptr(ops["v_tiles"]), _lib.dtype_id(ops["v_tiles"].dtype), _lib.ptr(out), _lib.dtype_id(out.dtype),
+                _lib.strides4(out), B, Hq, Hkv, N, D, ops["tile"], 1 if is_causal else 0, ops["mode"],
+                float(skip_thresh), _lib.ptr(skipped), _lib.stream_ptr(dev)))
+        return out
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().mpsa_attn_fwd(
             _lib.ptr(ops["q4"]), _lib.ptr(ops["qs4"]), _lib.ptr(ops["q8"]), _lib.ptr(ops["qs8"]),
@@ -70,12 +81,13 @@ def _normalise(q, k, v):
     return q.to(lp), k.to(lp), v.to(lp)
 
 
-def _reject_unsupported(attn_mask, dropout_p, attention_sink, return_sparsity, skip_thresh):
-    if attn_mask is not None or dropout_p != 0.0 or attention_sink or return_sparsity:
-        raise NotImplementedError("attn_mask, dropout_p, attention_sink and return_sparsity are not implemented "
+def _reject_unsupported(attn_mask, dropout_p, attention_sink, block_scale_type, skip_thresh):
+    if attn_mask is not None or dropout_p != 0.0 or attention_sink:
+        raise NotImplementedError("attn_mask, dropout_p and attention_sink are not implemented "
                                   "(the reference accepts and ignores them)")
-    if skip_thresh is not None:
-        raise NotImplementedError("tile skipping (skip_thresh) is not implemented")
+    if skip_thresh is not None and block_scale_type in _MODES and _MODES[block_scale_type] == _lib.MODE_DIAG:
+        raise NotImplementedError("tile skipping (skip_thresh) needs a single-precision block_scale_type "
+                                  "(mxfp4, mxfp8, mxfp8e5): its reference tile is the first key tile")
 
 
 @torch.compiler.disable
@@ -88,9 +100,11 @@ def mxfp_attn_kernel(q, k, v, attn_mask=None, dropout_p=0.0,
     Signature of the reference (ours/mxfp_attn_kernel.py:19-22) plus ``tile`` (score tile edge, 64 or 128).
     ``block_scale_type``: ``"mxfp4"``, ``"mxfp8"`` (E4M3), ``"mxfp8e5"`` (E5M2, the reference's 8-bit format),
     ``"diag"`` (tile j == i in MXFP8, the rest in MXFP4) or ``"diag_e5"``.  K/V may have fewer heads than Q
-    (grouped-query attention); ``is_causal`` is honoured."""
+    (grouped-query attention); ``is_causal`` is honoured.  ``skip_thresh`` switches on the reference's tile
+    skipping (ours/mxfp_attn_kernel.py:272-297; single-precision types only); ``return_sparsity`` adds the share of
+    skipped tiles as a second result."""
     _lib.require_device(q, k, v)
-    _reject_unsupported(attn_mask, dropout_p, attention_sink, return_sparsity, skip_thresh)
+    _reject_unsupported(attn_mask, dropout_p, attention_sink, block_scale_type, skip_thresh)
     torch.cuda.set_device(v.device)
     q, k, v = _normalise(q, k, v)
     q, k, v = _as_bhnd(q, tensor_layout), _as_bhnd(k, tensor_layout), _as_bhnd(v, tensor_layout)
@@ -104,10 +118,20 @@ def mxfp_attn_kernel(q, k, v, attn_mask=None, dropout_p=0.0,
     if v.stride(-1) != 1:
         v = v.contiguous()
     ops = prepare_operands(q, k, v, tile, block_scale_type, scale, smooth_k=smooth_k)
+    nt = (N + tile - 1) // tile
+    skipped = None
+    if skip_thresh is not None and return_sparsity:
+        skipped = torch.zeros((B, Hq, nt), dtype=torch.int32, device=q.device)
     if tensor_layout == "HND":
         out = torch.empty((B, Hq, N, D), dtype=output_dtype, device=q.device)
-        attention_from_operands(ops, out, is_causal)
+        attention_from_operands(ops, out, is_causal, skip_thresh, skipped)
+    else:
+        out = torch.empty((B, N, Hq, D), dtype=output_dtype, device=q.device)
+        attention_from_operands(ops, out.transpose(1, 2), is_causal, skip_thresh, skipped)
+    if not return_sparsity:
         return out
-    out = torch.empty((B, N, Hq, D), dtype=output_dtype, device=q.device)
-    attention_from_operands(ops, out.transpose(1, 2), is_causal)
-    return out
+    # share of the visited (query tile, key tile) pairs that were skipped
+    visited = B * Hq * (nt * (nt + 1) // 2 if is_causal else nt * nt)
+    if skipped is None:
+        return out, torch.zeros((), dtype=torch.float32, device=q.device)
+    return out, skipped.sum().to(torch.float32) / visited

@@ -45,14 +45,21 @@ def _prepare(q, k, mode, scale, fmt8):
 
 
 def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=False,
-            fmt8=FMT_E4M3, out_dtype=None, heads=None, q_tiles=None) -> torch.Tensor:
+            fmt8=FMT_E4M3, out_dtype=None, heads=None, q_tiles=None, skip_thresh=None, return_skipped=False,
+            ratios_out=None):
     """Tile-by-tile MXFP attention.  q ``[B,Hq,N,D]``, k/v ``[B,Hkv,N,D]`` in bf16 or fp16.
 
     P is rounded to v's dtype before P.V and the product of a tile is accumulated in float32
     (ours/mxfp_attn_kernel.py:339-340).  ``heads`` restricts the computation to a list of query
     heads (the output then has ``len(heads)`` heads).  N need not be a multiple of ``tile``:
     the last key tile is cut at N.  ``q_tiles`` restricts the computation to a list of query tiles (all
-    keys are still visited); the output then holds only those tiles' rows, concatenated in list order."""
+    keys are still visited); the output then holds only those tiles' rows, concatenated in list order.
+
+    ``skip_thresh``: the reference's tile skipping (ours/mxfp_attn_kernel.py:272-297, with the pointer advance
+    a skipped tile needs): the statistic of a score tile is the mean over its query rows of the row maximum; key
+    tile 0 is always kept and sets the reference value, tile j > 0 is kept iff its statistic is at least
+    ``skip_thresh`` times that.  ``return_skipped`` adds an int32 ``[B, heads, tiles]`` count of skipped tiles;
+    a list passed as ``ratios_out`` collects statistic(j) / statistic(0) of every tile j > 0 examined."""
     B, Hq, N, D = q.shape
     Hkv = k.shape[1]
     assert Hq % Hkv == 0
@@ -72,6 +79,7 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
         starts[i] = n_out
         n_out += min((i + 1) * tile, N) - i * tile
     out = torch.empty((B, len(head_list), n_out, D), dtype=out_dtype)
+    skipped = torch.zeros((B, len(head_list), len(tile_list)), dtype=torch.int32)
     for b in range(B):
         for hi_, h in enumerate(head_list):
             kvh = h // group
@@ -92,6 +100,15 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
                         rr = torch.arange(r0, r1).unsqueeze(1)
                         cc = torch.arange(c0, c1).unsqueeze(0)
                         s = torch.where(cc > rr, torch.tensor(float("-inf")), s)
+                    if skip_thresh is not None:
+                        stat = s.amax(dim=1).sum() / rows
+                        if j == 0:
+                            sink = stat
+                        elif ratios_out is not None:
+                            ratios_out.append(float(stat / sink))
+                        if j > 0 and not bool(stat >= sink * skip_thresh):
+                            skipped[b, hi_, tile_list.index(i)] += 1
+                            continue
                     m_new = torch.maximum(m, s.amax(dim=1))
                     p = torch.exp2(s - m_new.unsqueeze(1))
                     alpha = torch.exp2(m - m_new)
@@ -100,6 +117,8 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
                     acc = acc * alpha.unsqueeze(1) + pv
                     m = m_new
                 out[b, hi_, starts[i]:starts[i] + rows] = (acc / l.unsqueeze(1)).to(out_dtype)
+    if return_skipped:
+        return out, skipped
     return out
 
 

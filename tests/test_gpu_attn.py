@@ -117,6 +117,63 @@ def test_c5_dit_shape_non_causal_ragged():
     _compare(got[:, :, rows.to(got.device)], want, "C5 query tiles 0, 100, 200, 255")
 
 
+def _robust_thresh(q, k, v, **kw):
+    """A threshold in the widest gap of the tile statistics' ratios to their sink (middle half of the distribution):
+    float32 summation order inside the matrix cores moves a statistic by parts in 1e6, so a tile that close to the
+    threshold could go either way; the gap must be at least 0.2 % wide."""
+    ratios = []
+    O.attn_mx(q, k, v, skip_thresh=0.0, ratios_out=ratios, **kw)
+    r = torch.tensor(sorted(ratios), dtype=torch.float64)
+    lo, hi = len(r) // 4, 3 * len(r) // 4
+    gaps = (r[lo + 1:hi + 1] - r[lo:hi]) / r[lo:hi].abs()
+    g = int(gaps.argmax())
+    assert gaps[g] > 2e-3, "tile statistics too dense for a robust threshold"
+    return float((r[lo + g] + r[lo + g + 1]) / 2)
+
+
+@pytest.mark.parametrize("mode,causal,N,D,tile", [("mxfp4", False, 1024, 128, 128), ("mxfp4", True, 1024, 128, 128),
+                                                  ("mxfp8", False, 1000, 128, 128), ("mxfp4", False, 512, 64, 64),
+                                                  ("mxfp8", True, 640, 64, 128), ("mxfp4", False, 520, 128, 64)])
+def test_tile_skipping_follows_the_reference_rule(mode, causal, N, D, tile):
+    """skip_thresh: key tile 0 always kept; tile j kept iff mean-of-row-maxima(j) >= skip_thresh * that of tile 0.  The kernel must skip
+    exactly the tiles the oracle skips (counted per query tile) and match its output."""
+    g = torch.Generator().manual_seed(N + D + tile)
+    H = 2
+    q = torch.randn(1, 2 * H, N, D, generator=g)
+    k = torch.randn(1, H, N, D, generator=g)
+    v = torch.randn(1, H, N, D, generator=g)
+    nt = -(-N // tile)
+    q = q + 1.0                                                    # a common direction in q, a per-tile amount of it in k:
+    k = k + torch.rand(nt, generator=g).repeat_interleave(tile)[:N].view(1, 1, N, 1) * 0.5     # tile statistics spread out
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    kw = dict(tile=tile, causal=causal, mode=mode)
+    th = _robust_thresh(q, k, v, **kw)
+    want, want_sk = O.attn_mx(q, k, v, skip_thresh=th, return_skipped=True, **kw)
+    got, sparsity = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=causal, block_scale_type=mode, tile=tile,
+                                     output_dtype=torch.bfloat16, skip_thresh=th, return_sparsity=True)
+    visited = 2 * H * (nt * (nt + 1) // 2 if causal else nt * nt)
+    assert abs(sparsity.item() - want_sk.sum().item() / visited) < 1e-6, (sparsity.item(), want_sk.sum().item(), visited)
+    _compare(got, want, f"skip {mode} causal={causal} th={th}")
+    # per query tile counts, through the C ABI's own output
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands
+    ops = prepare_operands(q.to(DEV), k.to(DEV), v.to(DEV), tile, mode)
+    out = torch.empty((1, 2 * H, N, D), dtype=torch.bfloat16, device=DEV)
+    sk = torch.full((1, 2 * H, nt), -1, dtype=torch.int32, device=DEV)
+    attention_from_operands(ops, out, causal, th, sk)
+    assert torch.equal(sk.cpu(), want_sk)
+    # a threshold nothing fails: identical to the plain kernel's result; one nothing passes: only key tile 0 counts
+    none = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=causal, block_scale_type=mode, tile=tile,
+                            output_dtype=torch.bfloat16, skip_thresh=-1e30)
+    plain = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=causal, block_scale_type=mode, tile=tile,
+                             output_dtype=torch.bfloat16)
+    _compare(none, plain.cpu().float(), "skip nothing")
+    if not causal:
+        only0 = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=False, block_scale_type=mode, tile=tile,
+                                 output_dtype=torch.bfloat16, skip_thresh=1e30)
+        want0 = O.attn_mx(q, k, v, skip_thresh=1e30, **kw)
+        _compare(only0, want0, "skip all but the sink")
+
+
 def test_fp16_inputs_nhd_layout_scale_and_public_entry():
     q, k, v = make_qkv(1, 4, 2, 256, 64, seed=44, dtype=torch.float16)
     want = O.attn_mx(q, k, v, tile=128, causal=True, mode="mxfp4", scale=0.2, out_dtype=torch.float16)
@@ -147,7 +204,7 @@ def test_error_behaviour():
         mxfp_attn(q, k, v, block_scale_type="nvfp4")
     with pytest.raises(ValueError, match="Unsupported dtype"):
         mxfp_attn(q, k, v, output_dtype=torch.int8)
-    with pytest.raises(NotImplementedError):
-        mxfp_attn(q, k, v, skip_thresh=0.5)
+    with pytest.raises(NotImplementedError, match="single-precision"):
+        mxfp_attn(q, k, v, skip_thresh=0.5, block_scale_type="diag")
     with pytest.raises(AssertionError, match="multiple of key/value heads"):
         mxfp_attn(q[:, :3], k, v)

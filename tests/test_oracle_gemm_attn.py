@@ -102,3 +102,44 @@ def test_v_fragment_order_is_a_permutation_with_zero_padding():
     assert f[0, 0, 0, 1, 0, 0, 3, 1] == v[0, 0, 32 + 1, 3]
     assert f.float().sum() == v.float().sum()                # padding keys are zero
     assert (f[0, 0, 1, 1, 0, :, :32, 4:] == 0).all()          # keys 64+32+8.. >= 100
+
+
+def test_tile_skipping_rule_against_a_dense_float64_restatement():
+    """attn_mx(skip_thresh=...) against an independent dense formulation: dequantised operands, one float64 score
+    matrix, tile statistics = mean over the tile's rows of the row maximum, decisions relative to key tile 0, then a
+    float64 softmax over the kept tiles only."""
+    from oracle.mx_attention import _prepare
+    g = torch.Generator().manual_seed(11)
+    B, H, N, D, tile = 1, 2, 320, 64, 64
+    q = torch.randn(B, H, N, D, generator=g)
+    k = torch.randn(B, H, N, D, generator=g)
+    v = torch.randn(B, H, N, D, generator=g).bfloat16()
+    nt = N // tile
+    # a common direction in q and a per-tile amount of it in k spread the tile statistics out
+    q = q + 1.0
+    k = k + torch.rand(nt, generator=g).repeat_interleave(tile).view(1, 1, N, 1) * 0.5
+    q, k = q.bfloat16(), k.bfloat16()
+    for causal in (False, True):
+        for th in (0.7, 0.9, 1.05):
+            got, sk = O.attn_mx(q, k, v, tile=tile, causal=causal, mode="mxfp4", skip_thresh=th, return_skipped=True,
+                                out_dtype=torch.float32)
+            ops = _prepare(q, k, "mxfp4", None, O.FMT_E4M3)
+            s = ops["q4"].double() @ ops["k4"].double().transpose(-1, -2)            # [B,H,N,N], log2 units
+            if causal:
+                s = s.masked_fill(torch.triu(torch.ones(N, N, dtype=torch.bool), 1), float("-inf"))
+            keep = torch.ones(B, H, nt, nt, dtype=torch.bool)
+            for i in range(nt):
+                rows = slice(i * tile, (i + 1) * tile)
+                last = i if causal else nt - 1
+                stat = [s[:, :, rows, j * tile:(j + 1) * tile].amax(dim=-1).mean(dim=-1) for j in range(last + 1)]
+                for j in range(1, last + 1):
+                    keep[:, :, i, j] = stat[j] >= stat[0] * th
+                if causal:
+                    keep[:, :, i, i + 1:] = True      # not visited: already -inf
+            mask = keep.repeat_interleave(tile, 2).repeat_interleave(tile, 3)
+            p = torch.softmax(s.masked_fill(~mask, float("-inf")) * 0.6931471805599453, dim=-1)
+            want = p @ v.double()
+            visited = torch.tril(torch.ones(nt, nt, dtype=torch.bool)) if causal else torch.ones(nt, nt, dtype=torch.bool)
+            assert torch.equal(sk, ((~keep) & visited).sum(dim=-1).to(torch.int32))
+            assert 0 < sk.sum() < visited.sum() * B * H
+            assert (got.double() - want).abs().max() < 2e-2
