@@ -63,6 +63,16 @@ int mpsa_e8m0_encode(const float* x, int64_t n, uint8_t* codes, mpsa_stream_t st
 int mpsa_e8m0_decode(const uint8_t* codes, int64_t n, float* out, mpsa_stream_t stream);
 
 /*
+ * E8M0 scale re-layout between this library's linear form [batch, rows, K/32] and the 5-D packed form the
+ * reference's block-scaled kernels consume, [batch, rows/128, K/128, 32, 4, 4] with
+ * packed[cm][ck][r32][r4][c4] = linear[cm*128 + r4*32 + r32][ck*4 + c4].  Replaces the reshape/permute at
+ * ours/mxfp_attn_kernel.py:56-57 (to the packed form) and ours/block_scaled_matmul.py:384 (back), so that scale
+ * tensors can be exchanged with code written against the reference.  rows % 128 == 0, kblocks = K/32, kblocks % 4 == 0.
+ */
+int mpsa_scales_to_5d(const uint8_t* linear, int64_t batch, int64_t rows, int64_t kblocks, uint8_t* packed, mpsa_stream_t stream);
+int mpsa_scales_from_5d(const uint8_t* packed, int64_t batch, int64_t rows, int64_t kblocks, uint8_t* linear, mpsa_stream_t stream);
+
+/*
  * MX quantizer.  Replaces quant_mxfp4 / quant_mxfp8e5 and their Triton kernels
  * (ours/quant_mxint8.py:453-512, :276-351, :223-272, :164-219) together with the host-side
  * nibble packing MXFP4Tensor.to_packed_tensor (ours/mxfp.py:172-205).

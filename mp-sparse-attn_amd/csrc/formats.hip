@@ -70,7 +70,47 @@ int run(const char* what, K kern, int64_t n, hipStream_t st, A... args) {
     return MPSA_OK;
 }
 
+// Scale re-layout between the linear [rows, K/32] form and the 5-D packed form of the reference's block-scaled
+// kernels, [rows/128, K/128, 32, 4, 4] with packed[cm][ck][r32][r4][c4] = linear[cm*128 + r4*32 + r32][ck*4 + c4]
+// (ours/mxfp_attn_kernel.py:56-57, ours/block_scaled_matmul.py:384 for the way back).  The innermost c4 group is four
+// consecutive bytes in both forms, so a thread moves one 32-bit word; `w` runs over the packed form's words.
+template <bool TO_PACKED>
+__global__ __launch_bounds__(256) void scale_layout_kernel(const uint32_t* src, uint32_t* dst, int64_t words_per_batch, int kc) {
+    const int64_t w = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (w >= words_per_batch) return;
+    const int64_t boff = (int64_t)blockIdx.y * words_per_batch;
+    const int r4 = (int)(w & 3), r32 = (int)((w >> 2) & 31);
+    const int64_t t = w >> 7;                      // cm * kc + ck
+    const int64_t cm = t / kc;
+    const int ck = (int)(t - cm * kc);
+    const int64_t lin = (cm * 128 + r4 * 32 + r32) * kc + ck;
+    if (TO_PACKED) dst[boff + w] = src[boff + lin];
+    else           dst[boff + lin] = src[boff + w];
+}
+
+int scale_layout(const char* what, const uint8_t* src, int64_t batch, int64_t rows, int64_t kblocks, uint8_t* dst,
+                 bool to_packed, hipStream_t st) {
+    if (batch <= 0 || rows <= 0 || kblocks <= 0) return mpsa_fail(MPSA_EINVAL, "%s: bad shape", what);
+    if (rows % 128 || kblocks % 4) return mpsa_fail(MPSA_EUNSUPPORTED, "%s: rows must be a multiple of 128 and K of 128 (got rows=%lld, K/32=%lld)", what, (long long)rows, (long long)kblocks);
+    if (!src || !dst) return mpsa_fail(MPSA_EINVAL, "%s: null pointer", what);
+    if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 3) return mpsa_fail(MPSA_EALIGN, "%s: pointers must be 4-byte aligned", what);
+    const int64_t words = rows * (kblocks / 4);
+    if (batch > 65535 || words >= (int64_t(1) << 38)) return mpsa_fail(MPSA_EUNSUPPORTED, "%s: shape too large", what);
+    dim3 grid((unsigned)((words + 255) / 256), (unsigned)batch);
+    if (to_packed) hipLaunchKernelGGL(scale_layout_kernel<true>, grid, dim3(256), 0, st, reinterpret_cast<const uint32_t*>(src), reinterpret_cast<uint32_t*>(dst), words, (int)(kblocks / 4));
+    else           hipLaunchKernelGGL(scale_layout_kernel<false>, grid, dim3(256), 0, st, reinterpret_cast<const uint32_t*>(src), reinterpret_cast<uint32_t*>(dst), words, (int)(kblocks / 4));
+    MPSA_CHECK_LAUNCH(what);
+    return MPSA_OK;
+}
+
 }  // namespace
+
+extern "C" int mpsa_scales_to_5d(const uint8_t* linear, int64_t batch, int64_t rows, int64_t kblocks, uint8_t* packed, mpsa_stream_t stream) {
+    return scale_layout("scales_to_5d", linear, batch, rows, kblocks, packed, true, (hipStream_t)stream);
+}
+extern "C" int mpsa_scales_from_5d(const uint8_t* packed, int64_t batch, int64_t rows, int64_t kblocks, uint8_t* linear, mpsa_stream_t stream) {
+    return scale_layout("scales_from_5d", packed, batch, rows, kblocks, linear, false, (hipStream_t)stream);
+}
 
 extern "C" int mpsa_e2m1_encode(const float* x, int64_t n, uint8_t* codes, mpsa_stream_t stream) {
     if (n > 0 && (!x || !codes)) return mpsa_fail(MPSA_EINVAL, "e2m1_encode: null pointer");

@@ -2,7 +2,8 @@
 
 ``block_scaled_matmul(a, a_scale, b, b_scale, dtype_dst, M, N, K, configs)`` keeps the reference
 signature (ours/block_scaled_matmul.py:271).  Operands are what the quantizer emits: row-major codes
-(``[M, K/2]`` packed E2M1 or ``[M, K]`` 8-bit) and linear E8M0 scales ``[M, K/32]``; B is ``[N, K]``
+(``[M, K/2]`` packed E2M1 or ``[M, K]`` 8-bit) and linear E8M0 scales ``[M, K/32]`` (the reference's 5-D packed
+scales ``[M/128, K/128, 32, 4, 4]`` are accepted too and re-laid out first); B is ``[N, K]``
 (NT product).  The element format is read from ``configs["ELEM_PER_BYTE_A"]`` (2 = E2M1) and, for
 8-bit, ``configs.get("FMT8", "e4m3")``.
 """
@@ -35,6 +36,33 @@ def _fmt_of(configs):
     return _lib.FMT_E5M2 if configs.get("FMT8", "e4m3") == "e5m2" else _lib.FMT_E4M3
 
 
+def pack_scale_5d(scale):
+    """Linear E8M0 scales ``[..., rows, K/32]`` -> the reference's packed form ``[..., rows/128, K/128, 32, 4, 4]``
+    (ours/mxfp_attn_kernel.py:56-57), through ``mpsa_scales_to_5d``."""
+    _lib.require_device(scale)
+    scale = scale.contiguous()
+    rows, kb = scale.shape[-2], scale.shape[-1]
+    batch = scale.numel() // max(rows * kb, 1)
+    out = torch.empty((*scale.shape[:-2], rows // 128, kb // 4, 32, 4, 4), dtype=torch.uint8, device=scale.device)
+    with torch.cuda.device(scale.device):
+        _lib.check(_lib.lib().mpsa_scales_to_5d(_lib.ptr(scale), batch, rows, kb, _lib.ptr(out), _lib.stream_ptr(scale.device)))
+    return out
+
+
+def unpack_scale_5d(packed):
+    """The reference's packed scales ``[..., rows/128, K/128, 32, 4, 4]`` -> linear ``[..., rows, K/32]``
+    (ours/block_scaled_matmul.py:384), through ``mpsa_scales_from_5d``."""
+    _lib.require_device(packed)
+    assert packed.dim() >= 5 and packed.shape[-3:] == (32, 4, 4), "expected [..., rows/128, K/128, 32, 4, 4]"
+    packed = packed.contiguous()
+    rows, kb = packed.shape[-5] * 128, packed.shape[-4] * 4
+    batch = packed.numel() // max(rows * kb, 1)
+    out = torch.empty((*packed.shape[:-5], rows, kb), dtype=torch.uint8, device=packed.device)
+    with torch.cuda.device(packed.device):
+        _lib.check(_lib.lib().mpsa_scales_from_5d(_lib.ptr(packed), batch, rows, kb, _lib.ptr(out), _lib.stream_ptr(packed.device)))
+    return out
+
+
 def block_scaled_matmul(a, a_scale, b, b_scale, dtype_dst, M, N, K, configs):
     """``C = (A o 2^(sa-127)) @ (B o 2^(sb-127))^T`` with float32 accumulation.
 
@@ -43,6 +71,10 @@ def block_scaled_matmul(a, a_scale, b, b_scale, dtype_dst, M, N, K, configs):
         raise ValueError(f"Unsupported dtype: {dtype_dst}")
     fmt = _fmt_of(configs)
     _lib.require_device(a, a_scale, b, b_scale)
+    if a_scale.dim() == 5:                       # the reference's packed scale layout
+        a_scale = unpack_scale_5d(a_scale)
+    if b_scale.dim() == 5:
+        b_scale = unpack_scale_5d(b_scale)
     width = K // 2 if fmt == _lib.FMT_E2M1 else K
     a = a.view(torch.uint8).contiguous()
     b = b.view(torch.uint8).contiguous()

@@ -27,6 +27,8 @@ Parity status of each restated function:
   one ulp below a power of two; (2) an all-zero block gets scale byte 0 and
   codes +0.
 * ``gemm_mx`` -- dequantise + matmul; pinned against exact integer arithmetic.
+* ``scales_to_5d`` / ``scales_from_5d`` -- the reference's reshape/permute, pinned
+  by the explicit index formula and the round trip.
 * ``attn_mx`` -- pinned against dense float64 softmax attention on the same
   per-tile dequantised operands, and special cases (single tile, V = 1,
   identical keys, GQA == repeat_interleave).  Its tile-skipping rule
@@ -47,5 +49,5 @@ from .mx_formats import (  # noqa: F401
 from .mx_quantize import (  # noqa: F401
     FMT_E2M1, FMT_E4M3, FMT_E5M2, EMAX_ELEM, q_pre_scale, quantize_mx, dequantize_mx, smooth_k, seq_mean,
 )
-from .mx_gemm import gemm_mx  # noqa: F401
+from .mx_gemm import gemm_mx, scales_to_5d, scales_from_5d  # noqa: F401
 from .mx_attention import attn_mx, attn_dense_f64, precision_metric, v_fragment_order  # noqa: F401

@@ -22,3 +22,21 @@ def gemm_mx(a_codes, a_scales, b_codes, b_scales, fmt_a, fmt_b=None, acc_dtype=t
     b = dequantize_mx(b_codes, b_scales, fmt_b, acc_dtype)
     c = a @ b.transpose(-1, -2)
     return c if out_dtype is None else c.to(out_dtype)
+
+
+def scales_to_5d(scale: torch.Tensor) -> torch.Tensor:
+    """Linear ``[..., rows, K/32]`` scales -> the reference's packed ``[..., rows/128, K/128, 32, 4, 4]``:
+    ``reshape(..., rows//128, 4, 32, K//32//4, 4).permute(..., 0, 3, 2, 1, 4)`` -- ours/mxfp_attn_kernel.py:56-57."""
+    *lead, rows, kb = scale.shape
+    n = len(lead)
+    x = scale.reshape(*lead, rows // 128, 4, 32, kb // 4, 4)
+    return x.permute(*range(n), n + 0, n + 3, n + 2, n + 1, n + 4).contiguous()
+
+
+def scales_from_5d(packed: torch.Tensor) -> torch.Tensor:
+    """Inverse of :func:`scales_to_5d`: ``permute(0, 3, 2, 1, 4).reshape(chunks_m*128, chunks_k*4)`` --
+    ours/block_scaled_matmul.py:384."""
+    *lead, cm, ck, r32, r4, c4 = packed.shape
+    n = len(lead)
+    x = packed.permute(*range(n), n + 0, n + 3, n + 2, n + 1, n + 4)
+    return x.reshape(*lead, cm * 128, ck * 4).contiguous()

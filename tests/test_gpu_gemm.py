@@ -125,3 +125,23 @@ def test_errors():
         block_scaled_matmul(ac, asc, bc, bsc, torch.int32, 256, 256, 128, cfg)
     with pytest.raises(_lib.MpsaError, match="multiples of 256"):
         block_scaled_matmul(ac[:128], asc[:128], bc, bsc, torch.float32, 128, 256, 128, cfg)
+
+
+def test_scale_5d_layout_and_matmul_with_packed_scales():
+    """mpsa_scales_to_5d / _from_5d bit for bit against the reference's reshape/permute, and the matmul fed
+    5-D packed scales gives the same bits as with linear ones."""
+    from ours.block_scaled_matmul import pack_scale_5d, unpack_scale_5d
+    g = torch.Generator().manual_seed(9)
+    lin = torch.randint(0, 255, (3, 2, 384, 24), dtype=torch.uint8, generator=g)
+    pk = pack_scale_5d(lin.to(DEV))
+    assert torch.equal(pk.cpu(), O.scales_to_5d(lin))
+    assert torch.equal(unpack_scale_5d(pk).cpu(), lin)
+    M, N, K = 256, 512, 512
+    a = torch.randn(M, K, generator=g).bfloat16()
+    b = torch.randn(N, K, generator=g).bfloat16()
+    ac, asc, bc, bsc, cfg = initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), "mxfp4")
+    c_lin = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg)
+    c_pk = block_scaled_matmul(ac, pack_scale_5d(asc), bc, pack_scale_5d(bsc), torch.float32, M, N, K, cfg)
+    assert torch.equal(c_lin, c_pk)
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        pack_scale_5d(lin[:, :, :100].contiguous().to(DEV))

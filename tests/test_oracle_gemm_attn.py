@@ -143,3 +143,13 @@ def test_tile_skipping_rule_against_a_dense_float64_restatement():
             assert torch.equal(sk, ((~keep) & visited).sum(dim=-1).to(torch.int32))
             assert 0 < sk.sum() < visited.sum() * B * H
             assert (got.double() - want).abs().max() < 2e-2
+
+
+def test_scale_5d_layout_index_formula_and_round_trip():
+    rows, kb = 256, 8
+    lin = torch.arange(2 * rows * kb, dtype=torch.int64).remainder(251).to(torch.uint8).view(2, rows, kb)
+    pk = O.scales_to_5d(lin)
+    assert pk.shape == (2, rows // 128, kb // 4, 32, 4, 4)
+    for (bt, cm, ck, r32, r4, c4) in [(0, 0, 0, 0, 0, 0), (1, 1, 1, 31, 3, 3), (0, 1, 0, 7, 2, 1), (1, 0, 1, 30, 1, 2)]:
+        assert pk[bt, cm, ck, r32, r4, c4] == lin[bt, cm * 128 + r4 * 32 + r32, ck * 4 + c4]
+    assert torch.equal(O.scales_from_5d(pk), lin)
