@@ -142,6 +142,25 @@ int mpsa_v_tiles(const void* v, int v_dtype, int64_t B, int64_t H, int64_t N, in
                  const int64_t v_strides[4], int tile, void* v_tiles, mpsa_stream_t stream);
 
 /*
+ * All operands of one attention call in ONE launch: Q quantized with pre_scale_q folded in, K quantized (minus
+ * k_sub if given, see mpsa_quantize_mx), V repacked - the results are bit-identical to the separate calls
+ * mpsa_quantize_mx(_dual) on q and k (emax 3 for E2M1, 7 for the 8-bit format) and mpsa_v_tiles on v, rows padded to
+ * n_pad = ceil(N/tile)*tile.  Replaces the prologue of the reference's wrapper, ours/mxfp_attn_kernel.py:27-57.
+ *
+ *   q [B,Hq,N,D], k and v [B,Hkv,N,D] of dtype (MPSA_BF16 | MPSA_F16), element strides as for mpsa_quantize_mx
+ *   mode       MPSA_MODE_MXFP4: only the 4-bit outputs are written (8-bit pointers may be null),
+ *              MPSA_MODE_MXFP8: only the 8-bit ones, MPSA_MODE_DIAG: both
+ *   k_sub      NULL or [B,Hkv,D] (smooth-K mean from mpsa_seq_mean)
+ *   outputs    as the inputs of mpsa_attn_fwd
+ */
+int mpsa_attn_prepare(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                      const void* v, const int64_t v_strides[4], int dtype,
+                      int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int tile, int mode, int fmt8,
+                      float pre_scale_q, const void* k_sub,
+                      uint8_t* q4, uint8_t* qs4, uint8_t* q8, uint8_t* qs8,
+                      uint8_t* k4, uint8_t* ks4, uint8_t* k8, uint8_t* ks8, void* v_tiles, mpsa_stream_t stream);
+
+/*
  * Fused attention forward.  Replaces block_scaled_batched_attn and its Triton kernel
  * (ours/mxfp_attn_kernel.py:362-423, :103-359), with the causal tile structure and grouped-query
  * head mapping of ours/online_routing.py:68-77, :113-118, :160-171.

@@ -11,47 +11,11 @@
 //
 // Replaces the reference wrapper's V normalisation (ours/mxfp_attn_kernel.py:27-31).  HBM-bound:
 // 2 B/element in, 2 B/element out.
-#include "mpsa_common.h"
+#include "v_tiles_kernel.h"
 
-namespace {
-
-struct VTArgs {
-    const unsigned short* v;
-    int64_t sb, sh, sn;
-    int n, nt;
-    unsigned short* out;
-};
-
-template <int TILE, int D>
-__global__ __launch_bounds__(256) void v_tiles_kernel(VTArgs a) {
-    constexpr int NDB = D / 32;
-    constexpr int KB = TILE / 32;
-    const uint32_t per_head = (uint32_t)a.nt * (TILE * D / 8);
-    const uint32_t o = blockIdx.x * 256u + threadIdx.x;
-    if (o >= per_head) return;
-    const uint32_t lane = o & 63u;
-    uint32_t rest = o >> 6;
-    const uint32_t db = rest % NDB; rest /= NDB;
-    const uint32_t c = rest & 1u;   rest >>= 1;
-    const uint32_t kb = rest % KB;
-    const uint32_t it = rest / KB;
-    const uint32_t h = lane >> 5, r = lane & 31u;
-    const uint32_t key0 = TILE * it + 32u * kb + 16u * c + 4u * h;
-    const unsigned short* src = a.v + (int64_t)blockIdx.z * a.sb + (int64_t)blockIdx.y * a.sh + (32u * db + r);
-    v8us val;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        const uint32_t key = key0 + 8u * (t >> 2) + (t & 3);
-        val[t] = key < (uint32_t)a.n ? src[(int64_t)key * a.sn] : (unsigned short)0;
-    }
-    const int64_t head = (int64_t)blockIdx.z * gridDim.y + blockIdx.y;
-    reinterpret_cast<v8us*>(a.out)[head * per_head + o] = val;
-}
-
-}  // namespace
-
-extern "C" int mpsa_v_tiles(const void* v, int v_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
-                            const int64_t v_strides[4], int tile, void* v_tiles, mpsa_stream_t stream) {
+int mpsa_v_tiles_setup(const void* v, int v_dtype, int64_t B, int64_t H, int64_t N, int64_t D, const int64_t* v_strides,
+                       int tile, void* v_tiles, VTArgs* out, unsigned* blocks) {
+    *blocks = 0;
     if (!v || !v_tiles || !v_strides) return mpsa_fail(MPSA_EINVAL, "v_tiles: null pointer");
     if (v_dtype != MPSA_BF16 && v_dtype != MPSA_F16) return mpsa_fail(MPSA_EINVAL, "v_tiles: dtype must be bf16 or f16");
     if (B < 0 || H < 0 || N <= 0) return mpsa_fail(MPSA_EINVAL, "v_tiles: bad shape");
@@ -63,12 +27,22 @@ extern "C" int mpsa_v_tiles(const void* v, int v_dtype, int64_t B, int64_t H, in
     const int64_t nt = (N + tile - 1) / tile;
     const int64_t per_head = nt * (tile * D / 8);
     if (per_head >= (int64_t(1) << 31) || H > 65535 || B > 65535) return mpsa_fail(MPSA_EUNSUPPORTED, "v_tiles: tensor too large");
-    VTArgs a;
+    VTArgs& a = *out;
     a.v = static_cast<const unsigned short*>(v);
     a.sb = v_strides[0]; a.sh = v_strides[1]; a.sn = v_strides[2];
     a.n = (int)N; a.nt = (int)nt;
     a.out = static_cast<unsigned short*>(v_tiles);
-    dim3 grid((unsigned)((per_head + 255) / 256), (unsigned)H, (unsigned)B);
+    *blocks = (unsigned)((per_head + 255) / 256);
+    return MPSA_OK;
+}
+
+extern "C" int mpsa_v_tiles(const void* v, int v_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                            const int64_t v_strides[4], int tile, void* v_tiles, mpsa_stream_t stream) {
+    VTArgs a;
+    unsigned blocks = 0;
+    const int rc = mpsa_v_tiles_setup(v, v_dtype, B, H, N, D, v_strides, tile, v_tiles, &a, &blocks);
+    if (rc != MPSA_OK || blocks == 0) return rc;
+    dim3 grid(blocks, (unsigned)H, (unsigned)B);
     hipStream_t st = (hipStream_t)stream;
     if (tile == 128 && D == 128)      hipLaunchKernelGGL((v_tiles_kernel<128, 128>), grid, dim3(256), 0, st, a);
     else if (tile == 128 && D == 64)  hipLaunchKernelGGL((v_tiles_kernel<128, 64>), grid, dim3(256), 0, st, a);

@@ -1,15 +1,15 @@
 """Fused MXFP attention -- the reference's ``ours/mxfp_attn_kernel.py::mxfp_attn_kernel`` on HIP kernels.
 
 Pipeline per call (all on torch's current stream, no host synchronisation):
-  1. MX-quantize Q (with ``scale*log2e`` folded in) and K -- ``mpsa_quantize_mx`` / ``_dual``;
-  2. repack V into matrix-core operand order -- ``mpsa_v_tiles``;
-  3. fused attention -- ``mpsa_attn_fwd``.
+  1. MX-quantize Q (with ``scale*log2e`` folded in) and K, repack V into matrix-core operand order -- one launch,
+     ``mpsa_attn_prepare`` (preceded by ``mpsa_seq_mean`` when ``smooth_k``);
+  2. fused attention -- ``mpsa_attn_fwd`` / ``mpsa_attn_fwd_skip``.
 """
 
 import torch
 
 from . import _lib
-from .quant_mxint8 import quantize_mx, quantize_mx_dual, seq_mean, pre_scale_q, _as_bhnd
+from .quant_mxint8 import seq_mean, pre_scale_q, _as_bhnd, _check_input
 
 _MODES = {"mxfp4": _lib.MODE_MXFP4, "mxfp8": _lib.MODE_MXFP8, "mxfp8e5": _lib.MODE_MXFP8, "diag": _lib.MODE_DIAG,
           "diag_e5": _lib.MODE_DIAG}
@@ -31,19 +31,24 @@ def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False
            "k4": None, "ks4": None, "k8": None, "ks8": None}
     # smooth-K (ours/mxfp_attn_kernel.py:33-34): the mean over the sequence is subtracted inside the K quantizer
     kmean = seq_mean(k) if smooth_k else None
-    if mode == _lib.MODE_DIAG:
-        ops["q4"], ops["qs4"], ops["q8"], ops["qs8"] = quantize_mx_dual(q, pre, fmt8, n_pad)
-        ops["k4"], ops["ks4"], ops["k8"], ops["ks8"] = quantize_mx_dual(k, 1.0, fmt8, n_pad, sub=kmean)
-    elif mode == _lib.MODE_MXFP4:
-        ops["q4"], ops["qs4"] = quantize_mx(q, pre, _lib.FMT_E2M1, out_rows=n_pad)
-        ops["k4"], ops["ks4"] = quantize_mx(k, 1.0, _lib.FMT_E2M1, out_rows=n_pad, sub=kmean)
-    else:
-        ops["q8"], ops["qs8"] = quantize_mx(q, pre, fmt8, out_rows=n_pad)
-        ops["k8"], ops["ks8"] = quantize_mx(k, 1.0, fmt8, out_rows=n_pad, sub=kmean)
+    q, k = _check_input(q), _check_input(k)
+    dev = q.device
+    need4, need8 = mode != _lib.MODE_MXFP8, mode != _lib.MODE_MXFP4
+    u8 = lambda *shape: torch.empty(shape, dtype=torch.uint8, device=dev)
+    if need4:
+        ops["q4"], ops["qs4"] = u8(B, Hq, n_pad, D // 2), u8(B, Hq, n_pad, D // 32)
+        ops["k4"], ops["ks4"] = u8(B, Hkv, n_pad, D // 2), u8(B, Hkv, n_pad, D // 32)
+    if need8:
+        ops["q8"], ops["qs8"] = u8(B, Hq, n_pad, D), u8(B, Hq, n_pad, D // 32)
+        ops["k8"], ops["ks8"] = u8(B, Hkv, n_pad, D), u8(B, Hkv, n_pad, D // 32)
     v_tiles = torch.empty((B, Hkv, nt, tile * D), dtype=v.dtype, device=v.device)
-    with torch.cuda.device(v.device):
-        _lib.check(_lib.lib().mpsa_v_tiles(_lib.ptr(v), _lib.dtype_id(v.dtype), B, Hkv, N, D, _lib.strides4(v), tile,
-                                           _lib.ptr(v_tiles), _lib.stream_ptr(v.device)))
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mpsa_attn_prepare(
+            _lib.ptr(q), _lib.strides4(q), _lib.ptr(k), _lib.strides4(k), _lib.ptr(v), _lib.strides4(v),
+            _lib.dtype_id(q.dtype), B, Hq, Hkv, N, D, tile, mode, fmt8, pre, _lib.ptr(kmean),
+            _lib.ptr(ops["q4"]), _lib.ptr(ops["qs4"]), _lib.ptr(ops["q8"]), _lib.ptr(ops["qs8"]),
+            _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]), _lib.ptr(ops["ks8"]),
+            _lib.ptr(v_tiles), _lib.stream_ptr(dev)))
     ops["v_tiles"] = v_tiles
     ops["shape"] = (B, Hq, Hkv, N, D)
     return ops

@@ -174,6 +174,38 @@ def test_tile_skipping_follows_the_reference_rule(mode, causal, N, D, tile):
         _compare(only0, want0, "skip all but the sink")
 
 
+@pytest.mark.parametrize("mode", ["diag", "mxfp4", "mxfp8e5"])
+@pytest.mark.parametrize("dtype,N,D,tile", [(torch.bfloat16, 1000, 128, 128), (torch.float16, 200, 64, 64)])
+def test_one_launch_preparation_equals_the_separate_calls(mode, dtype, N, D, tile):
+    """mpsa_attn_prepare writes the same bits as mpsa_quantize_mx(_dual) on q and k plus mpsa_v_tiles on v,
+    strided (NHD) inputs and the smooth-K subtraction included."""
+    from ours.mxfp_attn_kernel import prepare_operands
+    from ours.quant_mxint8 import quantize_mx, quantize_mx_dual, seq_mean, pre_scale_q
+    q, k, v = make_qkv(2, 4, 2, N, D, seed=N, dtype=dtype)
+    qd, kd, vd = (t.transpose(1, 2).contiguous().to(DEV).transpose(1, 2) for t in (q, k, v))     # NHD storage
+    ops = prepare_operands(qd, kd, vd, tile, mode, None, smooth_k=True)
+    n_pad = -(-N // tile) * tile
+    pre, fmt8 = pre_scale_q(D), (_lib.FMT_E5M2 if mode.endswith("e5") else _lib.FMT_E4M3)
+    km = seq_mean(kd)
+    if mode == "diag":
+        want = dict(zip(("q4", "qs4", "q8", "qs8"), quantize_mx_dual(qd, pre, fmt8, n_pad)))
+        want.update(zip(("k4", "ks4", "k8", "ks8"), quantize_mx_dual(kd, 1.0, fmt8, n_pad, sub=km)))
+    elif mode == "mxfp4":
+        want = dict(zip(("q4", "qs4"), quantize_mx(qd, pre, _lib.FMT_E2M1, out_rows=n_pad)))
+        want.update(zip(("k4", "ks4"), quantize_mx(kd, 1.0, _lib.FMT_E2M1, out_rows=n_pad, sub=km)))
+    else:
+        want = dict(zip(("q8", "qs8"), quantize_mx(qd, pre, fmt8, out_rows=n_pad)))
+        want.update(zip(("k8", "ks8"), quantize_mx(kd, 1.0, fmt8, out_rows=n_pad, sub=km)))
+    for name, t in want.items():
+        assert torch.equal(ops[name], t), name
+    for name in ("q4", "q8", "k4", "k8"):
+        assert (name in want) == (ops[name] is not None)
+    vt = torch.empty_like(ops["v_tiles"])
+    _lib.check(_lib.lib().mpsa_v_tiles(_lib.ptr(vd), _lib.dtype_id(dtype), 2, 2, N, D, _lib.strides4(vd), tile,
+                                       _lib.ptr(vt), _lib.stream_ptr(vd.device)))
+    assert torch.equal(ops["v_tiles"], vt)
+
+
 def test_fp16_inputs_nhd_layout_scale_and_public_entry():
     q, k, v = make_qkv(1, 4, 2, 256, 64, seed=44, dtype=torch.float16)
     want = O.attn_mx(q, k, v, tile=128, causal=True, mode="mxfp4", scale=0.2, out_dtype=torch.float16)
