@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the diagonal-tiled MXFP attention path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c1] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c1|c5] [--no-cpu-baseline]
 
 One "step" is one full pass of the hot path over one synthetic batch already resident in HBM:
 MX-quantize Q and K (E2M1 + E4M3 in one pass each), repack V, fused attention (diagonal tiles MXFP8,
@@ -40,11 +40,22 @@ WORKLOADS = {
     "c1": (1, 8, 8, 1024, 64, 64, 0, "C1 B1 H8 N1024 D64 causal tile64 diag"),
     "c3": (1, 32, 8, 8192, 128, 128, 2, "C3 llama3-8b prefill B1 Hq32 Hkv8 N8192 D128 causal tile128 diag(MXFP8)/offdiag(MXFP4), outlier channels"),
     "c4": (1, 32, 8, 131072, 128, 128, 3, "C4 long-context prefill B1 Hq32 Hkv8 N131072 D128 causal tile128 diag, outlier channels"),
+    "c5": (1, 40, 40, 32760, 128, 128, 4, "C5 video-DiT B1 H40 N32760 (21 frames x 1560) D128 non-causal tile128 diag, sigma 0.5 + per-frame offsets"),
 }
+NON_CAUSAL = {"c5"}
 
 
-def make_inputs(B, Hq, Hkv, N, D, seed, device):
+def make_inputs(B, Hq, Hkv, N, D, seed, device, dit_frames=0):
     g = torch.Generator(device=device).manual_seed(seed)
+    if dit_frames:
+        # video-DiT statistics: sigma 0.5 draws plus one offset per frame and channel on q and k
+        q = 0.5 * torch.randn(B, Hq, N, D, generator=g, device=device)
+        k = 0.5 * torch.randn(B, Hkv, N, D, generator=g, device=device)
+        v = 0.5 * torch.randn(B, Hkv, N, D, generator=g, device=device)
+        off = 0.5 * torch.randn(dit_frames, 1, D, generator=g, device=device)
+        q = (q.view(B, Hq, dit_frames, N // dit_frames, D) + off).view(B, Hq, N, D)
+        k = (k.view(B, Hkv, dit_frames, N // dit_frames, D) + off).view(B, Hkv, N, D)
+        return q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
     q = torch.randn(B, Hq, N, D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
     k = torch.randn(B, Hkv, N, D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
     v = torch.randn(B, Hkv, N, D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
@@ -57,10 +68,10 @@ def make_inputs(B, Hq, Hkv, N, D, seed, device):
     return q, k, v
 
 
-def composite_peak_tflops(nt):
-    """Bound when Q.K^T runs at the MXFP4 / MXFP8 peak (diagonal share 2/(nt+1) of the visited tiles) and
-    P.V at the bf16 peak: half of the FLOPs each."""
-    diag = 2.0 / (nt + 1)
+def composite_peak_tflops(nt, causal=True):
+    """Bound when Q.K^T runs at the MXFP4 / MXFP8 peak (diagonal share 2/(nt+1) of the visited tiles, 1/nt
+    without the causal mask) and P.V at the bf16 peak: half of the FLOPs each."""
+    diag = 2.0 / (nt + 1) if causal else 1.0 / nt
     t = 0.5 * ((1 - diag) / PEAK_FP4_TFLOPS + diag / PEAK_FP8_TFLOPS) + 0.5 / PEAK_BF16_TFLOPS
     return 1.0 / t
 
@@ -78,7 +89,7 @@ def time_events(fn, iters):
     return start.elapsed_time(stop) / iters
 
 
-def cpu_baseline(q, k, v, tile, D):
+def cpu_baseline(q, k, v, tile, D, causal=True):
     """The CPU oracle (a port of the reference's fake-quant path) on the first 8192 positions of the workload
     (all of it for C1/C3), every head."""
     import oracle as O
@@ -89,13 +100,13 @@ def cpu_baseline(q, k, v, tile, D):
     ks = k[:, :, :n].cpu()
     vs = v[:, :, :n].cpu()
     t0 = time.perf_counter()
-    O.attn_mx(qs, ks, vs, tile=tile, causal=True, mode="diag")
+    O.attn_mx(qs, ks, vs, tile=tile, causal=causal, mode="diag")
     dt = time.perf_counter() - t0
-    flops = 2.0 * qs.shape[0] * group * n * n * D
+    flops = (2.0 if causal else 4.0) * qs.shape[0] * group * n * n * D
     return {
         "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
         "sample": f"oracle.attn_mx (quantize+dequantize+tiled attention, torch CPU) on {group} query heads / {Hkv} KV heads, "
-                  f"N={n}, D={D}, causal, diag mode: {dt:.2f} s",
+                  f"N={n}, D={D}, {'causal' if causal else 'non-causal'}, diag mode: {dt:.2f} s",
         "seconds": dt,
     }
 
@@ -145,10 +156,11 @@ def run_only(args, device):
         info = {"kernel": "torch copy", "bytes_read": src.numel() * 2, "bytes_written": src.numel() * 2}
     elif args.only == "attn":
         B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
-        q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device)
+        causal = args.workload not in NON_CAUSAL
+        q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21)
         out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
         ops = prepare_operands(q, k, v, tile, "diag")
-        fn = lambda: attention_from_operands(ops, out, True)
+        fn = lambda: attention_from_operands(ops, out, causal)
         info = {"kernel": "attention", "workload": desc}
     elif args.only == "quant":
         B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
@@ -201,12 +213,13 @@ def main():
         run_only(args, device)
         return
     B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
-    q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device)
+    causal = args.workload not in NON_CAUSAL
+    q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21)
     out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
 
     def step():
         ops = prepare_operands(q, k, v, tile, "diag")
-        attention_from_operands(ops, out, True)
+        attention_from_operands(ops, out, causal)
 
     for _ in range(args.warmup):
         step()
@@ -217,21 +230,22 @@ def main():
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt * 1e3 / args.steps
-    flops = 2.0 * B * Hq * N * N * D
+    flops = (2.0 if causal else 4.0) * B * Hq * N * N * D
     tflops = flops / (ms_per_step * 1e-3) / 1e12
 
     # dominant kernel alone: the fused attention kernel on prepared operands
     ops = prepare_operands(q, k, v, tile, "diag")
-    attention_from_operands(ops, out, True)
+    attention_from_operands(ops, out, causal)
     torch.cuda.synchronize()
     k_iters = max(5, args.steps)
-    attn_ms = time_events(lambda: attention_from_operands(ops, out, True), k_iters)
+    attn_ms = time_events(lambda: attention_from_operands(ops, out, causal), k_iters)
     prep_ms = time_events(lambda: prepare_operands(q, k, v, tile, "diag"), k_iters)
     achieved = flops / (attn_ms * 1e-3) / 1e12
     nt = (N + tile - 1) // tile
-    comp = composite_peak_tflops(nt)
+    comp = composite_peak_tflops(nt, causal)
+    paired = causal and D == 128 and tile == 128 and N % 256 == 0
     roofline = {
-        "bound": "mfma", "kernel": "attn_pp_kernel (fused attention)", "achieved": round(achieved, 2), "peak": PEAK_FP4_TFLOPS,
+        "bound": "mfma", "kernel": ("attn_pp_kernel" if paired else "attn_fwd_kernel") + " (fused attention)", "achieved": round(achieved, 2), "peak": PEAK_FP4_TFLOPS,
         "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP4_TFLOPS, 5),
         "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get(args.workload),
         "kernel_ms": round(attn_ms, 4), "prepare_ms": round(prep_ms, 4),
@@ -252,7 +266,7 @@ def main():
     if not args.no_secondary:
         result["secondary"] = secondary(device, quick=args.steps < 10)
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(q, k, v, tile, D)
+        result["cpu_baseline"] = cpu_baseline(q, k, v, tile, D, causal)
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))
