@@ -131,17 +131,18 @@ int mpsa_quantize_setup(const void* x, int x_dtype, int64_t B, int64_t H, int64_
                         const void* sub, float pre, bool do4, int emax4, bool do8, int fmt8, int emax8,
                         uint8_t* c4, uint8_t* s4, uint8_t* c8, uint8_t* s8, int64_t out_rows, QuantArgs* out, unsigned* blocks) {
     *blocks = 0;
-    if (!x || !xs) return mpsa_fail(MPSA_EINVAL, "quantize: null input");
-    if ((do4 && (!c4 || !s4)) || (do8 && (!c8 || !s8))) return mpsa_fail(MPSA_EINVAL, "quantize: null output");
+    if (!xs) return mpsa_fail(MPSA_EINVAL, "quantize: null input");
     if (x_dtype != MPSA_BF16 && x_dtype != MPSA_F16) return mpsa_fail(MPSA_EINVAL, "quantize: x_dtype must be bf16 or f16");
     if (do8 && fmt8 != MPSA_FMT_E4M3 && fmt8 != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "quantize: 8-bit format must be E4M3 or E5M2");
     if (B < 0 || H < 0 || N < 0 || D <= 0 || out_rows < N) return mpsa_fail(MPSA_EINVAL, "quantize: bad shape");
     if (D % 32) return mpsa_fail(MPSA_EINVAL, "quantize: D=%lld is not a multiple of 32", (long long)D);
+    if (B == 0 || H == 0 || out_rows == 0) return MPSA_OK;                // nothing to write (pointers may be null)
+    if (!x && N > 0) return mpsa_fail(MPSA_EINVAL, "quantize: null input");
+    if ((do4 && (!c4 || !s4)) || (do8 && (!c8 || !s8))) return mpsa_fail(MPSA_EINVAL, "quantize: null output");
     if (xs[3] != 1) return mpsa_fail(MPSA_EINVAL, "quantize: last dim of x must be contiguous");
     if (!mpsa_aligned16(x) || (xs[0] % 8) || (xs[1] % 8) || (xs[2] % 8)) return mpsa_fail(MPSA_EALIGN, "quantize: x rows must be 16-byte aligned");
     if ((do4 && !mpsa_aligned16(c4)) || (do8 && !mpsa_aligned16(c8))) return mpsa_fail(MPSA_EALIGN, "quantize: outputs must be 16-byte aligned");
     if (sub && !mpsa_aligned16(sub)) return mpsa_fail(MPSA_EALIGN, "quantize: sub must be 16-byte aligned");
-    if (B == 0 || H == 0 || out_rows == 0) return MPSA_OK;
     const int64_t chunks = out_rows * (D / 8);
     if (chunks >= (int64_t(1) << 31) || H > 65535 || B > 65535) return mpsa_fail(MPSA_EUNSUPPORTED, "quantize: a head has too many elements, or too many heads");
     QuantArgs& a = *out;

@@ -93,6 +93,18 @@ def test_ragged_length_tail_masking(causal):
     _compare(got, want, f"ragged causal={causal}")
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("N,tile", [(1, 64), (31, 128), (65, 64), (129, 128), (257, 128)])
+def test_tiny_and_barely_ragged_lengths(N, tile, causal):
+    """Fewer keys than one tile, and one key more than a whole number of tiles (a last tile with a single row)."""
+    q, k, v = make_qkv(1, 2, 1, N, 64, seed=N)
+    for mode in ("diag", "mxfp4"):
+        got = _run(q, k, v, is_causal=causal, block_scale_type=mode, tile=tile, output_dtype=torch.float32)
+        assert got.shape == (1, 2, N, 64)
+        want = O.attn_mx(q, k, v, tile=tile, causal=causal, mode=mode, out_dtype=torch.float32)
+        _compare(got, want, f"N={N} tile={tile} causal={causal} {mode}")
+
+
 def test_c5_dit_shape_non_causal_ragged():
     """The video-DiT shape: N = 32760 = 255*128 + 120 keys/queries, D = 128, non-causal, sigma 0.5 draws plus a
     per-frame offset (21 frames of 1560 tokens) on q and k.  Two heads run on the GPU at full length (the

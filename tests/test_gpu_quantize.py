@@ -188,3 +188,14 @@ def test_c2_gemm_operand_full_size(fmt):
     for r0 in range(0, 8192, 2048):                       # oracle in slabs to bound host memory
         wc, ws = O.quantize_mx(a[r0:r0 + 2048], 1.0, fmt)
         assert torch.equal(codes[r0:r0 + 2048], wc) and torch.equal(scales[r0:r0 + 2048], ws)
+
+
+def test_empty_and_single_row_inputs():
+    """Zero heads / zero rows are accepted and write nothing; one row works."""
+    for shape in [(0, 2, 16, 64), (1, 0, 16, 64), (1, 2, 0, 64)]:
+        x = torch.empty(shape, dtype=torch.bfloat16, device=DEV)
+        codes, scales = quantize_mx(x, 1.0, O.FMT_E2M1)
+        assert codes.shape == (*shape[:3], 32) and scales.shape == (*shape[:3], 2)
+    x = torch.randn(1, 1, 1, 32).bfloat16()
+    _check(x, 1.0, O.FMT_E2M1)
+    _check(x, 1.0, O.FMT_E4M3, out_rows=5)
