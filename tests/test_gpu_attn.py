@@ -83,6 +83,25 @@ def test_full_size_properties():
     assert torch.equal(a[:, :, 0].cpu(), v[:, :, 0].repeat_interleave(4, dim=1))
 
 
+def test_long_context_properties():
+    """N = 131072 (B=1, Hq=4, Hkv=1 of the long-context shape: the kernel's work per head is the full one): V = 1
+    gives 1 everywhere, the first causal row returns V[0], and the last query tile (1024 key tiles deep) agrees with
+    the oracle run on that tile alone."""
+    N = 131072
+    g = torch.Generator(device=DEV).manual_seed(3)
+    q = torch.randn(1, 4, N, 128, generator=g, device=DEV).bfloat16()
+    k = torch.randn(1, 1, N, 128, generator=g, device=DEV).bfloat16()
+    v = torch.randn(1, 1, N, 128, generator=g, device=DEV).bfloat16()
+    o1 = mxfp_attn_kernel(q, k, torch.ones_like(v), is_causal=True, block_scale_type="diag", output_dtype=torch.float32)
+    assert (o1 - 1).abs().max().item() < 8e-3
+    del o1
+    o = mxfp_attn_kernel(q, k, v, is_causal=True, block_scale_type="diag", output_dtype=torch.bfloat16)
+    assert torch.equal(o[:, :, 0], v[:, :, 0].expand(1, 4, 128))
+    assert torch.isfinite(o.float()).all()
+    want = O.attn_mx(q[:, :1].cpu(), k.cpu(), v.cpu(), tile=128, causal=True, mode="diag", q_tiles=[N // 128 - 1])
+    _compare(o[:, :1, -128:], want, "last query tile of N=131072")
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_ragged_length_tail_masking(causal):
     """N = 1000 is not a multiple of the tile: the last key tile is masked, the last query rows are not stored."""
