@@ -188,7 +188,8 @@ int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, cons
  * mxfp_attn_kernel, ours/mxfp_attn.py:32, ours/mxfp_attn_kernel.py:272-297, with the key/value pointers advancing
  * past a skipped tile, which the reference's loop forgets): for query tile i, the statistic of key tile j is the mean
  * over the tile's valid query rows of the row maximum of S (after masking); tile 0 is always kept and sets the
- * reference value; tile j > 0 is kept iff stat(j) >= stat(0) * skip_thresh; a skipped tile contributes nothing.
+ * reference value; tile j > 0 is kept iff stat(j) >= stat(0) * skip_thresh, and the diagonal tile of a causal run is
+ * always kept (ours/online_routing.py:68-77: its stage starts a loop of its own); a skipped tile contributes nothing.
  * Arguments as mpsa_attn_fwd, mode MPSA_MODE_MXFP4 or MPSA_MODE_MXFP8 only (the rule's reference tile must be the
  * first one visited), plus
  *   skip_thresh   the factor above (scores are in log2 units with sm_scale folded in, as in the reference)

@@ -29,8 +29,8 @@ struct Geom {
 //
 // SKIP adds the reference's tile-skipping rule (ours/mxfp_attn_kernel.py:272-297): the statistic of a score tile
 // is the mean over its query rows of the row maximum; the first key tile (the "sink") is always kept and sets the
-// reference value, any later tile is kept only if its statistic is at least skip_thresh times the sink's.  A
-// skipped tile contributes nothing (no softmax, no P.V).  The statistic needs all rows of the tile, i.e. all
+// reference value, any later tile is kept only if its statistic is at least skip_thresh times the sink's (the
+// diagonal tile of a causal run is always kept as well).  A skipped tile contributes nothing (no softmax, no P.V).  The statistic needs all rows of the tile, i.e. all
 // waves: one extra workgroup barrier per tile, through a few floats of LDS behind the K/V buffers.
 template <int D, int TILE, int PVT, int FMT8, int MODE, bool SKIP>
 __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
@@ -268,8 +268,10 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
             for (int x = 0; x < G::NW; ++x) tot += sl[x];
             const float stat = tot / (float)min(TILE, a.n - i * TILE);
+            // the diagonal tile of a causal run is exempt like the sink: the reference walks it in a stage of its
+            // own, whose first tile is always kept (ours/online_routing.py:68-77, :87-112)
             if (t == 0) sink_stat = stat;
-            else keep = stat >= sink_stat * a.skip_thresh;
+            else keep = (a.causal && j == i) || stat >= sink_stat * a.skip_thresh;
             if (!keep) ++n_skipped;
         }
         v4i pk[G::KB][2];                               // 8 packed 16-bit values = one P^T operand

@@ -58,7 +58,8 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
     ``skip_thresh``: the reference's tile skipping (ours/mxfp_attn_kernel.py:272-297, with the pointer advance
     a skipped tile needs): the statistic of a score tile is the mean over its query rows of the row maximum; key
     tile 0 is always kept and sets the reference value, tile j > 0 is kept iff its statistic is at least
-    ``skip_thresh`` times that.  ``return_skipped`` adds an int32 ``[B, heads, tiles]`` count of skipped tiles;
+    ``skip_thresh`` times that; the diagonal tile of a causal run is always kept too (the reference's causal loop,
+    ours/online_routing.py:68-77, walks it as a stage of its own whose first tile is exempt).  ``return_skipped`` adds an int32 ``[B, heads, tiles]`` count of skipped tiles;
     a list passed as ``ratios_out`` collects statistic(j) / statistic(0) of every tile j > 0 examined."""
     B, Hq, N, D = q.shape
     Hkv = k.shape[1]
@@ -106,7 +107,8 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
                             sink = stat
                         elif ratios_out is not None:
                             ratios_out.append(float(stat / sink))
-                        if j > 0 and not bool(stat >= sink * skip_thresh):
+                        exempt = j == 0 or (causal and j == i)       # ours/online_routing.py:68-77: the diagonal stage's first tile
+                        if not exempt and not bool(stat >= sink * skip_thresh):
                             skipped[b, hi_, tile_list.index(i)] += 1
                             continue
                     m_new = torch.maximum(m, s.amax(dim=1))

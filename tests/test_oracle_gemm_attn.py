@@ -135,6 +135,8 @@ def test_tile_skipping_rule_against_a_dense_float64_restatement():
                 for j in range(1, last + 1):
                     keep[:, :, i, j] = stat[j] >= stat[0] * th
                 if causal:
+                    keep[:, :, i, i] = True           # the diagonal tile is exempt
+                if causal:
                     keep[:, :, i, i + 1:] = True      # not visited: already -inf
             mask = keep.repeat_interleave(tile, 2).repeat_interleave(tile, 3)
             p = torch.softmax(s.masked_fill(~mask, float("-inf")) * 0.6931471805599453, dim=-1)
