@@ -145,9 +145,9 @@ int mpsa_v_tiles(const void* v, int v_dtype, int64_t B, int64_t H, int64_t N, in
  * All operands of one attention call in ONE launch: Q quantized with pre_scale_q folded in, K quantized (minus
  * k_sub if given, see mpsa_quantize_mx), V repacked - the results are bit-identical to the separate calls
  * mpsa_quantize_mx(_dual) on q and k (emax 3 for E2M1, 7 for the 8-bit format) and mpsa_v_tiles on v, rows padded to
- * n_pad = ceil(N/tile)*tile.  Replaces the prologue of the reference's wrapper, ours/mxfp_attn_kernel.py:27-57.
+ * ceil(Nq/tile)*tile and ceil(Nk/tile)*tile.  Replaces the prologue of the reference's wrapper, ours/mxfp_attn_kernel.py:27-57.
  *
- *   q [B,Hq,N,D], k and v [B,Hkv,N,D] of dtype (MPSA_BF16 | MPSA_F16), element strides as for mpsa_quantize_mx
+ *   q [B,Hq,Nq,D], k and v [B,Hkv,Nk,D] of dtype (MPSA_BF16 | MPSA_F16), element strides as for mpsa_quantize_mx
  *   mode       MPSA_MODE_MXFP4: only the 4-bit outputs are written (8-bit pointers may be null),
  *              MPSA_MODE_MXFP8: only the 8-bit ones, MPSA_MODE_DIAG: both
  *   k_sub      NULL or [B,Hkv,D] (smooth-K mean from mpsa_seq_mean)
@@ -155,7 +155,7 @@ int mpsa_v_tiles(const void* v, int v_dtype, int64_t B, int64_t H, int64_t N, in
  */
 int mpsa_attn_prepare(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
                       const void* v, const int64_t v_strides[4], int dtype,
-                      int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int tile, int mode, int fmt8,
+                      int64_t B, int64_t Hq, int64_t Hkv, int64_t Nq, int64_t Nk, int64_t D, int tile, int mode, int fmt8,
                       float pre_scale_q, const void* k_sub,
                       uint8_t* q4, uint8_t* qs4, uint8_t* q8, uint8_t* qs8,
                       uint8_t* k4, uint8_t* ks4, uint8_t* k8, uint8_t* ks8, void* v_tiles, mpsa_stream_t stream);
@@ -165,22 +165,24 @@ int mpsa_attn_prepare(const void* q, const int64_t q_strides[4], const void* k, 
  * (ours/mxfp_attn_kernel.py:362-423, :103-359), with the causal tile structure and grouped-query
  * head mapping of ours/online_routing.py:68-77, :113-118, :160-171.
  *
- *   q4,qs4 / q8,qs8   Q codes + scales from the quantizer, rows padded to n_pad per head:
- *                     [B,Hq,n_pad,D/2],[B,Hq,n_pad,D/32] and [B,Hq,n_pad,D],[B,Hq,n_pad,D/32]
- *   k4,ks4 / k8,ks8   same for K with Hkv heads
+ *   q4,qs4 / q8,qs8   Q codes + scales from the quantizer, rows padded to nq_pad per head:
+ *                     [B,Hq,nq_pad,D/2],[B,Hq,nq_pad,D/32] and [B,Hq,nq_pad,D],[B,Hq,nq_pad,D/32]
+ *   k4,ks4 / k8,ks8   same for K with Hkv heads and nk_pad rows
  *                     (the 4-bit set may be null in MPSA_MODE_MXFP8, the 8-bit set in MPSA_MODE_MXFP4)
  *   fmt8              MPSA_FMT_E4M3 | MPSA_FMT_E5M2
  *   v_tiles           output of mpsa_v_tiles for the same tile, pv_dtype (MPSA_BF16 | MPSA_F16);
  *                     P is rounded to that dtype before P.V
- *   o                 [B,Hq,N,D] of o_dtype (MPSA_BF16 | MPSA_F16 | MPSA_F32), element strides o_strides[4],
+ *   o                 [B,Hq,nq,D] of o_dtype (MPSA_BF16 | MPSA_F16 | MPSA_F32), element strides o_strides[4],
  *                     last dim contiguous
- *   n                 valid sequence length, n_pad = ceil(n/tile)*tile
+ *   nq, nk            valid query and key/value counts, each padded to ceil(count/tile)*tile rows; the reference takes them
+ *                     separately as well (M and N of block_scaled_batched_attn, ours/mxfp_attn_kernel.py:362-371);
+ *                     causal masking and MPSA_MODE_DIAG need nq == nk
  *   tile              64 | 128 (score tile edge = precision granularity), D in {64,128}
  */
 int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
                   const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
                   const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
-                  int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                  int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t nk, int64_t D, int tile, int causal, int mode,
                   mpsa_stream_t stream);
 
 /*
@@ -198,7 +200,7 @@ int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, cons
 int mpsa_attn_fwd_skip(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
                        const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
                        const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
-                       int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                       int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t nk, int64_t D, int tile, int causal, int mode,
                        float skip_thresh, int32_t* skipped, mpsa_stream_t stream);
 
 #ifdef __cplusplus

@@ -8,7 +8,8 @@ struct AttnArgs {
     const void* v;
     void* o;
     int64_t o_sb, o_sh, o_sn;
-    int B, Hq, Hkv, n, n_pad, nt;
+    int B, Hq, Hkv, n, n_pad, nt;        // n, n_pad, nt: keys/values
+    int nq, nq_pad, ntq;                 // queries (equal to the above for self-attention)
     int causal, mode, fmt8, o_dtype;
     int d, tile;
     float skip_thresh;         // tile-skipping variants only

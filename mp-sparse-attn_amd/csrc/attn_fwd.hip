@@ -55,7 +55,7 @@ int launch_dt(const AttnArgs& a, int pv_dtype, hipStream_t st) {
 static int attn_entry(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
                       const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
                       const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
-                      int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                      int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal, int mode,
                       bool skip, float skip_thresh, int32_t* skipped, mpsa_stream_t stream) {
     if (mode != MPSA_MODE_MXFP4 && mode != MPSA_MODE_MXFP8 && mode != MPSA_MODE_DIAG) return mpsa_fail(MPSA_EINVAL, "attn: unknown mode %d", mode);
     const bool need4 = mode != MPSA_MODE_MXFP8, need8 = mode != MPSA_MODE_MXFP4;
@@ -65,20 +65,22 @@ static int attn_entry(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, 
     if (need8 && fmt8 != MPSA_FMT_E4M3 && fmt8 != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "attn: 8-bit format must be E4M3 or E5M2");
     if (pv_dtype != MPSA_BF16 && pv_dtype != MPSA_F16) return mpsa_fail(MPSA_EINVAL, "attn: pv_dtype must be bf16 or f16");
     if (o_dtype != MPSA_BF16 && o_dtype != MPSA_F16 && o_dtype != MPSA_F32) return mpsa_fail(MPSA_EINVAL, "attn: bad output dtype");
-    if (B <= 0 || Hq <= 0 || Hkv <= 0 || n <= 0 || Hq % Hkv) return mpsa_fail(MPSA_EINVAL, "attn: bad shape (B=%lld Hq=%lld Hkv=%lld n=%lld)", (long long)B, (long long)Hq, (long long)Hkv, (long long)n);
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || n <= 0 || nq <= 0 || Hq % Hkv) return mpsa_fail(MPSA_EINVAL, "attn: bad shape (B=%lld Hq=%lld Hkv=%lld nq=%lld nk=%lld)", (long long)B, (long long)Hq, (long long)Hkv, (long long)nq, (long long)n);
+    if (nq != n && (causal || mode == MPSA_MODE_DIAG)) return mpsa_fail(MPSA_EINVAL, "attn: causal masking and the diag mode need as many queries as keys (nq=%lld nk=%lld)", (long long)nq, (long long)n);
     if ((D != 64 && D != 128) || (tile != 64 && tile != 128)) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: D=%lld tile=%d (both must be 64 or 128)", (long long)D, tile);
     if (o_strides[3] != 1 || (o_strides[0] % 4) || (o_strides[1] % 4) || (o_strides[2] % 4)) return mpsa_fail(MPSA_EALIGN, "attn: output rows must be contiguous and 8-byte aligned");
     const uintptr_t al = reinterpret_cast<uintptr_t>(q4) | reinterpret_cast<uintptr_t>(q8) | reinterpret_cast<uintptr_t>(k4) |
                          reinterpret_cast<uintptr_t>(k8) | reinterpret_cast<uintptr_t>(v_tiles) | reinterpret_cast<uintptr_t>(o);
     const uintptr_t al4 = reinterpret_cast<uintptr_t>(qs4) | reinterpret_cast<uintptr_t>(qs8) | reinterpret_cast<uintptr_t>(ks4) | reinterpret_cast<uintptr_t>(ks8);
     if ((al & 15) || (al4 & 3)) return mpsa_fail(MPSA_EALIGN, "attn: operands must be 16-byte (codes, v, o) / 4-byte (scales) aligned");
-    const int64_t nt = (n + tile - 1) / tile;
-    if (B * Hq * nt >= (int64_t(1) << 31) || nt * tile >= (int64_t(1) << 30)) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: problem too large");
+    const int64_t nt = (n + tile - 1) / tile, ntq = (nq + tile - 1) / tile;
+    if (B * Hq * ntq >= (int64_t(1) << 31) || nt * tile >= (int64_t(1) << 30) || ntq * tile >= (int64_t(1) << 30)) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: problem too large");
     AttnArgs a;
     a.q4 = q4; a.qs4 = qs4; a.q8 = q8; a.qs8 = qs8; a.k4 = k4; a.ks4 = ks4; a.k8 = k8; a.ks8 = ks8;
     a.v = v_tiles; a.o = o;
     a.o_sb = o_strides[0]; a.o_sh = o_strides[1]; a.o_sn = o_strides[2];
     a.B = (int)B; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.n = (int)n; a.nt = (int)nt; a.n_pad = (int)(nt * tile);
+    a.nq = (int)nq; a.ntq = (int)ntq; a.nq_pad = (int)(ntq * tile);
     a.causal = causal ? 1 : 0; a.mode = mode; a.fmt8 = fmt8; a.o_dtype = o_dtype;
     a.d = (int)D; a.tile = tile;
     a.skip_thresh = skip_thresh; a.skipped = skipped;
@@ -105,17 +107,17 @@ static int attn_entry(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, 
 extern "C" int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
                              const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
                              const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
-                             int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                             int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal, int mode,
                              mpsa_stream_t stream) {
     return attn_entry(q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
-                      B, Hq, Hkv, n, D, tile, causal, mode, false, 0.0f, nullptr, stream);
+                      B, Hq, Hkv, nq, n, D, tile, causal, mode, false, 0.0f, nullptr, stream);
 }
 
 extern "C" int mpsa_attn_fwd_skip(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
                                   const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
                                   const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
-                                  int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                                  int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal, int mode,
                                   float skip_thresh, int32_t* skipped, mpsa_stream_t stream) {
     return attn_entry(q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
-                      B, Hq, Hkv, n, D, tile, causal, mode, true, skip_thresh, skipped, stream);
+                      B, Hq, Hkv, nq, n, D, tile, causal, mode, true, skip_thresh, skipped, stream);
 }

@@ -44,19 +44,19 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
 
     // ---- which (batch, kv head, query head, query tile) -- XCD-aware, heavy causal tiles first ----
     const int group = a.Hq / a.Hkv;
-    const int total = a.B * a.Hq * a.nt;
+    const int total = a.B * a.Hq * a.ntq;
     int L = blockIdx.x;
     if ((total & 7) == 0) L = (L & 7) * (total >> 3) + (L >> 3);      // XCD x gets one contiguous logical range
-    const int per_unit = group * a.nt;
+    const int per_unit = group * a.ntq;
     const int unit = L / per_unit;
     const int rem = L - unit * per_unit;
     const int rank = rem / group;
     const int hq = (unit % a.Hkv) * group + (rem - rank * group);
     const int b = unit / a.Hkv;
     const int kvh = unit % a.Hkv;
-    const int i = a.causal ? a.nt - 1 - rank : rank;
+    const int i = a.causal ? a.ntq - 1 - rank : rank;
 
-    const int64_t qhead_row = ((int64_t)b * a.Hq + hq) * a.n_pad;
+    const int64_t qhead_row = ((int64_t)b * a.Hq + hq) * a.nq_pad;
     const int64_t khead_row = ((int64_t)b * a.Hkv + kvh) * a.n_pad;
     const int q_local = 32 * w + r;
     const int64_t q_row = qhead_row + (int64_t)i * TILE + q_local;
@@ -258,7 +258,7 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         bool keep = true;
         if constexpr (SKIP) {
             // row maximum of S itself (st holds S - m_run), summed over the wave's valid queries, then over the waves
-            float sv = (i * TILE + q_local < a.n) ? mx + m_run : 0.0f;
+            float sv = (i * TILE + q_local < a.nq) ? mx + m_run : 0.0f;
 #pragma unroll
             for (int o = 1; o < 32; o <<= 1) sv += __shfl_xor(sv, o);
             float* sl = stat_lds + (t & 1) * G::NW;
@@ -267,7 +267,7 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
             float tot = 0.0f;
 #pragma unroll
             for (int x = 0; x < G::NW; ++x) tot += sl[x];
-            const float stat = tot / (float)min(TILE, a.n - i * TILE);
+            const float stat = tot / (float)min(TILE, a.nq - i * TILE);
             // the diagonal tile of a causal run is exempt like the sink: the reference walks it in a stage of its
             // own, whose first tile is always kept (ours/online_routing.py:68-77, :87-112)
             if (t == 0) sink_stat = stat;
@@ -366,13 +366,13 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
 
     if constexpr (SKIP) {
-        if (a.skipped && tid == 0) a.skipped[((int64_t)b * a.Hq + hq) * a.nt + i] = n_skipped;
+        if (a.skipped && tid == 0) a.skipped[((int64_t)b * a.Hq + hq) * a.ntq + i] = n_skipped;
     }
     // ---- epilogue: O = acc / l ; register e of lane (h, r): dim 32*db + 8*(e/4) + 4*h + e%4 of query r ----
     const float l_tot = sum_lane_pair(l_run);
     const float inv = 1.0f / l_tot;
     const int q_global = i * TILE + q_local;
-    if (q_global < a.n) {
+    if (q_global < a.nq) {
         uint8_t* orow = static_cast<uint8_t*>(a.o);
         const int64_t off = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh + (int64_t)q_global * a.o_sn;
 #pragma unroll
@@ -409,7 +409,7 @@ int launch_one(const AttnArgs& a, hipStream_t st) {
         if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "attn: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
         attr_set = true;
     }
-    dim3 grid((unsigned)(a.B * a.Hq * a.nt));
+    dim3 grid((unsigned)(a.B * a.Hq * a.ntq));
     hipLaunchKernelGGL(kern, grid, dim3(G::NT), smem, st, a);
     MPSA_CHECK_LAUNCH("attn");
     return MPSA_OK;

@@ -61,33 +61,33 @@ void launch_mode(const PrepArgs& p, int mode, int fmt8, int tile, int d, unsigne
 
 extern "C" int mpsa_attn_prepare(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
                                  const void* v, const int64_t v_strides[4], int dtype,
-                                 int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int tile, int mode, int fmt8,
+                                 int64_t B, int64_t Hq, int64_t Hkv, int64_t Nq, int64_t Nk, int64_t D, int tile, int mode, int fmt8,
                                  float pre_scale_q, const void* k_sub,
                                  uint8_t* q4, uint8_t* qs4, uint8_t* q8, uint8_t* qs8,
                                  uint8_t* k4, uint8_t* ks4, uint8_t* k8, uint8_t* ks8, void* v_tiles, mpsa_stream_t stream) {
     if (mode != MPSA_MODE_MXFP4 && mode != MPSA_MODE_MXFP8 && mode != MPSA_MODE_DIAG) return mpsa_fail(MPSA_EINVAL, "prepare: unknown mode %d", mode);
     if (tile != 64 && tile != 128) return mpsa_fail(MPSA_EUNSUPPORTED, "prepare: tile must be 64 or 128 (got %d)", tile);
-    if (B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || Hq % Hkv) return mpsa_fail(MPSA_EINVAL, "prepare: bad shape (B=%lld Hq=%lld Hkv=%lld N=%lld)", (long long)B, (long long)Hq, (long long)Hkv, (long long)N);
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Nq <= 0 || Nk <= 0 || Hq % Hkv) return mpsa_fail(MPSA_EINVAL, "prepare: bad shape (B=%lld Hq=%lld Hkv=%lld Nq=%lld Nk=%lld)", (long long)B, (long long)Hq, (long long)Hkv, (long long)Nq, (long long)Nk);
     const bool do4 = mode != MPSA_MODE_MXFP8, do8 = mode != MPSA_MODE_MXFP4;
-    const int64_t n_pad = (N + tile - 1) / tile * tile;
+    const int64_t nq_pad = (Nq + tile - 1) / tile * tile, nk_pad = (Nk + tile - 1) / tile * tile;
     constexpr int EMAX4 = 3, EMAX8 = 7;            // ours/quant_mxint8.py:303, :191
     if (mpsa_quantize_sw_encoders()) {
         // the cross-checking encoders exist only as stand-alone kernels
-        int rc = do4 && do8 ? mpsa_quantize_mx_dual(q, dtype, B, Hq, N, D, q_strides, nullptr, pre_scale_q, EMAX4, fmt8, EMAX8, q4, qs4, q8, qs8, n_pad, stream)
-                            : mpsa_quantize_mx(q, dtype, B, Hq, N, D, q_strides, nullptr, pre_scale_q, do4 ? MPSA_FMT_E2M1 : fmt8, do4 ? EMAX4 : EMAX8, do4 ? q4 : q8, do4 ? qs4 : qs8, n_pad, stream);
+        int rc = do4 && do8 ? mpsa_quantize_mx_dual(q, dtype, B, Hq, Nq, D, q_strides, nullptr, pre_scale_q, EMAX4, fmt8, EMAX8, q4, qs4, q8, qs8, nq_pad, stream)
+                            : mpsa_quantize_mx(q, dtype, B, Hq, Nq, D, q_strides, nullptr, pre_scale_q, do4 ? MPSA_FMT_E2M1 : fmt8, do4 ? EMAX4 : EMAX8, do4 ? q4 : q8, do4 ? qs4 : qs8, nq_pad, stream);
         if (rc != MPSA_OK) return rc;
-        rc = do4 && do8 ? mpsa_quantize_mx_dual(k, dtype, B, Hkv, N, D, k_strides, k_sub, 1.0f, EMAX4, fmt8, EMAX8, k4, ks4, k8, ks8, n_pad, stream)
-                        : mpsa_quantize_mx(k, dtype, B, Hkv, N, D, k_strides, k_sub, 1.0f, do4 ? MPSA_FMT_E2M1 : fmt8, do4 ? EMAX4 : EMAX8, do4 ? k4 : k8, do4 ? ks4 : ks8, n_pad, stream);
+        rc = do4 && do8 ? mpsa_quantize_mx_dual(k, dtype, B, Hkv, Nk, D, k_strides, k_sub, 1.0f, EMAX4, fmt8, EMAX8, k4, ks4, k8, ks8, nk_pad, stream)
+                        : mpsa_quantize_mx(k, dtype, B, Hkv, Nk, D, k_strides, k_sub, 1.0f, do4 ? MPSA_FMT_E2M1 : fmt8, do4 ? EMAX4 : EMAX8, do4 ? k4 : k8, do4 ? ks4 : ks8, nk_pad, stream);
         if (rc != MPSA_OK) return rc;
-        return mpsa_v_tiles(v, dtype, B, Hkv, N, D, v_strides, tile, v_tiles, stream);
+        return mpsa_v_tiles(v, dtype, B, Hkv, Nk, D, v_strides, tile, v_tiles, stream);
     }
     PrepArgs p;
     unsigned bq = 0, bk = 0, bv = 0;
-    int rc = mpsa_quantize_setup(q, dtype, B, Hq, N, D, q_strides, nullptr, pre_scale_q, do4, EMAX4, do8, fmt8, EMAX8, q4, qs4, q8, qs8, n_pad, &p.q, &bq);
+    int rc = mpsa_quantize_setup(q, dtype, B, Hq, Nq, D, q_strides, nullptr, pre_scale_q, do4, EMAX4, do8, fmt8, EMAX8, q4, qs4, q8, qs8, nq_pad, &p.q, &bq);
     if (rc != MPSA_OK) return rc;
-    rc = mpsa_quantize_setup(k, dtype, B, Hkv, N, D, k_strides, k_sub, 1.0f, do4, EMAX4, do8, fmt8, EMAX8, k4, ks4, k8, ks8, n_pad, &p.k, &bk);
+    rc = mpsa_quantize_setup(k, dtype, B, Hkv, Nk, D, k_strides, k_sub, 1.0f, do4, EMAX4, do8, fmt8, EMAX8, k4, ks4, k8, ks8, nk_pad, &p.k, &bk);
     if (rc != MPSA_OK) return rc;
-    rc = mpsa_v_tiles_setup(v, dtype, B, Hkv, N, D, v_strides, tile, v_tiles, &p.v, &bv);
+    rc = mpsa_v_tiles_setup(v, dtype, B, Hkv, Nk, D, v_strides, tile, v_tiles, &p.v, &bv);
     if (rc != MPSA_OK) return rc;
     const int64_t total = (int64_t)bq * Hq * B + (int64_t)(bk + bv) * Hkv * B;
     if (total >= (int64_t(1) << 31)) return mpsa_fail(MPSA_EUNSUPPORTED, "prepare: problem too large for one launch");

@@ -36,12 +36,12 @@ SIGNATURES = {
                                      _vp, _vp, _vp, _vp, _i64, _vp]),
     "mpsa_gemm_mx": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
     "mpsa_v_tiles": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _int, _vp, _vp]),
-    "mpsa_attn_prepare": (_int, [_vp, _p64, _vp, _p64, _vp, _p64, _int, _i64, _i64, _i64, _i64, _i64, _int, _int, _int,
+    "mpsa_attn_prepare": (_int, [_vp, _p64, _vp, _p64, _vp, _p64, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int,
                                  _f32, _vp] + [_vp] * 9 + [_vp]),
     "mpsa_attn_fwd": (_int, [_vp] * 8 + [_int, _vp, _int, _vp, _int, _p64,
-                             _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
+                             _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
     "mpsa_attn_fwd_skip": (_int, [_vp] * 8 + [_int, _vp, _int, _vp, _int, _p64,
-                                  _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _vp, _vp]),
+                                  _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _vp, _vp]),
 }
 
 _lib = None

@@ -16,16 +16,18 @@ _MODES = {"mxfp4": _lib.MODE_MXFP4, "mxfp8": _lib.MODE_MXFP8, "mxfp8e5": _lib.MO
 
 
 def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False):
-    """Quantize Q/K (K minus its mean over the sequence if ``smooth_k``) and repack V for one attention call.  q ``[B,Hq,N,D]``, k/v ``[B,Hkv,N,D]`` of one
-    16-bit dtype.  Returns a dict of device tensors (rows padded to whole tiles) the launcher consumes."""
+    """Quantize Q/K (K minus its mean over the sequence if ``smooth_k``) and repack V for one attention call.
+    q ``[B,Hq,Nq,D]``, k/v ``[B,Hkv,Nk,D]`` of one 16-bit dtype.  Returns a dict of device tensors (rows padded to
+    whole tiles) the launcher consumes."""
     if block_scale_type not in _MODES:
         raise ValueError(f"Invalid block scale type: {block_scale_type}")
     mode = _MODES[block_scale_type]
     fmt8 = _lib.FMT_E5M2 if block_scale_type.endswith("e5") else _lib.FMT_E4M3
-    B, Hq, N, D = q.shape
-    Hkv = k.shape[1]
+    B, Hq, Nq, D = q.shape
+    Hkv, N = k.shape[1], k.shape[2]
     nt = (N + tile - 1) // tile
     n_pad = nt * tile
+    nq_pad = (Nq + tile - 1) // tile * tile
     pre = pre_scale_q(D, scale)
     ops = {"mode": mode, "fmt8": fmt8, "tile": tile, "n": N, "q4": None, "qs4": None, "q8": None, "qs8": None,
            "k4": None, "ks4": None, "k8": None, "ks8": None}
@@ -36,29 +38,29 @@ def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False
     need4, need8 = mode != _lib.MODE_MXFP8, mode != _lib.MODE_MXFP4
     u8 = lambda *shape: torch.empty(shape, dtype=torch.uint8, device=dev)
     if need4:
-        ops["q4"], ops["qs4"] = u8(B, Hq, n_pad, D // 2), u8(B, Hq, n_pad, D // 32)
+        ops["q4"], ops["qs4"] = u8(B, Hq, nq_pad, D // 2), u8(B, Hq, nq_pad, D // 32)
         ops["k4"], ops["ks4"] = u8(B, Hkv, n_pad, D // 2), u8(B, Hkv, n_pad, D // 32)
     if need8:
-        ops["q8"], ops["qs8"] = u8(B, Hq, n_pad, D), u8(B, Hq, n_pad, D // 32)
+        ops["q8"], ops["qs8"] = u8(B, Hq, nq_pad, D), u8(B, Hq, nq_pad, D // 32)
         ops["k8"], ops["ks8"] = u8(B, Hkv, n_pad, D), u8(B, Hkv, n_pad, D // 32)
     v_tiles = torch.empty((B, Hkv, nt, tile * D), dtype=v.dtype, device=v.device)
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().mpsa_attn_prepare(
             _lib.ptr(q), _lib.strides4(q), _lib.ptr(k), _lib.strides4(k), _lib.ptr(v), _lib.strides4(v),
-            _lib.dtype_id(q.dtype), B, Hq, Hkv, N, D, tile, mode, fmt8, pre, _lib.ptr(kmean),
+            _lib.dtype_id(q.dtype), B, Hq, Hkv, Nq, N, D, tile, mode, fmt8, pre, _lib.ptr(kmean),
             _lib.ptr(ops["q4"]), _lib.ptr(ops["qs4"]), _lib.ptr(ops["q8"]), _lib.ptr(ops["qs8"]),
             _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]), _lib.ptr(ops["ks8"]),
             _lib.ptr(v_tiles), _lib.stream_ptr(dev)))
     ops["v_tiles"] = v_tiles
-    ops["shape"] = (B, Hq, Hkv, N, D)
+    ops["shape"] = (B, Hq, Hkv, Nq, N, D)
     return ops
 
 
 def attention_from_operands(ops, out, is_causal, skip_thresh=None, skipped=None):
-    """Launch ``mpsa_attn_fwd`` on prepared operands; ``out`` is a ``[B,Hq,N,D]`` view (last dim contiguous).
+    """Launch ``mpsa_attn_fwd`` on prepared operands; ``out`` is a ``[B,Hq,Nq,D]`` view (last dim contiguous).
     With ``skip_thresh`` the tile-skipping entry point runs instead (``skipped``: optional int32 ``[B,Hq,nt]``
     that receives the number of skipped key tiles per query tile)."""
-    B, Hq, Hkv, N, D = ops["shape"]
+    B, Hq, Hkv, Nq, N, D = ops["shape"]
     dev = out.device
     if skip_thresh is not None:
         with torch.cuda.device(dev):
@@ -66,7 +68,7 @@ def attention_from_operands(ops, out, is_causal, skip_thresh=None, skipped=None)
                 _lib.ptr(ops["q4"]), _lib.ptr(ops["qs4"]), _lib.ptr(ops["q8"]), _lib.ptr(ops["qs8"]),
                 _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]), _lib.ptr(ops["ks8"]), ops["fmt8"],
                 _lib.ptr(ops["v_tiles"]), _lib.dtype_id(ops["v_tiles"].dtype), _lib.ptr(out), _lib.dtype_id(out.dtype),
-                _lib.strides4(out), B, Hq, Hkv, N, D, ops["tile"], 1 if is_causal else 0, ops["mode"],
+                _lib.strides4(out), B, Hq, Hkv, Nq, N, D, ops["tile"], 1 if is_causal else 0, ops["mode"],
                 float(skip_thresh), _lib.ptr(skipped), _lib.stream_ptr(dev)))
         return out
     with torch.cuda.device(dev):
@@ -74,7 +76,7 @@ def attention_from_operands(ops, out, is_causal, skip_thresh=None, skipped=None)
             _lib.ptr(ops["q4"]), _lib.ptr(ops["qs4"]), _lib.ptr(ops["q8"]), _lib.ptr(ops["qs8"]),
             _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]), _lib.ptr(ops["ks8"]), ops["fmt8"],
             _lib.ptr(ops["v_tiles"]), _lib.dtype_id(ops["v_tiles"].dtype), _lib.ptr(out), _lib.dtype_id(out.dtype),
-            _lib.strides4(out), B, Hq, Hkv, N, D, ops["tile"], 1 if is_causal else 0, ops["mode"],
+            _lib.strides4(out), B, Hq, Hkv, Nq, N, D, ops["tile"], 1 if is_causal else 0, ops["mode"],
             _lib.stream_ptr(dev)))
     return out
 
@@ -115,7 +117,11 @@ def mxfp_attn_kernel(q, k, v, attn_mask=None, dropout_p=0.0,
     q, k, v = _as_bhnd(q, tensor_layout), _as_bhnd(k, tensor_layout), _as_bhnd(v, tensor_layout)
     B, Hq, N, D = q.shape
     assert D in [64, 128], "headdim should be in [64, 128]."
-    assert k.shape[2] == N and v.shape[2] == N, "q, k and v must have the same sequence length"
+    Nk = k.shape[2]
+    assert v.shape[2] == Nk, "k and v must have the same sequence length"
+    if Nk != N:                      # cross attention: the reference's kernel takes M and N apart as well
+        assert not is_causal, "causal masking needs q and k of the same sequence length"
+        assert _MODES.get(block_scale_type) != _lib.MODE_DIAG, "the diag types need q and k of the same sequence length"
     assert k.shape[1] == v.shape[1] and Hq % k.shape[1] == 0, "query heads must be a multiple of key/value heads"
     assert tile in (64, 128), "tile must be 64 or 128"
     if output_dtype not in (torch.float16, torch.bfloat16, torch.float32):
@@ -123,7 +129,7 @@ def mxfp_attn_kernel(q, k, v, attn_mask=None, dropout_p=0.0,
     if v.stride(-1) != 1:
         v = v.contiguous()
     ops = prepare_operands(q, k, v, tile, block_scale_type, scale, smooth_k=smooth_k)
-    nt = (N + tile - 1) // tile
+    nt, ntk = (N + tile - 1) // tile, (Nk + tile - 1) // tile       # query tiles, key tiles
     skipped = None
     if skip_thresh is not None and return_sparsity:
         skipped = torch.zeros((B, Hq, nt), dtype=torch.int32, device=q.device)
@@ -136,7 +142,7 @@ def mxfp_attn_kernel(q, k, v, attn_mask=None, dropout_p=0.0,
     if not return_sparsity:
         return out
     # share of the visited (query tile, key tile) pairs that were skipped
-    visited = B * Hq * (nt * (nt + 1) // 2 if is_causal else nt * nt)
+    visited = B * Hq * (nt * (nt + 1) // 2 if is_causal else nt * ntk)
     if skipped is None:
         return out, torch.zeros((), dtype=torch.float32, device=q.device)
     return out, skipped.sum().to(torch.float32) / visited

@@ -62,8 +62,9 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
     ours/online_routing.py:68-77, walks it as a stage of its own whose first tile is exempt).  ``return_skipped`` adds an int32 ``[B, heads, tiles]`` count of skipped tiles;
     a list passed as ``ratios_out`` collects statistic(j) / statistic(0) of every tile j > 0 examined."""
     B, Hq, N, D = q.shape
-    Hkv = k.shape[1]
+    Hkv, Nk = k.shape[1], k.shape[2]
     assert Hq % Hkv == 0
+    assert Nk == N or (not causal and mode != "diag"), "cross attention: non-causal, single precision"
     group = Hq // Hkv
     if smooth_k:
         k = _smooth_k(k)
@@ -74,6 +75,7 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
     ops = _prepare(q[:, head_list], k, mode, scale, fmt8)
     vf = v.to(torch.float32)
     nt = (N + tile - 1) // tile
+    ntk = (Nk + tile - 1) // tile
     tile_list = list(range(nt)) if q_tiles is None else list(q_tiles)
     starts, n_out = {}, 0
     for i in tile_list:
@@ -90,9 +92,9 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
                 m = torch.full((rows,), float("-inf"))
                 l = torch.zeros((rows,))
                 acc = torch.zeros((rows, D))
-                last = i if causal else nt - 1
+                last = i if causal else ntk - 1
                 for j in range(last + 1):
-                    c0, c1 = j * tile, min((j + 1) * tile, N)
+                    c0, c1 = j * tile, min((j + 1) * tile, Nk)
                     tag = "8" if _tile_is_8bit(mode, i, j) else "4"
                     qt = ops["q" + tag][b, hi_, r0:r1]
                     kt = ops["k" + tag][b, kvh, c0:c1]

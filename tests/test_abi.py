@@ -48,12 +48,14 @@ def test_host_side_argument_validation():
     assert L.mpsa_gemm_mx(one, one, one, one, 4, 256, 256, 128, one, 7, 256, null) == -1           # bad dtype
     assert L.mpsa_v_tiles(one, 0, 1, 1, 128, 96, st_ok, 128, one, null) == -3                      # D = 96
     so = (ctypes.c_int64 * 4)(128 * 128, 128 * 128, 128, 1)
-    args = [one] * 8 + [0, one, 0, one, 0, so, 1, 4, 3, 128, 128, 128, 1, 2, null]
+    args = [one] * 8 + [0, one, 0, one, 0, so, 1, 4, 3, 128, 128, 128, 128, 1, 2, null]
     assert L.mpsa_attn_fwd(*args) == -1                                                            # Hq % Hkv
-    args = [null] * 4 + [one] * 4 + [0, one, 0, one, 0, so, 1, 4, 2, 128, 128, 128, 1, 2, null]
+    args = [null] * 4 + [one] * 4 + [0, one, 0, one, 0, so, 1, 4, 2, 128, 128, 128, 128, 1, 2, null]
     assert L.mpsa_attn_fwd(*args) == -1                                                            # diag needs 4-bit Q
-    args = [one] * 8 + [0, one, 0, one, 0, so, 1, 4, 2, 128, 96, 128, 1, 2, null]
+    args = [one] * 8 + [0, one, 0, one, 0, so, 1, 4, 2, 128, 128, 96, 128, 1, 2, null]
     assert L.mpsa_attn_fwd(*args) == -3                                                            # D = 96
+    args = [one] * 8 + [0, one, 0, one, 0, so, 1, 4, 2, 128, 256, 128, 128, 1, 0, null]
+    assert L.mpsa_attn_fwd(*args) == -1                                                            # causal with nq != nk
     assert L.mpsa_e2m1_encode(null, 4, one, null) == -1
     assert L.mpsa_e2m1_encode(null, 0, null, null) == 0                                            # empty is fine
 

@@ -124,6 +124,29 @@ def test_tiny_and_barely_ragged_lengths(N, tile, causal):
         _compare(got, want, f"N={N} tile={tile} causal={causal} {mode}")
 
 
+@pytest.mark.parametrize("mode", ["mxfp4", "mxfp8"])
+@pytest.mark.parametrize("Nq,Nk,D,tile", [(300, 77, 128, 128), (64, 1000, 64, 64), (1024, 512, 128, 128), (130, 129, 64, 128)])
+def test_cross_attention_different_query_and_key_lengths(mode, Nq, Nk, D, tile):
+    """Non-causal attention of Nq queries over Nk keys (the reference's kernel takes M and N apart,
+    ours/mxfp_attn_kernel.py:362-371), grouped-query heads, ragged on both sides; with tile skipping as well."""
+    g = torch.Generator().manual_seed(Nq + Nk)
+    q = torch.randn(2, 4, Nq, D, generator=g).bfloat16()
+    k = torch.randn(2, 2, Nk, D, generator=g).bfloat16()
+    v = torch.randn(2, 2, Nk, D, generator=g).bfloat16()
+    got = _run(q, k, v, is_causal=False, block_scale_type=mode, tile=tile, output_dtype=torch.bfloat16)
+    assert got.shape == (2, 4, Nq, D)
+    want = O.attn_mx(q, k, v, tile=tile, causal=False, mode=mode)
+    _compare(got, want, f"cross {Nq}x{Nk} {mode}")
+    got_s, sp = _run(q, k, v, is_causal=False, block_scale_type=mode, tile=tile, output_dtype=torch.bfloat16,
+                     skip_thresh=-1e30, return_sparsity=True)
+    assert sp.item() == 0.0
+    _compare(got_s, want, "cross, skipping nothing")
+    with pytest.raises(AssertionError, match="same sequence length"):
+        _run(q, k, v, is_causal=True, block_scale_type=mode, tile=tile)
+    with pytest.raises(AssertionError, match="same sequence length"):
+        _run(q, k, v, is_causal=False, block_scale_type="diag", tile=tile)
+
+
 def test_c5_dit_shape_non_causal_ragged():
     """The video-DiT shape: N = 32760 = 255*128 + 120 keys/queries, D = 128, non-causal, sigma 0.5 draws plus a
     per-frame offset (21 frames of 1560 tokens) on q and k.  Two heads run on the GPU at full length (the
