@@ -63,6 +63,16 @@ int mpsa_e8m0_encode(const float* x, int64_t n, uint8_t* codes, mpsa_stream_t st
 int mpsa_e8m0_decode(const uint8_t* codes, int64_t n, float* out, mpsa_stream_t stream);
 
 /*
+ * Nibble packing of E2M1 codes along one dimension of a contiguous tensor seen as [outer, n, inner]:
+ * packed [outer, ceil(n/2), inner], element 2i in the low nibble and 2i+1 in the high one, an odd n padded with a
+ * zero code; unpack writes n codes back.  Replaces MXFP4Tensor.to_packed_tensor / unpack_packed_tensor,
+ * ours/mxfp.py:172-205, :207-236 (the quantizer itself already emits packed codes; these serve code tensors that
+ * arrive one code per byte, as the reference's quantizer leaves them).
+ */
+int mpsa_e2m1_pack(const uint8_t* codes, int64_t outer, int64_t n, int64_t inner, uint8_t* packed, mpsa_stream_t stream);
+int mpsa_e2m1_unpack(const uint8_t* packed, int64_t outer, int64_t n, int64_t inner, uint8_t* codes, mpsa_stream_t stream);
+
+/*
  * E8M0 scale re-layout between this library's linear form [batch, rows, K/32] and the 5-D packed form the
  * reference's block-scaled kernels consume, [batch, rows/128, K/128, 32, 4, 4] with
  * packed[cm][ck][r32][r4][c4] = linear[cm*128 + r4*32 + r32][ck*4 + c4].  Replaces the reshape/permute at

@@ -88,6 +88,39 @@ __global__ __launch_bounds__(256) void scale_layout_kernel(const uint32_t* src, 
     else           dst[boff + lin] = src[boff + w];
 }
 
+// Nibble packing along one dimension of a contiguous code tensor seen as [outer, n, inner]:
+// packed[o][i][x] = codes[o][2i][x] | codes[o][2i+1][x] << 4, an odd n padded with a zero code
+// (MXFP4Tensor.to_packed_tensor / unpack_packed_tensor, ours/mxfp.py:172-236).  One thread per packed byte.
+template <bool PACK>
+__global__ __launch_bounds__(256) void nibble_kernel(const uint8_t* src, uint8_t* dst, int64_t outer, int64_t n, int64_t inner) {
+    const int64_t np = (n + 1) / 2;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= outer * np * inner) return;
+    const int64_t x = idx % inner, i = (idx / inner) % np, o = idx / (inner * np);
+    const int64_t lo = (o * n + 2 * i) * inner + x, hi = lo + inner;
+    const bool has_hi = 2 * i + 1 < n;
+    if (PACK) {
+        dst[idx] = (uint8_t)((src[lo] & 0xF) | (has_hi ? (src[hi] & 0xF) << 4 : 0));
+    } else {
+        const uint8_t b = src[idx];
+        dst[lo] = b & 0xF;
+        if (has_hi) dst[hi] = b >> 4;
+    }
+}
+
+int nibble_run(const char* what, const uint8_t* src, int64_t outer, int64_t n, int64_t inner, uint8_t* dst, bool pack, hipStream_t st) {
+    if (outer < 0 || n < 0 || inner < 0) return mpsa_fail(MPSA_EINVAL, "%s: bad shape", what);
+    const int64_t total = outer * ((n + 1) / 2) * inner;
+    if (total == 0) return MPSA_OK;
+    if (!src || !dst) return mpsa_fail(MPSA_EINVAL, "%s: null pointer", what);
+    if (total >= (int64_t(1) << 39)) return mpsa_fail(MPSA_EUNSUPPORTED, "%s: tensor too large", what);
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (pack) hipLaunchKernelGGL(nibble_kernel<true>, grid, dim3(256), 0, st, src, dst, outer, n, inner);
+    else      hipLaunchKernelGGL(nibble_kernel<false>, grid, dim3(256), 0, st, src, dst, outer, n, inner);
+    MPSA_CHECK_LAUNCH(what);
+    return MPSA_OK;
+}
+
 int scale_layout(const char* what, const uint8_t* src, int64_t batch, int64_t rows, int64_t kblocks, uint8_t* dst,
                  bool to_packed, hipStream_t st) {
     if (batch <= 0 || rows <= 0 || kblocks <= 0) return mpsa_fail(MPSA_EINVAL, "%s: bad shape", what);
@@ -104,6 +137,13 @@ int scale_layout(const char* what, const uint8_t* src, int64_t batch, int64_t ro
 }
 
 }  // namespace
+
+extern "C" int mpsa_e2m1_pack(const uint8_t* codes, int64_t outer, int64_t n, int64_t inner, uint8_t* packed, mpsa_stream_t stream) {
+    return nibble_run("e2m1_pack", codes, outer, n, inner, packed, true, (hipStream_t)stream);
+}
+extern "C" int mpsa_e2m1_unpack(const uint8_t* packed, int64_t outer, int64_t n, int64_t inner, uint8_t* codes, mpsa_stream_t stream) {
+    return nibble_run("e2m1_unpack", packed, outer, n, inner, codes, false, (hipStream_t)stream);
+}
 
 extern "C" int mpsa_scales_to_5d(const uint8_t* linear, int64_t batch, int64_t rows, int64_t kblocks, uint8_t* packed, mpsa_stream_t stream) {
     return scale_layout("scales_to_5d", linear, batch, rows, kblocks, packed, true, (hipStream_t)stream);

@@ -27,6 +27,8 @@ SIGNATURES = {
     "mpsa_e2m1_decode": (_int, [_vp, _i64, _vp, _vp]),
     "mpsa_e8m0_encode": (_int, [_vp, _i64, _vp, _vp]),
     "mpsa_e8m0_decode": (_int, [_vp, _i64, _vp, _vp]),
+    "mpsa_e2m1_pack": (_int, [_vp, _i64, _i64, _i64, _vp, _vp]),
+    "mpsa_e2m1_unpack": (_int, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "mpsa_scales_to_5d": (_int, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "mpsa_scales_from_5d": (_int, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "mpsa_quantize_mx": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _vp, _f32, _int, _int, _vp, _vp, _i64, _vp]),

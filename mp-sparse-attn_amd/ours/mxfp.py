@@ -3,10 +3,11 @@
   * MXFP4Tensor   four-bit E2M1 data, one code per byte (``SEEM`` in the low nibble)
   * MXScaleTensor eight-bit E8M0 block scale factors
 
-Conversions run in HIP kernels of libmpsa (``mpsa_e2m1_encode`` ... ``mpsa_e8m0_decode``); packing
-along an arbitrary dimension is pure byte shuffling and stays in torch.  Tensors must live on the
-HIP device.
+Conversions and nibble packing run in HIP kernels of libmpsa (``mpsa_e2m1_encode`` ... ``mpsa_e8m0_decode``,
+``mpsa_e2m1_pack`` / ``mpsa_e2m1_unpack``).  Tensors must live on the HIP device.
 """
+
+import math
 
 import torch
 
@@ -66,25 +67,34 @@ class MXFP4Tensor:
 
     def to_packed_tensor(self, dim):
         """Two codes per byte along ``dim``: element 2i in the low nibble, 2i+1 in the high one; an
-        odd length is zero-padded (reference: ours/mxfp.py:172-205)."""
+        odd length is zero-padded (reference: ours/mxfp.py:172-205).  Runs ``mpsa_e2m1_pack``."""
         data = self.data
         assert 0 <= dim < data.ndim, "The dimension to pack along is not within the range of tensor dimensions"
+        _lib.require_device(data)
+        data = data.contiguous()
         n = data.size(dim)
-        if n % 2:
-            pad_shape = list(data.shape)
-            pad_shape[dim] = 1
-            data = torch.cat([data, torch.zeros(pad_shape, dtype=data.dtype, device=data.device)], dim=dim)
-        data = data.unflatten(dim, ((n + 1) // 2, 2))
-        return (data.select(dim + 1, 1) << 4) | data.select(dim + 1, 0)
+        outer = math.prod(data.shape[:dim])
+        inner = math.prod(data.shape[dim + 1:])
+        shape = list(data.shape)
+        shape[dim] = (n + 1) // 2
+        out = torch.empty(shape, dtype=torch.uint8, device=data.device)
+        with torch.cuda.device(data.device):
+            _lib.check(_lib.lib().mpsa_e2m1_pack(_lib.ptr(data), outer, n, inner, _lib.ptr(out), _lib.stream_ptr(data.device)))
+        return out
 
     def unpack_packed_tensor(self, packed_tensor, dim, original_shape):
-        """Inverse of :meth:`to_packed_tensor` (reference: ours/mxfp.py:207-236)."""
-        low = packed_tensor & 0xF
-        high = (packed_tensor >> 4) & 0xF
-        data = torch.stack((low, high), dim=dim + 1).flatten(dim, dim + 1)
-        if original_shape[dim] % 2:
-            data = data.narrow(dim, 0, original_shape[dim])
-        return data.type(torch.uint8)
+        """Inverse of :meth:`to_packed_tensor` (reference: ours/mxfp.py:207-236).  Runs ``mpsa_e2m1_unpack``."""
+        _lib.require_device(packed_tensor)
+        packed = packed_tensor.contiguous().view(torch.uint8)
+        original_shape = tuple(original_shape)
+        n = original_shape[dim]
+        assert packed.size(dim) == (n + 1) // 2, "packed tensor does not match the original shape"
+        outer = math.prod(original_shape[:dim])
+        inner = math.prod(original_shape[dim + 1:])
+        out = torch.empty(original_shape, dtype=torch.uint8, device=packed.device)
+        with torch.cuda.device(packed.device):
+            _lib.check(_lib.lib().mpsa_e2m1_unpack(_lib.ptr(packed), outer, n, inner, _lib.ptr(out), _lib.stream_ptr(packed.device)))
+        return out
 
 
 class MXScaleTensor:

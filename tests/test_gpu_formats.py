@@ -40,6 +40,22 @@ def test_e2m1_decode_pack_roundtrip():
         p = t.to_packed_tensor(dim)
         assert torch.equal(t.unpack_packed_tensor(p, dim, t.data.shape), t.data)
     assert torch.equal(t.to_packed_tensor(2).cpu(), O.pack_fp4(t.data.cpu()))
+    # literal cases: even and odd lengths, packing along the leading dimension
+    e = MXFP4Tensor(data=torch.arange(16, dtype=torch.uint8, device=DEV).reshape(2, 8), dtype=torch.uint8)
+    p = e.to_packed_tensor(dim=1)
+    assert p.tolist() == [[0x10, 0x32, 0x54, 0x76], [0x98, 0xBA, 0xDC, 0xFE]]
+    assert torch.equal(e.unpack_packed_tensor(p, 1, (2, 8)), e.data)
+    odd = MXFP4Tensor(data=torch.arange(6, dtype=torch.uint8, device=DEV).reshape(2, 3), dtype=torch.uint8)
+    po = odd.to_packed_tensor(dim=1)
+    assert po.tolist() == [[0x10, 0x02], [0x43, 0x05]]
+    assert torch.equal(odd.unpack_packed_tensor(po, 1, (2, 3)), odd.data)
+    p0 = e.to_packed_tensor(dim=0)
+    assert p0.shape == (1, 8) and p0[0, 3].item() == (11 << 4 | 3)
+    o3 = MXFP4Tensor(size=(3, 5, 7), device=DEV).random()
+    for dim in (0, 1, 2):
+        p = o3.to_packed_tensor(dim)
+        assert p.shape[dim] == (o3.data.shape[dim] + 1) // 2
+        assert torch.equal(o3.unpack_packed_tensor(p, dim, o3.data.shape), o3.data)
     assert torch.equal(MXFP4Tensor(data=t.to(torch.float32)).data, t.data & 0xF | (t.data & 8))
 
 
