@@ -27,6 +27,7 @@ typedef void* mpsa_stream_t;
 #define MPSA_BF16 0
 #define MPSA_F16  1
 #define MPSA_F32  2
+#define MPSA_F8E5M2 3   /* output of mpsa_gemm_mx only */
 
 /* MX element formats; the values are the CDNA4 scaled-MFMA format selectors */
 #define MPSA_FMT_E4M3 0
@@ -136,7 +137,9 @@ int mpsa_seq_mean(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, i
  *   a, b     packed codes [M,K/2] / [N,K/2] (E2M1) or [M,K] / [N,K] (8-bit), row-major, contiguous
  *   sa, sb   E8M0 bytes [M,K/32] / [N,K/32], row-major (the linear layout, not the 5-D packed one)
  *   fmt      element format of both operands
- *   c        [M,N] of c_dtype (MPSA_BF16 | MPSA_F16 | MPSA_F32), leading dimension ldc elements
+ *   c        [M,N] of c_dtype (MPSA_BF16 | MPSA_F16 | MPSA_F32 | MPSA_F8E5M2: one E5M2 byte per element, round to
+ *            nearest even, overflow to infinity - the reference's output dtypes are f32, f16 and e5m2,
+ *            ours/block_scaled_matmul.py:185-190, :273-280), leading dimension ldc elements
  *   M % 256 == 0, N % 256 == 0, K % 128 == 0
  */
 int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,

@@ -54,6 +54,24 @@ template <typename T> __device__ __forceinline__ T cvt_out(float v);
 template <> __device__ __forceinline__ float cvt_out<float>(float v) { return v; }
 template <> __device__ __forceinline__ __bf16 cvt_out<__bf16>(float v) { return (__bf16)v; }
 template <> __device__ __forceinline__ _Float16 cvt_out<_Float16>(float v) { return (_Float16)v; }
+// E5M2 output byte, round to nearest even, overflow to infinity (what a float32 -> float8_e5m2 cast does in torch;
+// the reference's kernel casts with c.to(tl.float8e5), ours/block_scaled_matmul.py:185-190)
+struct OutE5M2 { uint8_t b; };
+template <> __device__ __forceinline__ OutE5M2 cvt_out<OutE5M2>(float v) {
+    const uint32_t u = mpsa_f2u(v);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return OutE5M2{(uint8_t)(sign | 0x7Fu)};
+    uint32_t code;
+    if (a >= 0x38800000u) {                       // |v| >= 2^-14: normal
+        a += 0xFFFFFu + ((a >> 21) & 1u);
+        code = (a >> 21) - (112u << 2);
+        code = code > 0x7Cu ? 0x7Cu : code;
+    } else {                                      // subnormal, unit 2^-16
+        code = mpsa_f2u(mpsa_u2f(a) + 128.0f) - 0x43000000u;
+    }
+    return OutE5M2{(uint8_t)(sign | code)};
+}
 
 // Direct-to-LDS load written as inline assembly: lane L's BYTES bytes at gsrc land at lds_wave_base + L*BYTES
 // (M0 carries the wave-uniform LDS base).  The compiler's own builtin for this instruction makes it wait for
@@ -321,6 +339,7 @@ void launch_one(const GemmArgs& g, dim3 grid, hipStream_t st) {
 template <int FMT>
 void launch_fmt(const GemmArgs& g, int c_dtype, dim3 grid, hipStream_t st) {
     if (c_dtype == MPSA_BF16)      launch_one<FMT, __bf16>(g, grid, st);
+    else if (c_dtype == MPSA_F8E5M2) launch_one<FMT, OutE5M2>(g, grid, st);
     else if (c_dtype == MPSA_F16)  launch_one<FMT, _Float16>(g, grid, st);
     else                           launch_one<FMT, float>(g, grid, st);
 }
@@ -331,7 +350,7 @@ extern "C" int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, const uint8_t* 
                             int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
     if (!a || !sa || !b || !sb || !c) return mpsa_fail(MPSA_EINVAL, "gemm: null pointer");
     if (fmt != MPSA_FMT_E2M1 && fmt != MPSA_FMT_E4M3 && fmt != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "gemm: unknown format %d", fmt);
-    if (c_dtype != MPSA_BF16 && c_dtype != MPSA_F16 && c_dtype != MPSA_F32) return mpsa_fail(MPSA_EINVAL, "gemm: unsupported output dtype %d", c_dtype);
+    if (c_dtype != MPSA_BF16 && c_dtype != MPSA_F16 && c_dtype != MPSA_F32 && c_dtype != MPSA_F8E5M2) return mpsa_fail(MPSA_EINVAL, "gemm: unsupported output dtype %d", c_dtype);
     if (M <= 0 || N <= 0 || K <= 0 || ldc < N) return mpsa_fail(MPSA_EINVAL, "gemm: bad shape");
     if (M % BM || N % BN || K % 128) return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: M,N must be multiples of 256 and K of 128 (got %lld,%lld,%lld)", (long long)M, (long long)N, (long long)K);
     if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30) || (M / BM) * (N / BN) > (int64_t(1) << 30)) return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: shape too large");

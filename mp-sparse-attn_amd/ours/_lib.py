@@ -9,7 +9,7 @@ import os
 
 import torch
 
-BF16, F16, F32 = 0, 1, 2
+BF16, F16, F32, F8E5M2 = 0, 1, 2, 3
 FMT_E4M3, FMT_E5M2, FMT_E2M1 = 0, 1, 4
 MODE_MXFP4, MODE_MXFP8, MODE_DIAG = 0, 1, 2
 
@@ -86,6 +86,8 @@ def dtype_id(dtype):
         return F16
     if dtype == torch.float32:
         return F32
+    if dtype == torch.float8_e5m2:
+        return F8E5M2
     raise ValueError(f"unsupported dtype {dtype}")
 
 

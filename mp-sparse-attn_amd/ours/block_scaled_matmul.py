@@ -67,7 +67,7 @@ def block_scaled_matmul(a, a_scale, b, b_scale, dtype_dst, M, N, K, configs):
     """``C = (A o 2^(sa-127)) @ (B o 2^(sb-127))^T`` with float32 accumulation.
 
     Reference: ours/block_scaled_matmul.py:271-296 (ValueError for an unsupported output dtype, :280)."""
-    if dtype_dst not in (torch.float32, torch.float16, torch.bfloat16):
+    if dtype_dst not in (torch.float32, torch.float16, torch.bfloat16, torch.float8_e5m2):
         raise ValueError(f"Unsupported dtype: {dtype_dst}")
     fmt = _fmt_of(configs)
     _lib.require_device(a, a_scale, b, b_scale)

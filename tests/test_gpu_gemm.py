@@ -145,3 +145,20 @@ def test_scale_5d_layout_and_matmul_with_packed_scales():
     assert torch.equal(c_lin, c_pk)
     with pytest.raises(RuntimeError, match="multiple of 128"):
         pack_scale_5d(lin[:, :, :100].contiguous().to(DEV))
+
+
+def test_e5m2_output_dtype():
+    """The reference's third output dtype (ours/block_scaled_matmul.py:185-190): every byte equals torch's own
+    float32 -> float8_e5m2 cast of the kernel's float32 result, overflow to infinity included."""
+    M, N, K = 256, 256, 512
+    g = torch.Generator().manual_seed(21)
+    a = (torch.randn(M, K, generator=g) * 8).bfloat16()
+    b = (torch.randn(N, K, generator=g) * 8).bfloat16()
+    a[0] *= 64                                                   # one row large enough to overflow E5M2 (57344)
+    ac, asc, bc, bsc, cfg = initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), "mxfp4")
+    c32 = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg)
+    c8 = block_scaled_matmul(ac, asc, bc, bsc, torch.float8_e5m2, M, N, K, cfg)
+    assert c8.dtype == torch.float8_e5m2
+    want = c32.cpu().to(torch.float8_e5m2)
+    assert torch.equal(c8.cpu().view(torch.uint8), want.view(torch.uint8))
+    assert torch.isinf(want.float()).any() and (want.float().abs() < 1).any()
