@@ -146,6 +146,17 @@ int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const ui
                  int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream);
 
 /*
+ * The same product for every (batch, head): a [batch,heads_a,M,K'] and sa [batch,heads_a,M,K/32], b
+ * [batch,heads_b,N,K'] and sb likewise, c [batch,heads_a,M,ldc], all contiguous; head h of a multiplies head
+ * h / (heads_a/heads_b) of b (grouped heads; heads_a % heads_b == 0).  Replaces block_scaled_batched_matmul and its
+ * Triton kernel (ours/batched_block_scaled_matmul.py:183-236, :43-180) - the batched Q.K^T of the reference's
+ * mxfp_attn (ours/mxfp_attn.py:64-66) - with the 2-D kernel's semantics.
+ */
+int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
+                         int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
+                         void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream);
+
+/*
  * Value-tile repack: v [B,H,N,D] (bf16 | f16, strided, last dim contiguous) -> v_tiles
  * [B,H,ceil(N/tile),tile*D] of the same dtype in matrix-core operand order, keys past N zero.
  * Replaces the dtype normalisation / .contiguous() of V in the reference wrapper

@@ -48,6 +48,7 @@ struct GemmArgs {
     void* c;
     int64_t ldc;
     int M, N, K;
+    int heads_a, heads_b;      // batched runs: blockIdx.y = batch * heads_a + head; B's head is head / (heads_a / heads_b)
 };
 
 template <typename T> __device__ __forceinline__ T cvt_out(float v);
@@ -125,6 +126,14 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
 
     // ---- direct-to-LDS staging: wave w moves chunks [4w, 4w+4) x 1 KiB of either operand and the scale bytes
     //      of rows [64w, 64w+64); chunk position p = row*4 + slot holds row's 16-byte piece slot ^ ((row>>2)&3)
+    // batched runs (blockIdx.y): operands of this batch entry; grouped heads share a B operand
+    const int bz = blockIdx.y;
+    const int bb = bz / g.heads_a, ha = bz - bb * g.heads_a;
+    const int64_t zb = (int64_t)bb * g.heads_b + ha / (g.heads_a / g.heads_b);
+    g.a += (int64_t)bz * g.M * row_bytes;
+    g.sa += (int64_t)bz * g.M * srow_bytes;
+    g.b += zb * g.N * row_bytes;
+    g.sb += zb * g.N * srow_bytes;
     const uint8_t* ga[4];
     const uint8_t* gb[4];
 #pragma unroll
@@ -305,7 +314,7 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
 
     // epilogue: accumulator register e of lane (h, r) is C[8*(e/4) + 4*h + e%4][r] of its 32x32 block
-    OutT* c = static_cast<OutT*>(g.c);
+    OutT* c = static_cast<OutT*>(g.c) + (int64_t)bz * g.M * g.ldc;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -346,24 +355,33 @@ void launch_fmt(const GemmArgs& g, int c_dtype, dim3 grid, hipStream_t st) {
 
 }  // namespace
 
-extern "C" int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
-                            int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
+extern "C" int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
+                                    int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
+                                    void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
     if (!a || !sa || !b || !sb || !c) return mpsa_fail(MPSA_EINVAL, "gemm: null pointer");
     if (fmt != MPSA_FMT_E2M1 && fmt != MPSA_FMT_E4M3 && fmt != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "gemm: unknown format %d", fmt);
     if (c_dtype != MPSA_BF16 && c_dtype != MPSA_F16 && c_dtype != MPSA_F32 && c_dtype != MPSA_F8E5M2) return mpsa_fail(MPSA_EINVAL, "gemm: unsupported output dtype %d", c_dtype);
     if (M <= 0 || N <= 0 || K <= 0 || ldc < N) return mpsa_fail(MPSA_EINVAL, "gemm: bad shape");
+    if (batch <= 0 || heads_a <= 0 || heads_b <= 0 || heads_a % heads_b) return mpsa_fail(MPSA_EINVAL, "gemm: bad batch shape (batch=%lld heads_a=%lld heads_b=%lld)", (long long)batch, (long long)heads_a, (long long)heads_b);
     if (M % BM || N % BN || K % 128) return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: M,N must be multiples of 256 and K of 128 (got %lld,%lld,%lld)", (long long)M, (long long)N, (long long)K);
-    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30) || (M / BM) * (N / BN) > (int64_t(1) << 30)) return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: shape too large");
+    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30) || (M / BM) * (N / BN) > (int64_t(1) << 30) || batch * heads_a > 65535)
+        return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: shape too large");
     if (!mpsa_aligned16(a) || !mpsa_aligned16(b) || (reinterpret_cast<uintptr_t>(sa) & 3) || (reinterpret_cast<uintptr_t>(sb) & 3))
         return mpsa_fail(MPSA_EALIGN, "gemm: codes must be 16-byte and scales 4-byte aligned");
     GemmArgs g;
     g.a = a; g.sa = sa; g.b = b; g.sb = sb; g.c = c; g.ldc = ldc;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
-    dim3 grid((unsigned)((M / BM) * (N / BN)));
+    g.heads_a = (int)heads_a; g.heads_b = (int)heads_b;
+    dim3 grid((unsigned)((M / BM) * (N / BN)), (unsigned)(batch * heads_a));
     hipStream_t st = (hipStream_t)stream;
     if (fmt == MPSA_FMT_E2M1)      launch_fmt<MPSA_FMT_E2M1>(g, c_dtype, grid, st);
     else if (fmt == MPSA_FMT_E4M3) launch_fmt<MPSA_FMT_E4M3>(g, c_dtype, grid, st);
     else                           launch_fmt<MPSA_FMT_E5M2>(g, c_dtype, grid, st);
     MPSA_CHECK_LAUNCH("gemm");
     return MPSA_OK;
+}
+
+extern "C" int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
+                            int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
+    return mpsa_gemm_mx_batched(a, sa, b, sb, fmt, 1, 1, 1, M, N, K, c, c_dtype, ldc, stream);
 }

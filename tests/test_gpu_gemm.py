@@ -15,6 +15,7 @@ import pytest
 import torch
 
 import oracle as O
+from conftest import make_qkv
 from ours import _lib
 from ours.block_scaled_matmul import block_scaled_matmul, initialize_block_scaled_from_tensor, make_configs
 from ours.mxfp import MXFP4Tensor, MXScaleTensor
@@ -162,3 +163,32 @@ def test_e5m2_output_dtype():
     want = c32.cpu().to(torch.float8_e5m2)
     assert torch.equal(c8.cpu().view(torch.uint8), want.view(torch.uint8))
     assert torch.isinf(want.float()).any() and (want.float().abs() < 1).any()
+
+
+@pytest.mark.parametrize("bst", ["mxfp4", "mxfp8", "mxfp8e5"])
+def test_batched_matmul_scores_with_grouped_heads(bst):
+    """block_scaled_batched_matmul on attention-shaped operands (K = head dim 128): every (batch, head) slice
+    equals the 2-D entry point's result bit for bit, grouped heads read the right B slice, and the scores match
+    the oracle; the reference's packed 5-D scales are accepted."""
+    from ours.batched_block_scaled_matmul import block_scaled_batched_matmul
+    from ours.block_scaled_matmul import pack_scale_5d
+    from ours.quant_mxint8 import quantize_mx
+    B, H, Hkv, M, N, K = 2, 4, 2, 512, 256, 128
+    q, k, _ = make_qkv(B, H, Hkv, M, K, seed=5)
+    k = k[:, :, :N]
+    cfg = make_configs(bst)
+    fmt = {"mxfp4": O.FMT_E2M1, "mxfp8": O.FMT_E4M3, "mxfp8e5": O.FMT_E5M2}[bst]
+    qc, qs = quantize_mx(q.to(DEV), O.q_pre_scale(K), fmt)
+    kc, ks = quantize_mx(k.contiguous().to(DEV), 1.0, fmt)
+    got = block_scaled_batched_matmul(qc, qs, kc, ks, torch.float32, B, H, M, N, K, cfg)
+    assert got.shape == (B, H, M, N)
+    for b in range(B):
+        for h in range(H):
+            one = block_scaled_matmul(qc[b, h], qs[b, h], kc[b, h // 2], ks[b, h // 2], torch.float32, M, N, K, cfg)
+            assert torch.equal(got[b, h], one)
+    want = O.gemm_mx(qc.cpu(), qs.cpu(), kc.cpu().repeat_interleave(2, dim=1), ks.cpu().repeat_interleave(2, dim=1), fmt)
+    mag = O.gemm_mx(qc.cpu(), qs.cpu(), kc.cpu().repeat_interleave(2, dim=1), ks.cpu().repeat_interleave(2, dim=1), fmt,
+                    acc_dtype=torch.float64).abs()
+    assert ((got.cpu() - want).abs() <= 1e-3 * want.abs() + 3e-5 * mag.float().amax()).all()
+    got5 = block_scaled_batched_matmul(qc, pack_scale_5d(qs), kc, pack_scale_5d(ks), torch.float32, B, H, M, N, K, cfg)
+    assert torch.equal(got5, got)
