@@ -6,6 +6,7 @@ Modules keep the reference's names so that ``from ours.mxfp_attn import mxfp_att
   ours.mxfp                  format helper classes            (reference: ours/mxfp.py)
   ours.quant_mxint8          MX quantizer entry points        (reference: ours/quant_mxint8.py)
   ours.block_scaled_matmul   block-scaled GEMM                (reference: ours/block_scaled_matmul.py)
+  ours.batched_block_scaled_matmul  batched block-scaled GEMM (reference: ours/batched_block_scaled_matmul.py)
   ours.mxfp_attn_kernel      fused attention                  (reference: ours/mxfp_attn_kernel.py)
   ours.mxfp_attn             public attention entry           (reference: ours/mxfp_attn.py)
 
