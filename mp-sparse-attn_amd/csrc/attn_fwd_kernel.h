@@ -402,13 +402,10 @@ template <int D, int TILE, int PVT, int FMT8, int MODE, bool SKIP = false>
 int launch_one(const AttnArgs& a, hipStream_t st) {
     typedef Geom<D, TILE> G;
     constexpr int smem = G::SMEM + (SKIP ? 2 * G::NW * (int)sizeof(float) : 0);
-    static bool attr_set = false;      // idempotent; a race only repeats the same call
+    static bool reserved[MPSA_MAX_DEVICES] = {};
     auto kern = attn_fwd_kernel<D, TILE, PVT, FMT8, MODE, SKIP>;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "attn: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
-        attr_set = true;
-    }
+    const hipError_t e = mpsa_reserve_lds(reinterpret_cast<const void*>(kern), smem, reserved);
+    if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "attn: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
     dim3 grid((unsigned)(a.B * a.Hq * a.ntq));
     hipLaunchKernelGGL(kern, grid, dim3(G::NT), smem, st, a);
     MPSA_CHECK_LAUNCH("attn");

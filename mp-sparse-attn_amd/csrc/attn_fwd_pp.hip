@@ -342,13 +342,10 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
 
 template <int PVT, int FMT8, int MODE>
 int launch_pp(const AttnArgs& a, hipStream_t st) {
-    static bool attr_set = false;      // idempotent; a race only repeats the same call
+    static bool reserved[MPSA_MAX_DEVICES] = {};
     auto kern = attn_pp_kernel<PVT, FMT8, MODE>;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
-        if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "attn: cannot reserve %d bytes of LDS: %s", SMEM, hipGetErrorString(e));
-        attr_set = true;
-    }
+    const hipError_t e = mpsa_reserve_lds(reinterpret_cast<const void*>(kern), SMEM, reserved);
+    if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "attn: cannot reserve %d bytes of LDS: %s", SMEM, hipGetErrorString(e));
     dim3 grid((unsigned)(a.B * a.Hq * (a.nt / 2)));
     hipLaunchKernelGGL(kern, grid, dim3(512), SMEM, st, a);
     MPSA_CHECK_LAUNCH("attn(pp)");

@@ -330,12 +330,10 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
 
 template <int FMT, typename OutT, bool WIDE>
 void launch_kernel(const GemmArgs& g, dim3 grid, hipStream_t st) {
-    static bool attr_set = false;      // idempotent; a race only repeats the same call
+    static bool reserved[MPSA_MAX_DEVICES] = {};
     auto kern = gemm_mx_kernel<FMT, OutT, WIDE>;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes<WIDE>());
-        attr_set = true;
-    }
+    // a failure here shows up as a launch error, which the caller reports
+    (void)mpsa_reserve_lds(reinterpret_cast<const void*>(kern), smem_bytes<WIDE>(), reserved);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem_bytes<WIDE>(), st, g);
 }
 

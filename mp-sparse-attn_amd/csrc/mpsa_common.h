@@ -19,6 +19,20 @@ int mpsa_fail(int code, const char* fmt, ...);
 
 static inline bool mpsa_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Kernels that need more dynamic LDS than the default limit get the function attribute once per device (the
+// attribute is per device); `done` is a per-kernel array of MPSA_MAX_DEVICES flags.  A race only repeats the call.
+#define MPSA_MAX_DEVICES 64
+static inline hipError_t mpsa_reserve_lds(const void* kern, int bytes, bool* done) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= MPSA_MAX_DEVICES) return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (done[dev]) return hipSuccess;
+    e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done[dev] = true;
+    return e;
+}
+
 #define MPSA_CHECK_LAUNCH(what)                                                        \
     do {                                                                               \
         hipError_t e__ = hipGetLastError();                                            \
