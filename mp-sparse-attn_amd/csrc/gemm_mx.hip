@@ -199,20 +199,23 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
 
     // One matrix-instruction step's operands: 4 + 4 fragments and their scale bytes.  Two sets alternate: while
     // the 16 instructions of one set run, the LDS reads of the next set are in flight.
-    struct Frag { v8i a[4], b[4]; int sa[4], sb[4]; };
+    // Scale bytes: the four bytes of a row's aligned scale word cover an even step and the odd step after it
+    // (bytes h and 2+h of the lane half h).  The word is read once, with the even step's operands, shifted right by
+    // 8h when that step starts, and handed on to the odd step's set, whose instructions select byte 2.
+    struct Frag { v8i a[4], b[4]; int sa[4], sb[4]; uint32_t ra[4], rb[4]; };
 
     // reads operands of step s of stage kt out of the ring: part 0 the B fragments and their scale bytes,
     // part 1 the A fragments and theirs
-    auto read_part = [&](Frag& f, int kt, int s, int part) __attribute__((always_inline)) {
+    auto read_part = [&](Frag& f, const Frag& even, int kt, int s, int part, bool fresh) __attribute__((always_inline)) {
         const uint8_t* st = smem + (kt % NSTAGE) * STAGE_BYTES;
-        // the lane's scale byte of this step: byte 2s+h of the stage's four (4-bit codes), byte h of its two (8-bit)
+        // the row's scale word of this step pair
         const uint8_t* sc;
         int sstride;
         if constexpr (WIDE) {
-            sc = scg + ((kt / GROUP) & 1) * 2 * SCG_BYTES + (FP4 ? 4 * (kt % GROUP) + 2 * s + h : 2 * (kt % GROUP) + h);
+            sc = scg + ((kt / GROUP) & 1) * 2 * SCG_BYTES + 4 * (FP4 ? kt % GROUP : (kt % GROUP) >> 1);
             sstride = 16;
         } else {
-            sc = st + 2 * OP_BYTES + (FP4 ? 2 * s + h : 2 * (kt & 1) + h);
+            sc = st + 2 * OP_BYTES;
             sstride = 4;
         }
         const bool isb = part == 0;
@@ -222,9 +225,12 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         for (int i = 0; i < 4; ++i) {
             const int row = (isb ? wn : wm) * 128 + i * 32 + r;
             const int off = isb ? offb[i] : offa[i], swz = isb ? swz_b[i] : swz_a[i];
-            int& fs = isb ? f.sb[i] : f.sa[i];
             v8i& fx = isb ? f.b[i] : f.a[i];
-            fs = sc[row * sstride];
+            if (fresh) {
+                (isb ? f.rb[i] : f.ra[i]) = *reinterpret_cast<const uint32_t*>(sc + row * sstride);
+            } else {
+                if (isb) f.sb[i] = even.sb[i]; else f.sa[i] = even.sa[i];
+            }
             if constexpr (FP4) {
                 const v4i x = *reinterpret_cast<const v4i*>(lx + off + (((2 * s + h) ^ swz) * 16));
                 fx = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
@@ -238,17 +244,27 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         }
     };
     // the four matrix instructions of accumulator row i
-    auto multiply_row = [&](const Frag& f, int i) __attribute__((always_inline)) {
+    auto multiply_row = [&](const Frag& f, int i, bool odd) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)   // op_sel 0: the lane's scale byte was read into bits 7:0
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMT, 0, f.sa[i], 0, f.sb[j]);
+        for (int j = 0; j < 4; ++j) {
+            if (odd) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMT, 2, f.sa[i], 2, f.sb[j]);
+            else     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMT, 0, f.sa[i], 0, f.sb[j]);
+        }
     };
     // One step: the 16 matrix instructions on operand set `cur`, in four rows.  Between them go the LDS reads
     // that fill the other set `nxt` with step ns of stage nkt (rows 0 and 1) and, when `refill` is set, the
     // loads of stage lkt into the buffer of stage lkt-NSTAGE (two per row; on the wide path the first stage of
     // a group also brings the next group's scale bytes), so that the matrix pipe keeps running while they issue.
-    auto step = [&](const Frag& cur, Frag& nxt, int nkt, int ns, bool refill, int lkt) __attribute__((always_inline)) {
+    // `odd`: cur is the odd step of its pair (its scale words were handed on by the even step's set)
+    auto step = [&](Frag& cur, Frag& nxt, int nkt, int ns, bool refill, int lkt, bool odd) __attribute__((always_inline)) {
         constexpr int PER = FP4 ? 2 : 3;                   // LDS reads issued behind each matrix instruction
+        if (!odd) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                cur.sa[i] = (int)(cur.ra[i] >> (8 * h));
+                cur.sb[i] = (int)(cur.rb[i] >> (8 * h));
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             if (refill) {
@@ -258,8 +274,8 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (i < 2) read_part(nxt, nkt, ns, i);
-            multiply_row(cur, i);
+            if (i < 2) read_part(nxt, cur, nkt, ns, i, odd);          // the step after an odd one starts a new pair
+            multiply_row(cur, i, odd);
             if (i < 2) {
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -292,23 +308,23 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
     }
-    read_part(f0, 0, 0, 0);
-    read_part(f0, 0, 0, 1);
+    read_part(f0, f0, 0, 0, 0, true);
+    read_part(f0, f0, 0, 0, 1, true);
     if constexpr (FP4) {
         // a stage is two steps: the second step's operands load under the first step's instructions, and the
         // next stage's first operands (after the barrier that publishes it) under the second step's
         for (int kt = 0; kt < KT; ++kt) {
-            step(f0, f1, kt, 1, false, 0);
+            step(f0, f1, kt, 1, false, 0, false);
             publish();
-            step(f1, f0, kt + 1, 0, true, kt + NSTAGE);
+            step(f1, f0, kt + 1, 0, true, kt + NSTAGE, true);
         }
     } else {
         // a stage is one step; two stages per trip so that the two operand sets keep their registers
         for (int kt = 0; kt < KT; kt += 2) {
             publish();
-            step(f0, f1, kt + 1, 0, true, kt + NSTAGE);
+            step(f0, f1, kt + 1, 0, true, kt + NSTAGE, false);
             publish();
-            step(f1, f0, kt + 2, 0, true, kt + 1 + NSTAGE);
+            step(f1, f0, kt + 2, 0, true, kt + 1 + NSTAGE, true);
         }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
