@@ -84,7 +84,8 @@ __device__ __forceinline__ float round16(float v) {
 // reference's rule (argmin of float32 distances with 1e-6 taken off the even-mantissa candidate, e2m1_index in
 // mx_codec.h) differs from that only for a value within about 1e-6 of the midpoint between two E2M1 values.  Such
 // a value is found by converting the inputs nudged down and up by 2^-17 of themselves: if the two conversions
-// differ anywhere in the word, the lane falls back to the explicit rule.  (2^-17 of a value near a midpoint - the
+// agree, no rounding boundary lies between them and that word is the result; if they differ anywhere in the word,
+// the lane falls back to the explicit rule.  (2^-17 of a value near a midpoint - the
 // smallest is 0.25 - is at least 1.9e-6.)  Scales too small for a normal float32 take the explicit rule as well.
 // When the pre-scale is a power of two the scaled values are 16-bit inputs times a power of two, at most 11
 // significant bits: such a value is either exactly a midpoint - where the two rules agree (both take the even
@@ -96,12 +97,16 @@ __device__ __forceinline__ uint32_t e2m1_pack8(const float (&x)[8], int se, bool
         if (se >= -126) {
             const float sc = mpsa_u2f((uint32_t)(se + 127) << 23);
             const float dn = 1.0f - 0x1p-17f, up = 1.0f + 0x1p-17f;
-            uint32_t w = 0, wd = 0, wu = 0;
-            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[0], x[1], sc, 0);
-            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[2], x[3], sc, 1);
-            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[4], x[5], sc, 2);
-            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[6], x[7], sc, 3);
-            if (exact16) return w;
+            if (exact16) {
+                uint32_t w = 0;
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[0], x[1], sc, 0);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[2], x[3], sc, 1);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[4], x[5], sc, 2);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[6], x[7], sc, 3);
+                return w;
+            }
+            // no boundary between the two nudged values: the value itself converts to the same codes
+            uint32_t wd = 0, wu = 0;
             wd = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wd, x[0] * dn, x[1] * dn, sc, 0);
             wd = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wd, x[2] * dn, x[3] * dn, sc, 1);
             wd = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wd, x[4] * dn, x[5] * dn, sc, 2);
@@ -110,7 +115,7 @@ __device__ __forceinline__ uint32_t e2m1_pack8(const float (&x)[8], int se, bool
             wu = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wu, x[2] * up, x[3] * up, sc, 1);
             wu = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wu, x[4] * up, x[5] * up, sc, 2);
             wu = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(wu, x[6] * up, x[7] * up, sc, 3);
-            if (wd == wu) return w;
+            if (wd == wu) return wd;
         }
     }
     uint32_t word = 0;
