@@ -74,17 +74,20 @@ template <> __device__ __forceinline__ OutE5M2 cvt_out<OutE5M2>(float v) {
     return OutE5M2{(uint8_t)(sign | code)};
 }
 
-// Direct-to-LDS load written as inline assembly: lane L's BYTES bytes at gsrc land at lds_wave_base + L*BYTES
-// (M0 carries the wave-uniform LDS base).  The compiler's own builtin for this instruction makes it wait for
+// Direct-to-LDS load written as inline assembly: lane L's BYTES bytes at wave_base + lane_off land at
+// lds_wave_base + L*BYTES (M0 carries the wave-uniform LDS base; the global address is a scalar base plus a
+// 32-bit lane offset, so advancing along K costs scalar additions only).  The compiler's own builtin for this instruction makes it wait for
 // every outstanding load (vmcnt(0)) before the next barrier or LDS read, which would drain the ring each stage;
 // as assembly the loads are invisible to that bookkeeping and the kernel's explicit partial waits stand.
 template <int BYTES>
-__device__ __forceinline__ void load_to_lds(const uint8_t* gsrc, uint8_t* lds_wave_base) {
+__device__ __forceinline__ void load_to_lds(uint32_t lane_off, const uint8_t* wave_base, uint8_t* lds_wave_base) {
+    // address = wave-uniform base (scalar registers) + the lane's unsigned 32-bit byte offset
     const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds_wave_base);
+    const uint64_t gb = (uint64_t)(uintptr_t)wave_base;
     if constexpr (BYTES == 16)
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(gsrc) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(base), "v"(lane_off), "s"(gb) : "memory", "m0");
     else
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(gsrc) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(base), "v"(lane_off), "s"(gb) : "memory", "m0");
 }
 
 template <int FMT, typename OutT, bool WIDE>
@@ -134,32 +137,34 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     g.sa += (int64_t)bz * g.M * srow_bytes;
     g.b += zb * g.N * row_bytes;
     g.sb += zb * g.N * srow_bytes;
-    const uint8_t* ga[4];
-    const uint8_t* gb[4];
+    // lane offsets inside a tile's operand (the same for A and B) and inside its scale rows; tile bases are scalar
+    uint32_t lo[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         const int p = (wave * 4 + c) * 64 + lane;
         const int row = p >> 2, slot = p & 3;
         const int cb = slot ^ ((row >> 2) & 3);
-        ga[c] = g.a + (int64_t)(m0 + row) * row_bytes + cb * 16;
-        gb[c] = g.b + (int64_t)(n0 + row) * row_bytes + cb * 16;
+        lo[c] = (uint32_t)row * (uint32_t)row_bytes + cb * 16;
     }
-    const uint8_t* gsa = g.sa + (int64_t)(m0 + wave * 64 + lane) * srow_bytes;
-    const uint8_t* gsb = g.sb + (int64_t)(n0 + wave * 64 + lane) * srow_bytes;
+    const uint32_t los = (uint32_t)(wave * 64 + lane) * (uint32_t)srow_bytes;
+    const uint8_t* const a_base = g.a + (int64_t)m0 * row_bytes;
+    const uint8_t* const b_base = g.b + (int64_t)n0 * row_bytes;
+    const uint8_t* const sa_base = g.sa + (int64_t)m0 * srow_bytes;
+    const uint8_t* const sb_base = g.sb + (int64_t)n0 * srow_bytes;
     // a stage's loads go out in four parts (two code instructions each, the narrow path's scale words with the
     // last) so that they can be spread between the matrix instructions of a step
     auto issue_part = [&](int kt, int part) __attribute__((always_inline)) {
         const int kc = kt < KT ? kt : KT - 1;             // past the end: re-load the last stage (keeps the count uniform)
         uint8_t* st = smem + (kt % NSTAGE) * STAGE_BYTES;
-        load_to_lds<16>(ga[part] + (int64_t)kc * ROWB, st + (wave * 4 + part) * 1024);
-        load_to_lds<16>(gb[part] + (int64_t)kc * ROWB, st + OP_BYTES + (wave * 4 + part) * 1024);
+        load_to_lds<16>(lo[part], a_base + (int64_t)kc * ROWB, st + (wave * 4 + part) * 1024);
+        load_to_lds<16>(lo[part], b_base + (int64_t)kc * ROWB, st + OP_BYTES + (wave * 4 + part) * 1024);
         if constexpr (!WIDE) {
             if (part == 3) {
                 // four scale bytes per row: the stage's own with 4-bit codes; with 8-bit codes the aligned word
                 // that holds this stage's two bytes (the stage count is even, so the word is inside the row)
                 const int sco = FP4 ? kc * 4 : (kc >> 1) * 4;
-                load_to_lds<4>(gsa + sco, st + 2 * OP_BYTES + wave * 256);
-                load_to_lds<4>(gsb + sco, st + 2 * OP_BYTES + SC_BYTES + wave * 256);
+                load_to_lds<4>(los, sa_base + sco, st + 2 * OP_BYTES + wave * 256);
+                load_to_lds<4>(los, sb_base + sco, st + 2 * OP_BYTES + SC_BYTES + wave * 256);
             }
         }
     };
@@ -172,8 +177,8 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         const int ng = KT / GROUP;
         const int gc = grp < ng ? grp : ng - 1;
         uint8_t* dst = scg + (grp & 1) * 2 * SCG_BYTES + wave * 1024;
-        load_to_lds<16>(gsa + gc * 16, dst);
-        load_to_lds<16>(gsb + gc * 16, dst + SCG_BYTES);
+        load_to_lds<16>(los, sa_base + gc * 16, dst);
+        load_to_lds<16>(los, sb_base + gc * 16, dst + SCG_BYTES);
     };
 
     v16f acc[4][4];
@@ -378,7 +383,7 @@ extern "C" int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, const u
     if (M <= 0 || N <= 0 || K <= 0 || ldc < N) return mpsa_fail(MPSA_EINVAL, "gemm: bad shape");
     if (batch <= 0 || heads_a <= 0 || heads_b <= 0 || heads_a % heads_b) return mpsa_fail(MPSA_EINVAL, "gemm: bad batch shape (batch=%lld heads_a=%lld heads_b=%lld)", (long long)batch, (long long)heads_a, (long long)heads_b);
     if (M % BM || N % BN || K % 128) return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: M,N must be multiples of 256 and K of 128 (got %lld,%lld,%lld)", (long long)M, (long long)N, (long long)K);
-    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30) || (M / BM) * (N / BN) > (int64_t(1) << 30) || batch * heads_a > 65535)
+    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 24) || (M / BM) * (N / BN) > (int64_t(1) << 30) || batch * heads_a > 65535)
         return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: shape too large");
     if (!mpsa_aligned16(a) || !mpsa_aligned16(b) || (reinterpret_cast<uintptr_t>(sa) & 3) || (reinterpret_cast<uintptr_t>(sb) & 3))
         return mpsa_fail(MPSA_EALIGN, "gemm: codes must be 16-byte and scales 4-byte aligned");
