@@ -38,6 +38,7 @@ typedef void* mpsa_stream_t;
 #define MPSA_MODE_MXFP4 0   /* every tile 4-bit */
 #define MPSA_MODE_MXFP8 1   /* every tile 8-bit */
 #define MPSA_MODE_DIAG  2   /* tile j == i 8-bit, all others 4-bit */
+#define MPSA_MODE_ROUTED 3  /* per-tile precision from a visiting list (mpsa_route_tiles, mpsa_attn_fwd_routed) */
 
 #define MPSA_OK             0
 #define MPSA_EINVAL        -1   /* null pointer, bad enum, bad shape */
@@ -173,7 +174,7 @@ int mpsa_v_tiles(const void* v, int v_dtype, int64_t B, int64_t H, int64_t N, in
  *
  *   q [B,Hq,Nq,D], k and v [B,Hkv,Nk,D] of dtype (MPSA_BF16 | MPSA_F16), element strides as for mpsa_quantize_mx
  *   mode       MPSA_MODE_MXFP4: only the 4-bit outputs are written (8-bit pointers may be null),
- *              MPSA_MODE_MXFP8: only the 8-bit ones, MPSA_MODE_DIAG: both
+ *              MPSA_MODE_MXFP8: only the 8-bit ones, MPSA_MODE_DIAG / MPSA_MODE_ROUTED: both
  *   k_sub      NULL or [B,Hkv,D] (smooth-K mean from mpsa_seq_mean)
  *   outputs    as the inputs of mpsa_attn_fwd
  */
@@ -226,6 +227,45 @@ int mpsa_attn_fwd_skip(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8,
                        const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
                        int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t nk, int64_t D, int tile, int causal, int mode,
                        float skip_thresh, int32_t* skipped, mpsa_stream_t stream);
+
+/*
+ * Tile router: precision class of every (query tile, key tile) pair from the 4-bit E8M0 scale bytes of Q and K.
+ * The reference's online routing keeps or skips a tile by comparing a tile statistic with the first tile's
+ * (ours/online_routing.py:87-112, the skip_thresh of ours/mxfp_attn.py:32); this router extends that to a precision
+ * choice and takes the statistic from the quantizer's own output.  Per tile and 32-wide block c of the head
+ * dimension, over the tile's rows r (e = scale byte): M[c] = max_r e[r][c], F[c] = sum_r 2^(10 - (M[c] - e[r][c]))
+ * with terms below 1 dropped.  For query tile I and key tile J: s[c] = Mq[I][c] + Mk[J][c], w[c] = Fq[I][c] * Fk[J][c],
+ * smax[I] the largest s[c] over the visited key tiles, T[I][J] = (sum_c (w[c] >> (smax[I] - s[c]))) >> 13 (shifts
+ * above 40 give 0) and Tmax[I] the largest T[I][J]:
+ *     8-bit    if (float)T >= hi_thresh * (float)Tmax
+ *     skipped  else if (float)T < skip_thresh * (float)Tmax and J != 0 and not (causal and J == I)
+ *     4-bit    otherwise;                         a threshold <= 0 switches its class off.
+ * T is proportional to the summed magnitude bound of the tile's scores, i.e. to the absolute error of a 4-bit product.
+ *   qs4, ks4   [B,Hq,nq_pad,D/32], [B,Hkv,nk_pad,D/32] from the quantizer (padding rows zero)
+ *   work       mpsa_route_workspace(...) bytes of device memory (the per-tile statistics), 4-byte aligned
+ *   cls        out, uint8 [B,Hq,ntq,ntk]: 0 skipped, 1 4-bit, 2 8-bit, 255 not visited (causal, J > I)
+ *   order      out, int32 [B,Hq,ntq,ntk]: per query tile the key tiles to visit -- 4-bit ones that need no mask
+ *              (ascending), 4-bit ones that do (the diagonal tile of a causal run, the tile holding a ragged sequence
+ *              end), then the 8-bit ones likewise; the rest is -1
+ *   counts     out, int32 [B,Hq,ntq,4]: lengths of those four runs
+ */
+int64_t mpsa_route_workspace(int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t nk, int64_t D, int tile);
+int mpsa_route_tiles(const uint8_t* qs4, const uint8_t* ks4, int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t nk,
+                     int64_t D, int tile, int causal, float hi_thresh, float skip_thresh, void* work,
+                     uint8_t* cls, int32_t* order, int32_t* counts, mpsa_stream_t stream);
+
+/*
+ * Fused attention forward over visiting lists (per-tile precision; BLKQ x BLKQ granularity as in mpsa_attn_fwd).
+ * Arguments as mpsa_attn_fwd without mode (both operand sets are needed), plus order / counts as written by
+ * mpsa_route_tiles -- or by the caller: any list of distinct key tiles works, as long as every tile that needs a mask
+ * sits in a masked run.  Key tiles not on a query tile's list contribute nothing; a query tile with an empty list
+ * returns zeros.  Out-of-range list entries and run lengths are clamped, never followed.
+ */
+int mpsa_attn_fwd_routed(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
+                         const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
+                         const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
+                         int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t nk, int64_t D, int tile, int causal,
+                         const int32_t* order, const int32_t* counts, mpsa_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -15,13 +15,14 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libmpsa.so")
 
-SOURCES = ["api.hip", "formats.hip", "quantize.hip", "v_tiles.hip", "prepare.hip", "gemm_mx.hip", "attn_fwd.hip", "attn_fwd_skip.hip", "attn_fwd_pp.hip"]
+SOURCES = ["api.hip", "formats.hip", "quantize.hip", "v_tiles.hip", "prepare.hip", "gemm_mx.hip", "attn_fwd.hip", "attn_fwd_skip.hip", "attn_fwd_routed.hip", "attn_fwd_pp.hip", "route.hip"]
 
 # packed-fp32 instructions are switched off on purpose (the flag is for the device pass; the host
 # pass warns that it does not know the feature, which is harmless)
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-PER_FILE = {"quantize.hip": ["-ffp-contract=off"], "formats.hip": ["-ffp-contract=off"], "prepare.hip": ["-ffp-contract=off"]}
+PER_FILE = {"quantize.hip": ["-ffp-contract=off"], "formats.hip": ["-ffp-contract=off"], "prepare.hip": ["-ffp-contract=off"],
+            "route.hip": ["-ffp-contract=off"]}
 
 
 def _hipcc():

@@ -14,6 +14,8 @@ struct AttnArgs {
     int d, tile;
     float skip_thresh;         // tile-skipping variants only
     int32_t* skipped;          // optional [B,Hq,nt] count of skipped key tiles per query tile
+    const int32_t* order;      // routed runs only: [B,Hq,ntq,nt] visiting lists and [B,Hq,ntq,4] run lengths
+    const int32_t* counts;
 };
 
 template <int PVT> struct PV;
@@ -75,6 +77,9 @@ __device__ __forceinline__ void load16_to_lds(const uint8_t* gsrc, uint8_t* lds_
 
 // Tile-skipping variants of the general kernel (modes mxfp4 / mxfp8): attn_fwd_skip.hip
 int attn_skip_launch(const AttnArgs& a, int pv_dtype, hipStream_t st);
+
+// Routed variants of the general kernel (per-tile precision from a visiting list): attn_fwd_routed.hip
+int attn_routed_launch(const AttnArgs& a, int pv_dtype, hipStream_t st);
 
 // Paired-tile ("ping-pong") kernel for causal runs with D = 128, tile = 128 and whole tile pairs: attn_fwd_pp.hip
 bool attn_pp_supported(const AttnArgs& a, int pv_dtype);

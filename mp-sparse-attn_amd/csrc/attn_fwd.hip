@@ -56,8 +56,12 @@ static int attn_entry(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, 
                       const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
                       const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
                       int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal, int mode,
-                      bool skip, float skip_thresh, int32_t* skipped, mpsa_stream_t stream) {
-    if (mode != MPSA_MODE_MXFP4 && mode != MPSA_MODE_MXFP8 && mode != MPSA_MODE_DIAG) return mpsa_fail(MPSA_EINVAL, "attn: unknown mode %d", mode);
+                      bool skip, float skip_thresh, int32_t* skipped, const int32_t* order, const int32_t* counts,
+                      mpsa_stream_t stream) {
+    if (mode != MPSA_MODE_MXFP4 && mode != MPSA_MODE_MXFP8 && mode != MPSA_MODE_DIAG && mode != MPSA_MODE_ROUTED) return mpsa_fail(MPSA_EINVAL, "attn: unknown mode %d", mode);
+    const bool routed = mode == MPSA_MODE_ROUTED;
+    if (routed && (!order || !counts)) return mpsa_fail(MPSA_EINVAL, "attn: a routed run needs the visiting lists (order, counts)");
+    if (routed && ((reinterpret_cast<uintptr_t>(order) | reinterpret_cast<uintptr_t>(counts)) & 3)) return mpsa_fail(MPSA_EALIGN, "attn: order and counts must be 4-byte aligned");
     const bool need4 = mode != MPSA_MODE_MXFP8, need8 = mode != MPSA_MODE_MXFP4;
     if (need4 && (!q4 || !qs4 || !k4 || !ks4)) return mpsa_fail(MPSA_EINVAL, "attn: 4-bit operands missing");
     if (need8 && (!q8 || !qs8 || !k8 || !ks8)) return mpsa_fail(MPSA_EINVAL, "attn: 8-bit operands missing");
@@ -84,7 +88,9 @@ static int attn_entry(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, 
     a.causal = causal ? 1 : 0; a.mode = mode; a.fmt8 = fmt8; a.o_dtype = o_dtype;
     a.d = (int)D; a.tile = tile;
     a.skip_thresh = skip_thresh; a.skipped = skipped;
+    a.order = order; a.counts = counts;
     hipStream_t st = (hipStream_t)stream;
+    if (routed) return attn_routed_launch(a, pv_dtype, st);
     if (skip) {
         if (mode == MPSA_MODE_DIAG) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: tile skipping needs a single-precision mode (mxfp4 or mxfp8): the rule's reference tile is the first key tile, which a diag run visits last for query tile 0");
         if (!(skip_thresh == skip_thresh)) return mpsa_fail(MPSA_EINVAL, "attn: skip_thresh is NaN");
@@ -110,7 +116,7 @@ extern "C" int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_
                              int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal, int mode,
                              mpsa_stream_t stream) {
     return attn_entry(q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
-                      B, Hq, Hkv, nq, n, D, tile, causal, mode, false, 0.0f, nullptr, stream);
+                      B, Hq, Hkv, nq, n, D, tile, causal, mode, false, 0.0f, nullptr, nullptr, nullptr, stream);
 }
 
 extern "C" int mpsa_attn_fwd_skip(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
@@ -119,5 +125,14 @@ extern "C" int mpsa_attn_fwd_skip(const uint8_t* q4, const uint8_t* qs4, const u
                                   int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal, int mode,
                                   float skip_thresh, int32_t* skipped, mpsa_stream_t stream) {
     return attn_entry(q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
-                      B, Hq, Hkv, nq, n, D, tile, causal, mode, true, skip_thresh, skipped, stream);
+                      B, Hq, Hkv, nq, n, D, tile, causal, mode, true, skip_thresh, skipped, nullptr, nullptr, stream);
+}
+
+extern "C" int mpsa_attn_fwd_routed(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
+                                    const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
+                                    const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
+                                    int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal,
+                                    const int32_t* order, const int32_t* counts, mpsa_stream_t stream) {
+    return attn_entry(q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
+                      B, Hq, Hkv, nq, n, D, tile, causal, MPSA_MODE_ROUTED, false, 0.0f, nullptr, order, counts, stream);
 }

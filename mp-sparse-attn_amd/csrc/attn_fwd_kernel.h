@@ -27,6 +27,10 @@ struct Geom {
 // fragments in registers (read from global memory one step ahead), and a "diag" run pipelines 4-bit tiles through
 // LDS and fetches its single 8-bit tile when it gets there.
 //
+// A "routed" run (MPSA_MODE_ROUTED) walks a visiting list made by the tile router (route.hip): the 4-bit tiles through
+// the LDS pipeline, then the 8-bit tiles with their K fragments prefetched from global memory; inside each precision
+// the tiles that need a mask come last, so the two long loops keep the single-variant body.
+//
 // SKIP adds the reference's tile-skipping rule (ours/mxfp_attn_kernel.py:272-297): the statistic of a score tile
 // is the mean over its query rows of the row maximum; the first key tile (the "sink") is always kept and sets the
 // reference value, any later tile is kept only if its statistic is at least skip_thresh times the sink's (the
@@ -69,20 +73,39 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     // Visiting order.  The order of key tiles does not matter to the softmax, so the tiles that need special
     // treatment go LAST: first every plain tile (main precision, no mask) in one tight loop, then the tile that
     // holds the sequence tail (masked) if there is one, then the diagonal tile i (causal mask and / or 8-bit).
+    constexpr bool ROUTED = MODE == MPSA_MODE_ROUTED;
     constexpr bool HAS4 = MODE != MPSA_MODE_MXFP8;        // 4-bit tiles exist (LDS pipeline in use)
-    constexpr bool PRE8 = MODE == MPSA_MODE_MXFP8;        // 8-bit K fragments are prefetched one step ahead
+    constexpr bool PRE8 = MODE == MPSA_MODE_MXFP8 || ROUTED;   // 8-bit K fragments are prefetched one step ahead
     const bool tail = a.n < a.n_pad;
     const bool diag_special = a.causal || MODE == MPSA_MODE_DIAG;
     const bool tail_special = tail && !a.causal && !(MODE == MPSA_MODE_DIAG && i == a.nt - 1);
-    const int nsteps = a.causal ? i + 1 : a.nt;
+    // routed: lengths of the list's four runs (4-bit plain, 4-bit masked, 8-bit plain, 8-bit masked), clamped so
+    // that a malformed list cannot take the kernel outside its buffers
+    const int64_t route_row = ((int64_t)b * a.Hq + hq) * a.ntq + i;
+    const int32_t* const ord = ROUTED ? a.order + route_row * a.nt : nullptr;
+    int r4p = 0, r4 = 0, r8p = 0;
+    int nsteps = a.causal ? i + 1 : a.nt;
+    if constexpr (ROUTED) {
+        const int32_t* cn = a.counts + route_row * 4;
+        const int c0 = min(max(cn[0], 0), a.nt);
+        const int c1 = min(max(cn[1], 0), a.nt - c0);
+        const int c2 = min(max(cn[2], 0), a.nt - c0 - c1);
+        const int c3 = min(max(cn[3], 0), a.nt - c0 - c1 - c2);
+        r4p = c0; r4 = c0 + c1; r8p = r4 + c2; nsteps = r8p + c3;
+    }
     const int n_plain = nsteps - (diag_special ? 1 : 0) - (tail_special ? 1 : 0);
     const int skip = (MODE == MPSA_MODE_DIAG && !a.causal) ? i : 0x7fffffff;   // plain steps jump over tile i
+    const int n_k4 = ROUTED ? r4 : nsteps;                // steps whose K tile travels through LDS
     auto tile_at = [&](int t) {
+        if constexpr (ROUTED) return t < nsteps ? min(max(ord[t], 0), a.nt - 1) : 0;
         if (t < n_plain) return t + (t >= skip ? 1 : 0);
         if (tail_special && t == n_plain) return a.nt - 1;
         return i;
     };
-    auto step_is8 = [&](int t) { return MODE == MPSA_MODE_MXFP8 || (MODE == MPSA_MODE_DIAG && t == nsteps - 1); };
+    auto step_is8 = [&](int t) {
+        if constexpr (ROUTED) return t >= r4;
+        return MODE == MPSA_MODE_MXFP8 || (MODE == MPSA_MODE_DIAG && t == nsteps - 1);
+    };
 
     // ---- Q fragments of the current precision stay in registers; re-read when the precision changes ----
     v8i qf[G::SST];
@@ -187,12 +210,14 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     const bool first8 = step_is8(0);
     issue_v(0);
     if constexpr (HAS4) {
-        issue_k4(0);
-        if (nsteps > 1) issue_k4(1);
+        if (n_k4 > 0) issue_k4(0);
+        if (n_k4 > 1) issue_k4(1);
     }
     load_kscales(0, first8);
     load_q(first8);
-    if constexpr (PRE8) load_kf8(0, kf8);
+    if constexpr (PRE8) {
+        if (!ROUTED || first8) load_kf8(0, kf8);
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0)
     __syncthreads();
     if constexpr (HAS4) read_kf4(0);
@@ -319,7 +344,7 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
 
         if (t + 1 < nsteps) issue_v(t + 1);
         if constexpr (HAS4) {
-            if (t + 2 < nsteps) issue_k4(t + 2);
+            if (t + 2 < n_k4) issue_k4(t + 2);
         }
 
         // ---- O^T += V^T P^T, V fragments prefetched PRE instructions ahead ----
@@ -333,9 +358,13 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         // operands of the next step: scales (and 8-bit K) from global memory, 4-bit K from LDS.  Past the last
         // step this reads a valid but unused tile.
         if constexpr (PREP) {
-            load_kscales(t + 1, PRE8);
-            if constexpr (PRE8) load_kf8(t + 1, kf8);
-            if constexpr (HAS4) read_kf4(t + 1);
+            load_kscales(t + 1, IS8);
+            if constexpr (PRE8) {
+                if constexpr (IS8) load_kf8(t + 1, kf8);
+            }
+            if constexpr (HAS4) {
+                if constexpr (!IS8) read_kf4(t + 1);
+            }
         }
         if (keep) {
 #pragma unroll
@@ -349,11 +378,24 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     };
 
     // ---- plain tiles: one tight single-variant loop ----
-    for (int t = 0; t < n_plain; ++t) step(t, std::integral_constant<bool, PRE8>{}, std::false_type{}, std::true_type{});
+    if constexpr (!ROUTED) {
+        for (int t = 0; t < n_plain; ++t) step(t, std::integral_constant<bool, PRE8>{}, std::false_type{}, std::true_type{});
+    }
     // ---- the (at most two) special tiles: the sequence-tail tile, then the diagonal tile; both run the masked
     //      variant (a mask that hides nothing is harmless).  The step before has already fetched their K operand
     //      unless the precision changes. ----
-    if constexpr (MODE == MPSA_MODE_DIAG) {
+    if constexpr (ROUTED) {
+        // (the first loop above is empty: n_plain is not used by routed runs)
+        for (int t = 0; t < r4p; ++t) step(t, std::false_type{}, std::false_type{}, std::true_type{});
+        for (int t = r4p; t < r4; ++t) step(t, std::false_type{}, std::true_type{}, std::true_type{});
+        if (r4 > 0 && r4 < nsteps) {                   // otherwise the prologue already loaded the 8-bit operands
+            load_kscales(r4, true);
+            load_q(true);
+            load_kf8(r4, kf8);
+        }
+        for (int t = r4; t < r8p; ++t) step(t, std::true_type{}, std::false_type{}, std::true_type{});
+        for (int t = r8p; t < nsteps; ++t) step(t, std::true_type{}, std::true_type{}, std::true_type{});
+    } else if constexpr (MODE == MPSA_MODE_DIAG) {
         if (tail_special) step(n_plain, std::false_type{}, std::true_type{}, std::true_type{});
         if (nsteps > 1) {                              // otherwise the prologue already loaded 8-bit Q and scales
             load_kscales(nsteps - 1, true);
@@ -363,6 +405,7 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     } else {
         for (int t = n_plain; t < nsteps; ++t) step(t, std::integral_constant<bool, PRE8>{}, std::true_type{}, std::true_type{});
     }
+    (void)r4p; (void)r8p;
     __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
 
     if constexpr (SKIP) {
@@ -370,7 +413,7 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     }
     // ---- epilogue: O = acc / l ; register e of lane (h, r): dim 32*db + 8*(e/4) + 4*h + e%4 of query r ----
     const float l_tot = sum_lane_pair(l_run);
-    const float inv = 1.0f / l_tot;
+    const float inv = (ROUTED && !(l_tot > 0.0f)) ? 0.0f : 1.0f / l_tot;   // routed: a row with every tile skipped gives zeros
     const int q_global = i * TILE + q_local;
     if (q_global < a.nq) {
         uint8_t* orow = static_cast<uint8_t*>(a.o);

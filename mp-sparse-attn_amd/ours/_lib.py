@@ -11,7 +11,7 @@ import torch
 
 BF16, F16, F32, F8E5M2 = 0, 1, 2, 3
 FMT_E4M3, FMT_E5M2, FMT_E2M1 = 0, 1, 4
-MODE_MXFP4, MODE_MXFP8, MODE_DIAG = 0, 1, 2
+MODE_MXFP4, MODE_MXFP8, MODE_DIAG, MODE_ROUTED = 0, 1, 2, 3
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("MPSA_LIB_PATH") or os.path.join(os.path.dirname(_HERE), "lib", "libmpsa.so")
@@ -45,6 +45,10 @@ SIGNATURES = {
                              _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
     "mpsa_attn_fwd_skip": (_int, [_vp] * 8 + [_int, _vp, _int, _vp, _int, _p64,
                                   _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _vp, _vp]),
+    "mpsa_route_workspace": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
+    "mpsa_route_tiles": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _f32, _f32, _vp, _vp, _vp, _vp, _vp]),
+    "mpsa_attn_fwd_routed": (_int, [_vp] * 8 + [_int, _vp, _int, _vp, _int, _p64,
+                                    _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp, _vp]),
 }
 
 _lib = None

@@ -35,6 +35,10 @@ Parity status of each restated function:
   (``skip_thresh``) is pinned against an independent dense float64 formulation
   of the statistic, the decisions and the restricted softmax
   (tests/test_oracle_gemm_attn.py).
+* ``route_tiles`` / ``route_order`` -- this build's own integer rule (the reference has no precision router);
+  pinned against a float64 evaluation of the score bound it stands for and hand-worked maps
+  (tests/test_oracle_route.py); ``attn_mx(mode="routed")`` is pinned against the dense float64 attention on the
+  same map and must reproduce the fixed modes on the maps that describe them.
 * ``seq_mean`` / ``smooth_k`` -- the once-rounded mean is pinned against
   float64 arithmetic and exactly representable cases; the float32 summation
   order of the reference's device mean is not reproducible (PARITY UNPINNED in
@@ -50,4 +54,5 @@ from .mx_quantize import (  # noqa: F401
     FMT_E2M1, FMT_E4M3, FMT_E5M2, EMAX_ELEM, q_pre_scale, quantize_mx, dequantize_mx, smooth_k, seq_mean,
 )
 from .mx_gemm import gemm_mx, scales_to_5d, scales_from_5d  # noqa: F401
+from .mx_route import route_tiles, route_order, tile_scale_stats  # noqa: F401
 from .mx_attention import attn_mx, attn_dense_f64, precision_metric, v_fragment_order  # noqa: F401

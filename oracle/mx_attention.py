@@ -17,10 +17,12 @@ import torch.nn.functional as Fnn
 
 from .mx_quantize import FMT_E2M1, FMT_E4M3, quantize_mx, dequantize_mx, q_pre_scale, smooth_k as _smooth_k
 
-MODES = ("mxfp4", "mxfp8", "diag")
+MODES = ("mxfp4", "mxfp8", "diag", "routed")
 
 
-def _tile_is_8bit(mode: str, i: int, j: int) -> bool:
+def _tile_is_8bit(mode: str, i: int, j: int, route=None) -> bool:
+    if mode == "routed":
+        return int(route[i, j]) == 2
     if mode == "mxfp8":
         return True
     if mode == "mxfp4":
@@ -35,10 +37,10 @@ def _prepare(q, k, mode, scale, fmt8):
     D = q.shape[-1]
     pre = q_pre_scale(D, scale)
     ops = {}
-    if mode in ("mxfp4", "diag"):
+    if mode in ("mxfp4", "diag", "routed"):
         ops["q4"] = dequantize_mx(*quantize_mx(q, pre, FMT_E2M1), FMT_E2M1)
         ops["k4"] = dequantize_mx(*quantize_mx(k, 1.0, FMT_E2M1), FMT_E2M1)
-    if mode in ("mxfp8", "diag"):
+    if mode in ("mxfp8", "diag", "routed"):
         ops["q8"] = dequantize_mx(*quantize_mx(q, pre, fmt8), fmt8)
         ops["k8"] = dequantize_mx(*quantize_mx(k, 1.0, fmt8), fmt8)
     return ops
@@ -46,7 +48,7 @@ def _prepare(q, k, mode, scale, fmt8):
 
 def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=False,
             fmt8=FMT_E4M3, out_dtype=None, heads=None, q_tiles=None, skip_thresh=None, return_skipped=False,
-            ratios_out=None):
+            ratios_out=None, route=None):
     """Tile-by-tile MXFP attention.  q ``[B,Hq,N,D]``, k/v ``[B,Hkv,N,D]`` in bf16 or fp16.
 
     P is rounded to v's dtype before P.V and the product of a tile is accumulated in float32
@@ -60,11 +62,15 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
     tile 0 is always kept and sets the reference value, tile j > 0 is kept iff its statistic is at least
     ``skip_thresh`` times that; the diagonal tile of a causal run is always kept too (the reference's causal loop,
     ours/online_routing.py:68-77, walks it as a stage of its own whose first tile is exempt).  ``return_skipped`` adds an int32 ``[B, heads, tiles]`` count of skipped tiles;
-    a list passed as ``ratios_out`` collects statistic(j) / statistic(0) of every tile j > 0 examined."""
+    a list passed as ``ratios_out`` collects statistic(j) / statistic(0) of every tile j > 0 examined.
+
+    ``mode="routed"``: ``route`` ``[B,Hq,tiles,key tiles]`` gives every tile's class (0 skip, 1 4-bit, 2 8-bit, 255 not
+    visited), see :mod:`oracle.mx_route`; a query row whose every tile is skipped returns zeros."""
     B, Hq, N, D = q.shape
     Hkv, Nk = k.shape[1], k.shape[2]
     assert Hq % Hkv == 0
     assert Nk == N or (not causal and mode != "diag"), "cross attention: non-causal, single precision"
+    assert (mode == "routed") == (route is not None)
     group = Hq // Hkv
     if smooth_k:
         k = _smooth_k(k)
@@ -95,7 +101,9 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
                 last = i if causal else ntk - 1
                 for j in range(last + 1):
                     c0, c1 = j * tile, min((j + 1) * tile, Nk)
-                    tag = "8" if _tile_is_8bit(mode, i, j) else "4"
+                    if mode == "routed" and int(route[b, h, i, j]) not in (1, 2):
+                        continue
+                    tag = "8" if _tile_is_8bit(mode, i, j, None if route is None else route[b, h]) else "4"
                     qt = ops["q" + tag][b, hi_, r0:r1]
                     kt = ops["k" + tag][b, kvh, c0:c1]
                     s = qt @ kt.T                                    # float32, already in log2 units
@@ -120,6 +128,9 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
                     pv = p.to(lp).to(torch.float32) @ vf[b, kvh, c0:c1]
                     acc = acc * alpha.unsqueeze(1) + pv
                     m = m_new
+                if mode == "routed":
+                    acc = torch.where(l.unsqueeze(1) > 0, acc, torch.zeros(()))
+                    l = torch.where(l > 0, l, torch.ones(()))
                 out[b, hi_, starts[i]:starts[i] + rows] = (acc / l.unsqueeze(1)).to(out_dtype)
     if return_skipped:
         return out, skipped
@@ -127,7 +138,7 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
 
 
 def attn_dense_f64(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=False,
-                   fmt8=FMT_E4M3, heads=None) -> torch.Tensor:
+                   fmt8=FMT_E4M3, heads=None, route=None) -> torch.Tensor:
     """Brute-force check of :func:`attn_mx`: the full score matrix is assembled tile by tile from
     the per-tile-precision dequantised operands, then a dense base-2 softmax and P.V in float64
     (no online rescaling, no low-precision P)."""
@@ -146,7 +157,9 @@ def attn_dense_f64(q, k, v, tile=128, causal=True, mode="diag", scale=None, smoo
             s = torch.full((N, N), float("-inf"), dtype=torch.float64)
             for i in range(nt):
                 for j in range((i if causal else nt - 1) + 1):
-                    tag = "8" if _tile_is_8bit(mode, i, j) else "4"
+                    if mode == "routed" and int(route[b, h, i, j]) not in (1, 2):
+                        continue                                     # skipped: the tile's scores stay -inf
+                    tag = "8" if _tile_is_8bit(mode, i, j, None if route is None else route[b, h]) else "4"
                     r = slice(i * tile, min((i + 1) * tile, N))
                     c = slice(j * tile, min((j + 1) * tile, N))
                     s[r, c] = ops["q" + tag][b, hi_, r] @ ops["k" + tag][b, kvh, c].T
