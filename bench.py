@@ -146,7 +146,7 @@ def secondary(device, quick):
 def run_only(args, device):
     """Launch one kernel repeatedly (for rocprofv3 --pmc / --kernel-trace runs)."""
     from ours import _lib
-    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, route_tiles
     from ours.quant_mxint8 import quantize_mx, quantize_mx_dual
     from ours.block_scaled_matmul import block_scaled_matmul, make_configs
     if args.only == "copy":
@@ -159,9 +159,10 @@ def run_only(args, device):
         causal = args.workload not in NON_CAUSAL
         q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21)
         out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
-        ops = prepare_operands(q, k, v, tile, "diag")
-        fn = lambda: attention_from_operands(ops, out, causal)
-        info = {"kernel": "attention", "workload": desc}
+        ops = prepare_operands(q, k, v, tile, args.mode)
+        route = route_tiles(ops, causal, args.route_thresh, args.skip_thresh) if args.mode == "routed" else None
+        fn = lambda: attention_from_operands(ops, out, causal, route=route)
+        info = {"kernel": "attention", "workload": desc, "mode": args.mode}
     elif args.only == "quant":
         B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
         q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device)
@@ -191,6 +192,11 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--mode", default="diag", choices=["diag", "mxfp4", "mxfp8", "routed"],
+                    help="per-tile precision: diag (the headline configuration), one precision everywhere, or routed "
+                         "(tile router on the scale bytes, thresholds below)")
+    ap.add_argument("--route-thresh", type=float, default=0.9, help="routed: 8-bit at or above this share of the row's largest tile statistic")
+    ap.add_argument("--skip-thresh", type=float, default=None, help="routed: skipped below this share")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--only", default=None, choices=["attn", "copy", "quant", "gemm4", "gemm8"],
@@ -205,7 +211,7 @@ def main():
         print("bench.py needs a HIP device", file=sys.stderr)
         sys.exit(1)
 
-    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, route_tiles
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
@@ -217,9 +223,12 @@ def main():
     q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21)
     out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
 
+    routed = args.mode == "routed"
+
     def step():
-        ops = prepare_operands(q, k, v, tile, "diag")
-        attention_from_operands(ops, out, causal)
+        ops = prepare_operands(q, k, v, tile, args.mode)
+        route = route_tiles(ops, causal, args.route_thresh, args.skip_thresh) if routed else None
+        attention_from_operands(ops, out, causal, route=route)
 
     for _ in range(args.warmup):
         step()
@@ -234,32 +243,40 @@ def main():
     tflops = flops / (ms_per_step * 1e-3) / 1e12
 
     # dominant kernel alone: the fused attention kernel on prepared operands
-    ops = prepare_operands(q, k, v, tile, "diag")
-    attention_from_operands(ops, out, causal)
+    ops = prepare_operands(q, k, v, tile, args.mode)
+    route = route_tiles(ops, causal, args.route_thresh, args.skip_thresh) if routed else None
+    attention_from_operands(ops, out, causal, route=route)
     torch.cuda.synchronize()
     k_iters = max(5, args.steps)
-    attn_ms = time_events(lambda: attention_from_operands(ops, out, causal), k_iters)
-    prep_ms = time_events(lambda: prepare_operands(q, k, v, tile, "diag"), k_iters)
+    attn_ms = time_events(lambda: attention_from_operands(ops, out, causal, route=route), k_iters)
+    prep_ms = time_events(lambda: prepare_operands(q, k, v, tile, args.mode), k_iters)
     achieved = flops / (attn_ms * 1e-3) / 1e12
     nt = (N + tile - 1) // tile
     comp = composite_peak_tflops(nt, causal)
-    paired = causal and D == 128 and tile == 128 and N % 256 == 0
+    paired = causal and D == 128 and tile == 128 and N % 256 == 0 and args.mode in ("diag", "mxfp4")
     roofline = {
         "bound": "mfma", "kernel": ("attn_pp_kernel" if paired else "attn_fwd_kernel") + " (fused attention)", "achieved": round(achieved, 2), "peak": PEAK_FP4_TFLOPS,
         "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP4_TFLOPS, 5),
-        "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get(args.workload),
+        "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get(args.workload) if args.mode == "diag" else None,
         "kernel_ms": round(attn_ms, 4), "prepare_ms": round(prep_ms, 4),
         "composite_peak": round(comp, 1), "frac_composite": round(achieved / comp, 5),
         "flops_per_launch": flops,
     }
+    if routed:
+        cls = route[0]
+        visited = float((cls != 255).sum())
+        roofline["route_ms"] = round(time_events(lambda: route_tiles(ops, causal, args.route_thresh, args.skip_thresh), k_iters), 4)
+        roofline["tile_shares"] = {"mxfp8": round(float((cls == 2).sum()) / visited, 4),
+                                   "mxfp4": round(float((cls == 1).sum()) / visited, 4),
+                                   "skipped": round(float((cls == 0).sum()) / visited, 4)}
 
     result = {
         "metric": "MXFP attn TFLOPS + % of scaled-MFMA peak, causal N=8K/128K D=128, 1 GPU",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "mxfp4/mxfp8 scores (E2M1/E4M3 + E8M0), bf16 P.V, f32 accumulate", "data": "synthetic",
-        "config": {"workload": desc, "B": B, "Hq": Hq, "Hkv": Hkv, "N": N, "D": D, "tile": tile,
-                   "step": "quantize Q,K (dual) + V repack + fused attention"},
+        "config": {"workload": desc, "B": B, "Hq": Hq, "Hkv": Hkv, "N": N, "D": D, "tile": tile, "mode": args.mode,
+                   "step": "quantize Q,K (dual) + V repack + " + ("tile router + " if routed else "") + "fused attention"},
         "frac_mxfp4_peak": round(tflops / PEAK_FP4_TFLOPS, 5),
         "roofline": roofline,
     }

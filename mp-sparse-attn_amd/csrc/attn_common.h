@@ -74,6 +74,35 @@ __device__ __forceinline__ void load16_to_lds(const uint8_t* gsrc, uint8_t* lds_
                                      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
+// A wave-uniform pointer as a 64-bit value the compiler knows to be uniform (scalar registers).
+__device__ __forceinline__ uint64_t uniform_bits(const void* p) {
+    // the broadcast builtin returns a signed int: widen through uint32_t, or the low half sign-extends
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return (uint64_t)lo | ((uint64_t)hi << 32);
+}
+
+// The same load with the address split into a wave-uniform 64-bit base (scalar registers) and the lane's unsigned
+// 32-bit byte offset: no per-lane 64-bit pointers to keep or to compute.  Written as assembly (the builtin only
+// takes a full per-lane pointer); the compiler does not count these loads, so the kernel waits for them itself
+// (s_waitcnt vmcnt(0) before the barrier that publishes the data).
+__device__ __forceinline__ void load16_to_lds_sv(uint32_t lane_off, const uint8_t* wave_base, uint8_t* lds_wave_base) {
+    // the low 32 bits of a generic pointer into LDS are the LDS byte address (the aperture base has none set)
+    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_wave_base);
+    const uint64_t gb = uniform_bits(wave_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(base), "v"(lane_off), "s"(gb) : "memory", "m0");
+}
+
+// A scalar load of one list entry.  The compiler turns a plain load that follows a workgroup barrier into a vector
+// load plus a broadcast; as assembly it stays a scalar load.  The wait is part of the same statement (a register
+// that is still being loaded must not be visible to the compiler as holding a value), so callers place it where
+// a short stall costs nothing.
+__device__ __forceinline__ int scalar_load(const int32_t* uniform_ptr) {
+    int x;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(x) : "s"(uniform_bits(uniform_ptr)) : "memory");
+    return x;
+}
 
 // Tile-skipping variants of the general kernel (modes mxfp4 / mxfp8): attn_fwd_skip.hip
 int attn_skip_launch(const AttnArgs& a, int pv_dtype, hipStream_t st);

@@ -102,6 +102,21 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         if (tail_special && t == n_plain) return a.nt - 1;
         return i;
     };
+    // routed: the key tiles of steps t, t+1, t+2 are kept in scalar registers and the list entry of step t+3 is
+    // fetched a whole step before its first use -- a scalar load that is waited for in the middle of a step would
+    // also wait for the step's outstanding LDS reads (they share a counter)
+    int jq0 = 0, jq1 = 0, jq2 = 0;
+    if constexpr (ROUTED) {
+        jq0 = tile_at(0); jq1 = tile_at(1); jq2 = tile_at(2);
+    }
+    auto tile_rel = [&](int t, auto k_c) {               // key tile of step t + K, t being the step in progress
+        constexpr int K = decltype(k_c)::value;
+        if constexpr (ROUTED) return K == 0 ? jq0 : (K == 1 ? jq1 : jq2);
+        else return tile_at(t + K);
+    };
+    typedef std::integral_constant<int, 0> R0;
+    typedef std::integral_constant<int, 1> R1;
+    typedef std::integral_constant<int, 2> R2;
     auto step_is8 = [&](int t) {
         if constexpr (ROUTED) return t >= r4;
         return MODE == MPSA_MODE_MXFP8 || (MODE == MPSA_MODE_DIAG && t == nsteps - 1);
@@ -132,33 +147,36 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     };
 
     // ---- staging ----
-    auto issue_k4 = [&](int t) __attribute__((always_inline)) {           // 4-bit K tile of step t -> kbuf[t & 1], swizzled rows
-        const uint8_t* src = a.k4 + (khead_row + (int64_t)tile_at(t) * TILE) * G::ROW4;
+    const int wu = __builtin_amdgcn_readfirstlane(w);    // the wave index, known to be uniform
+    uint32_t koff[G::KI4];                                // this lane's byte offsets into a 4-bit K tile (swizzled rows)
+#pragma unroll
+    for (int c = 0; c < G::KI4; ++c) {
+        const int p = (w * G::KI4 + c) * 64 + lane;
+        const int row = p / G::CPR4, slot = p % G::CPR4;
+        const int cb = slot ^ ((row >> G::SH4) & (G::CPR4 - 1));
+        koff[c] = (uint32_t)(row * G::ROW4 + cb * 16);
+    }
+    auto issue_k4 = [&](int t, int j) __attribute__((always_inline)) {    // 4-bit K tile j (step t) -> kbuf[t & 1], swizzled rows
+        const uint8_t* src = a.k4 + (khead_row + (int64_t)j * TILE) * G::ROW4;
         uint8_t* dst = kbuf0 + (t & 1) * G::K_BYTES;
 #pragma unroll
-        for (int c = 0; c < G::KI4; ++c) {
-            const int ci = w * G::KI4 + c;
-            const int p = ci * 64 + lane;
-            const int row = p / G::CPR4, slot = p % G::CPR4;
-            const int cb = slot ^ ((row >> G::SH4) & (G::CPR4 - 1));
-            load16_to_lds(src + row * G::ROW4 + cb * 16, dst + ci * 1024);
-        }
+        for (int c = 0; c < G::KI4; ++c) load16_to_lds_sv(koff[c], src, dst + (wu * G::KI4 + c) * 1024);
     };
-    auto issue_v = [&](int t) __attribute__((always_inline)) {            // V tile of step t -> vbuf[t & 1], flat
-        const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)tile_at(t) * TILE) * (D * 2);
+    auto issue_v = [&](int t, int j) __attribute__((always_inline)) {     // V tile j (step t) -> vbuf[t & 1], flat
+        const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)j * TILE) * (D * 2);
         uint8_t* dst = vbuf0 + (t & 1) * G::V_BYTES;
 #pragma unroll
         for (int c = 0; c < G::VI; ++c) {
-            const int ci = w * G::VI + c;
-            load16_to_lds(src + ci * 1024 + lane * 16, dst + ci * 1024);
+            const int ci = wu * G::VI + c;
+            load16_to_lds_sv((uint32_t)lane * 16u, src + ci * 1024, dst + ci * 1024);
         }
     };
     // K operand of the coming step, in registers: 4-bit fragments come from LDS, 8-bit ones straight from global
     v4i kf4[HAS4 ? G::KB : 1][G::SST];
     v8i kf8[PRE8 ? G::KB : 1][G::SST];
     int ksc[G::KB];             // E8M0 bytes of this lane's key rows, shifted so bytes 0 / 2 belong to MX block h / 2+h
-    auto load_kscales = [&](int t, bool is8) __attribute__((always_inline)) {
-        const uint8_t* sp = (is8 ? a.ks8 : a.ks4) + (khead_row + (int64_t)tile_at(t) * TILE + r) * (D / 32);
+    auto load_kscales = [&](int j, bool is8) __attribute__((always_inline)) {
+        const uint8_t* sp = (is8 ? a.ks8 : a.ks4) + (khead_row + (int64_t)j * TILE + r) * (D / 32);
 #pragma unroll
         for (int kb = 0; kb < G::KB; ++kb) {
             const uint32_t sw = (D == 128) ? *reinterpret_cast<const uint32_t*>(sp + kb * 32 * (D / 32))
@@ -177,8 +195,8 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
                 kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * G::ROW4 + (((2 * s + h) ^ f) * 16));
         }
     };
-    auto load_kf8 = [&](int t, v8i (&dstf)[G::KB][G::SST]) __attribute__((always_inline)) {
-        const uint8_t* src = a.k8 + (khead_row + (int64_t)tile_at(t) * TILE + r) * G::ROW8 + h * 16;
+    auto load_kf8 = [&](int j, v8i (&dstf)[G::KB][G::SST]) __attribute__((always_inline)) {
+        const uint8_t* src = a.k8 + (khead_row + (int64_t)j * TILE + r) * G::ROW8 + h * 16;
 #pragma unroll
         for (int kb = 0; kb < G::KB; ++kb)
 #pragma unroll
@@ -208,15 +226,15 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
 
     // ---- prologue: V(0), K(0), K(1) on their way; operands of step 0 into registers ----
     const bool first8 = step_is8(0);
-    issue_v(0);
+    issue_v(0, tile_rel(0, R0{}));
     if constexpr (HAS4) {
-        if (n_k4 > 0) issue_k4(0);
-        if (n_k4 > 1) issue_k4(1);
+        if (n_k4 > 0) issue_k4(0, tile_rel(0, R0{}));
+        if (n_k4 > 1) issue_k4(1, tile_rel(0, R1{}));
     }
-    load_kscales(0, first8);
+    load_kscales(tile_rel(0, R0{}), first8);
     load_q(first8);
     if constexpr (PRE8) {
-        if (!ROUTED || first8) load_kf8(0, kf8);
+        if (!ROUTED || first8) load_kf8(tile_rel(0, R0{}), kf8);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0)
     __syncthreads();
@@ -229,7 +247,8 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         constexpr bool IS8 = decltype(is8_c)::value;
         constexpr bool MASKED = decltype(masked_c)::value;
         constexpr bool PREP = decltype(prep_c)::value;
-        const int j = tile_at(t);                          // key tile of this step
+        const int j = tile_rel(t, R0{});                   // key tile of this step
+        int jq3 = 0;
 
         // ---- S^T - m_run = K Q^T + (-m_run) ----
         v16f st[G::KB];
@@ -257,6 +276,12 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
                     st[kb] = score_mfma4(k8v, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
                 }
             }
+        }
+
+        // routed: fetch the list entry of step t + 3 while the matrix cores work on the scores (the operand reads
+        // from LDS are complete at this point, so the scalar load's wait holds up nothing else)
+        if constexpr (ROUTED) {
+            if (t + 3 < nsteps) jq3 = min(max(scalar_load(ord + t + 3), 0), a.nt - 1);
         }
 
         // ---- masks: causal on the diagonal tile, key tail on the last tile ----
@@ -342,9 +367,9 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
 
-        if (t + 1 < nsteps) issue_v(t + 1);
+        if (t + 1 < nsteps) issue_v(t + 1, tile_rel(t, R1{}));
         if constexpr (HAS4) {
-            if (t + 2 < n_k4) issue_k4(t + 2);
+            if (t + 2 < n_k4) issue_k4(t + 2, tile_rel(t, R2{}));
         }
 
         // ---- O^T += V^T P^T, V fragments prefetched PRE instructions ahead ----
@@ -358,9 +383,9 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         // operands of the next step: scales (and 8-bit K) from global memory, 4-bit K from LDS.  Past the last
         // step this reads a valid but unused tile.
         if constexpr (PREP) {
-            load_kscales(t + 1, IS8);
+            load_kscales(tile_rel(t, R1{}), IS8);
             if constexpr (PRE8) {
-                if constexpr (IS8) load_kf8(t + 1, kf8);
+                if constexpr (IS8) load_kf8(tile_rel(t, R1{}), kf8);
             }
             if constexpr (HAS4) {
                 if constexpr (!IS8) read_kf4(t + 1);
@@ -374,6 +399,9 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
                 if (idx + PRE < G::NV) vf[idx % PRE] = *reinterpret_cast<const typename P::vec*>(vl + (idx + PRE) * 1024);
                 acc[d] = P::mfma(cur, __builtin_bit_cast(typename P::vec, pk[kc >> 1][kc & 1]), acc[d]);
             }
+        }
+        if constexpr (ROUTED) {
+            jq0 = jq1; jq1 = jq2; jq2 = jq3;
         }
     };
 
@@ -389,16 +417,16 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         for (int t = 0; t < r4p; ++t) step(t, std::false_type{}, std::false_type{}, std::true_type{});
         for (int t = r4p; t < r4; ++t) step(t, std::false_type{}, std::true_type{}, std::true_type{});
         if (r4 > 0 && r4 < nsteps) {                   // otherwise the prologue already loaded the 8-bit operands
-            load_kscales(r4, true);
+            load_kscales(jq0, true);
             load_q(true);
-            load_kf8(r4, kf8);
+            load_kf8(jq0, kf8);
         }
         for (int t = r4; t < r8p; ++t) step(t, std::true_type{}, std::false_type{}, std::true_type{});
         for (int t = r8p; t < nsteps; ++t) step(t, std::true_type{}, std::true_type{}, std::true_type{});
     } else if constexpr (MODE == MPSA_MODE_DIAG) {
         if (tail_special) step(n_plain, std::false_type{}, std::true_type{}, std::true_type{});
         if (nsteps > 1) {                              // otherwise the prologue already loaded 8-bit Q and scales
-            load_kscales(nsteps - 1, true);
+            load_kscales(tile_at(nsteps - 1), true);
             load_q(true);
         }
         step(nsteps - 1, std::true_type{}, std::true_type{}, std::false_type{});
