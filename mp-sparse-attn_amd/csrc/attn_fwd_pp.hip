@@ -109,20 +109,25 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     };
 
     // ---- staging: every wave issues its share of each tile ----
-    auto issue_k4 = [&](int t) __attribute__((always_inline)) {
-        const uint8_t* src = a.k4 + (khead_row + (int64_t)t * TILE) * ROW4;
+    const int wu = __builtin_amdgcn_readfirstlane(w);    // the wave index, known to be uniform
+    uint32_t koff;                                        // this lane's byte offset into a 4-bit K tile (swizzled rows)
+    {
         const int p = w * 64 + lane;
         const int row = p / CPR4, slot = p % CPR4;
         const int cb = slot ^ ((row >> SH4) & (CPR4 - 1));
-        load16_to_lds(src + row * ROW4 + cb * 16, kbuf0 + (t & 1) * K_BYTES + w * 1024);
+        koff = (uint32_t)(row * ROW4 + cb * 16);
+    }
+    auto issue_k4 = [&](int t) __attribute__((always_inline)) {
+        const uint8_t* src = a.k4 + (khead_row + (int64_t)t * TILE) * ROW4;
+        load16_to_lds_sv(koff, src, kbuf0 + (t & 1) * K_BYTES + wu * 1024);
     };
     auto issue_v = [&](int t) __attribute__((always_inline)) {
         const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)t * TILE) * (D * 2);
         uint8_t* dst = vbuf0 + (t & 1) * V_BYTES;
 #pragma unroll
         for (int c = 0; c < VI; ++c) {
-            const int ci = w * VI + c;
-            load16_to_lds(src + ci * 1024 + lane * 16, dst + ci * 1024);
+            const int ci = wu * VI + c;
+            load16_to_lds_sv((uint32_t)lane * 16u, src + ci * 1024, dst + ci * 1024);
         }
     };
     // barrier of step t: this wave's pieces of V(t) and K(t+1) have landed, after it everybody's have and everybody
