@@ -208,30 +208,37 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     // (bytes h and 2+h of the lane half h).  The word is read once, with the even step's operands, shifted right by
     // 8h when that step starts, and handed on to the odd step's set, whose instructions select byte 2.
     struct Frag { v8i a[4], b[4]; int sa[4], sb[4]; uint32_t ra[4], rb[4]; };
+    // Wide path, 4-bit codes: a row's 16 scale bytes of the current group are read from LDS ONCE per group with one
+    // 128-bit read per row (16 consecutive rows x 16 bytes are conflict-free; a 32-bit read per step pair at this
+    // 16-byte row pitch is a four-way bank conflict, and those conflicts were 38 % of the kernel's LDS cycles).
+    // Dword k of a row covers step pair k of the group.  With 8-bit codes the operand sets fill the register file:
+    // 32 (or, reading half a group at a time, 16) more registers spill and the kernel gets slower, so that path
+    // keeps the 32-bit read per step pair.
+    constexpr bool GREAD = WIDE && FP4;
+    v4i w_a[4], w_b[4];
 
     // reads operands of step s of stage kt out of the ring: part 0 the B fragments and their scale bytes,
-    // part 1 the A fragments and theirs
-    auto read_part = [&](Frag& f, const Frag& even, int kt, int s, int part, bool fresh) __attribute__((always_inline)) {
+    // part 1 the A fragments and theirs.  grp >= 0 (wide path): also this part's scale rows of group grp.
+    auto read_part = [&](Frag& f, const Frag& even, int kt, int s, int part, bool fresh, int grp) __attribute__((always_inline)) {
         const uint8_t* st = smem + (kt % NSTAGE) * STAGE_BYTES;
-        // the row's scale word of this step pair
-        const uint8_t* sc;
-        int sstride;
-        if constexpr (WIDE) {
-            sc = scg + ((kt / GROUP) & 1) * 2 * SCG_BYTES + 4 * (FP4 ? kt % GROUP : (kt % GROUP) >> 1);
-            sstride = 16;
-        } else {
-            sc = st + 2 * OP_BYTES;
-            sstride = 4;
-        }
         const bool isb = part == 0;
         const uint8_t* lx = isb ? st + OP_BYTES : st;
-        if (isb) sc += WIDE ? SCG_BYTES : SC_BYTES;
+        // the row's scale word of this step pair (paths without the per-group read)
+        const uint8_t* sc = WIDE ? scg + ((kt / GROUP) & 1) * 2 * SCG_BYTES + 4 * (FP4 ? kt % GROUP : (kt % GROUP) >> 1) + (isb ? SCG_BYTES : 0)
+                                 : st + 2 * OP_BYTES + (isb ? SC_BYTES : 0);
+        constexpr int sstride = WIDE ? 16 : 4;
+        const uint8_t* sg = scg + (grp & 1) * 2 * SCG_BYTES + (isb ? SCG_BYTES : 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int row = (isb ? wn : wm) * 128 + i * 32 + r;
             const int off = isb ? offb[i] : offa[i], swz = isb ? swz_b[i] : swz_a[i];
             v8i& fx = isb ? f.b[i] : f.a[i];
-            if (fresh) {
+            if constexpr (GREAD) {
+                if (grp >= 0) (isb ? w_b[i] : w_a[i]) = *reinterpret_cast<const v4i*>(sg + row * 16);
+                if (!fresh) {
+                    if (isb) f.sb[i] = even.sb[i]; else f.sa[i] = even.sa[i];
+                }
+            } else if (fresh) {
                 (isb ? f.rb[i] : f.ra[i]) = *reinterpret_cast<const uint32_t*>(sc + row * sstride);
             } else {
                 if (isb) f.sb[i] = even.sb[i]; else f.sa[i] = even.sa[i];
@@ -261,13 +268,21 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     // loads of stage lkt into the buffer of stage lkt-NSTAGE (two per row; on the wide path the first stage of
     // a group also brings the next group's scale bytes), so that the matrix pipe keeps running while they issue.
     // `odd`: cur is the odd step of its pair (its scale words were handed on by the even step's set)
-    auto step = [&](Frag& cur, Frag& nxt, int nkt, int ns, bool refill, int lkt, bool odd) __attribute__((always_inline)) {
+    // wide path: `kd` = which dword of the group's scale rows an even step uses; `fetch_grp` >= 0: the refill also
+    // fetches that group's scale bytes; `read_grp` >= 0: the operand reads also bring that group's scale rows into
+    // registers (the step after the group's last even step, so the registers are free)
+    auto step = [&](Frag& cur, Frag& nxt, int nkt, int ns, bool refill, int lkt, bool odd, int kd, int fetch_grp, int read_grp) __attribute__((always_inline)) {
         constexpr int PER = FP4 ? 2 : 3;                   // LDS reads issued behind each matrix instruction
         if (!odd) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                cur.sa[i] = (int)(cur.ra[i] >> (8 * h));
-                cur.sb[i] = (int)(cur.rb[i] >> (8 * h));
+                if constexpr (GREAD) {
+                    cur.sa[i] = (int)((uint32_t)w_a[i][kd] >> (8 * h));
+                    cur.sb[i] = (int)((uint32_t)w_b[i][kd] >> (8 * h));
+                } else {
+                    cur.sa[i] = (int)(cur.ra[i] >> (8 * h));
+                    cur.sb[i] = (int)(cur.rb[i] >> (8 * h));
+                }
             }
         }
 #pragma unroll
@@ -275,11 +290,11 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
             if (refill) {
                 issue_part(lkt, i);
                 if constexpr (WIDE) {
-                    if (i == 3 && (lkt - NSTAGE) % GROUP == 0) issue_scales((lkt - NSTAGE) / GROUP + 1);
+                    if (i == 3 && fetch_grp >= 0) issue_scales(fetch_grp);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (i < 2) read_part(nxt, cur, nkt, ns, i, odd);          // the step after an odd one starts a new pair
+            if (i < 2) read_part(nxt, cur, nkt, ns, i, odd, read_grp);   // the step after an odd one starts a new pair
             multiply_row(cur, i, odd);
             if (i < 2) {
 #pragma unroll
@@ -313,23 +328,39 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
     }
-    read_part(f0, f0, 0, 0, 0, true);
-    read_part(f0, f0, 0, 0, 1, true);
-    if constexpr (FP4) {
+    read_part(f0, f0, 0, 0, 0, true, GREAD ? 0 : -1);
+    read_part(f0, f0, 0, 0, 1, true, GREAD ? 0 : -1);
+    // wide path without the per-group read: the group whose scale bytes the refill of stage kt also fetches
+    auto fetch_at = [&](int kt) { return (WIDE && kt % GROUP == 0) ? kt / GROUP + 1 : -1; };
+    if constexpr (GREAD) {
+        // one trip = one scale group (4 stages = four step pairs), unrolled so that the dword a pair takes from the
+        // group's scale rows, the refill that fetches the next group's scale bytes and the step that reads them
+        // into registers are all fixed at compile time
+        for (int kt0 = 0; kt0 < KT; kt0 += GROUP) {
+            const int grp = kt0 / GROUP;
+#pragma unroll
+            for (int u = 0; u < GROUP; ++u) {
+                const int kt = kt0 + u;
+                step(f0, f1, kt, 1, false, 0, false, u, -1, -1);
+                publish();
+                step(f1, f0, kt + 1, 0, true, kt + NSTAGE, true, 0, u == 0 ? grp + 1 : -1, u == GROUP - 1 ? grp + 1 : -1);
+            }
+        }
+    } else if constexpr (FP4) {
         // a stage is two steps: the second step's operands load under the first step's instructions, and the
         // next stage's first operands (after the barrier that publishes it) under the second step's
         for (int kt = 0; kt < KT; ++kt) {
-            step(f0, f1, kt, 1, false, 0, false);
+            step(f0, f1, kt, 1, false, 0, false, 0, -1, -1);
             publish();
-            step(f1, f0, kt + 1, 0, true, kt + NSTAGE, true);
+            step(f1, f0, kt + 1, 0, true, kt + NSTAGE, true, 0, fetch_at(kt), -1);
         }
     } else {
         // a stage is one step; two stages per trip so that the two operand sets keep their registers
         for (int kt = 0; kt < KT; kt += 2) {
             publish();
-            step(f0, f1, kt + 1, 0, true, kt + NSTAGE, false);
+            step(f0, f1, kt + 1, 0, true, kt + NSTAGE, false, 0, fetch_at(kt), -1);
             publish();
-            step(f1, f0, kt + 2, 0, true, kt + 1 + NSTAGE, true);
+            step(f1, f0, kt + 2, 0, true, kt + 1 + NSTAGE, true, 0, fetch_at(kt + 1), -1);
         }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
