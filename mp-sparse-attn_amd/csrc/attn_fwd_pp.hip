@@ -195,6 +195,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         }
     };
     auto softmax = [&](bool first, auto masked_c) __attribute__((always_inline)) {
+        __builtin_amdgcn_s_setprio(0);
         if constexpr (decltype(masked_c)::value) {      // diagonal tile: keys after the query are dead
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb)
@@ -240,6 +241,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                     if (e & 2) ps1 = P::add2(pp, ps1); else ps0 = P::add2(pp, ps0);
                 }
         l_run += ps0 + ps1;
+        __builtin_amdgcn_s_setprio(2);
     };
     auto pv = [&](int t) __attribute__((always_inline)) {
         constexpr int PRE = 8;
