@@ -443,9 +443,39 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     const float l_tot = sum_lane_pair(l_run);
     const float inv = (ROUTED && !(l_tot > 0.0f)) ? 0.0f : 1.0f / l_tot;   // routed: a row with every tile skipped gives zeros
     const int q_global = i * TILE + q_local;
-    if (q_global < a.nq) {
-        uint8_t* orow = static_cast<uint8_t*>(a.o);
-        const int64_t off = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh + (int64_t)q_global * a.o_sn;
+    uint8_t* orow = static_cast<uint8_t*>(a.o);
+    const int64_t off = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh + (int64_t)q_global * a.o_sn;
+    if (a.o_dtype != MPSA_F32 && ((a.o_sn | a.o_sh | a.o_sb) & 7) == 0 && (reinterpret_cast<uintptr_t>(a.o) & 15) == 0) {
+        // 16-bit output: the two lanes of a query trade register groups (lane half 0 hands over dims 8..11 of every
+        // 16 and receives dims 4..7), so that each lane owns 8 consecutive dims and stores 16 bytes at a time.
+        // Every lane takes part in the exchange; only queries inside the sequence are stored.
+#pragma unroll
+        for (int d = 0; d < G::NDB; ++d)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                int x[2], y[2];                           // packed dims 16u+4h .. +3 (x) and 16u+8+4h .. +3 (y)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const float x0 = acc[d][8 * u + 2 * c] * inv, x1 = acc[d][8 * u + 2 * c + 1] * inv;
+                    const float y0 = acc[d][8 * u + 4 + 2 * c] * inv, y1 = acc[d][8 * u + 4 + 2 * c + 1] * inv;
+                    if (a.o_dtype == MPSA_BF16) {
+                        typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+                        x[c] = __builtin_bit_cast(int, (v2bf){(__bf16)x0, (__bf16)x1});
+                        y[c] = __builtin_bit_cast(int, (v2bf){(__bf16)y0, (__bf16)y1});
+                    } else {
+                        typedef _Float16 v2hh __attribute__((ext_vector_type(2)));
+                        x[c] = __builtin_bit_cast(int, (v2hh){(_Float16)x0, (_Float16)x1});
+                        y[c] = __builtin_bit_cast(int, (v2hh){(_Float16)y0, (_Float16)y1});
+                    }
+                    // swap x of lanes 32-63 with y of lanes 0-31: half 0 ends with dims 16u .. 16u+7 in (x, y),
+                    // half 1 with dims 16u+8 .. 16u+15
+                    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x[c]), "+v"(y[c]));
+                }
+                const int dim = 32 * d + 16 * u + 8 * h;
+                const v4i pk8 = {x[0], x[1], y[0], y[1]};
+                if (q_global < a.nq) *reinterpret_cast<v4i*>(orow + (off + dim) * 2) = pk8;
+            }
+    } else if (q_global < a.nq) {
 #pragma unroll
         for (int d = 0; d < G::NDB; ++d)
 #pragma unroll
