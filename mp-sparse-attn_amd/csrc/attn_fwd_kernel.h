@@ -18,14 +18,21 @@ struct Geom {
     static constexpr int K_BYTES = TILE * ROW4;   // one 4-bit K tile
     static constexpr int V_BYTES = TILE * D * 2;
     static constexpr int SMEM = 2 * K_BYTES + 2 * V_BYTES;
+    static constexpr int CPR8 = ROW8 / 16;        // 16-byte chunks per 8-bit K row (4 | 8)
+    static constexpr int SH8 = CPR8 == 4 ? 2 : 1; // log2(rows per 256 bytes)
+    static constexpr int K8_BYTES = TILE * ROW8;  // one 8-bit K tile: exactly the two 4-bit buffers
+    static constexpr int KI8 = K8_BYTES / 1024 / NW;
     static constexpr int KI4 = K_BYTES / 1024 / NW;                   // direct-load instructions per wave
     static constexpr int VI = V_BYTES / 1024 / NW;
     static constexpr int NV = KB * 2 * NDB;       // V fragments (= P.V matrix instructions) per tile
 };
 
-// MODE is compile-time: an all-4-bit run carries no 8-bit code, an all-8-bit run keeps the next tile's 8-bit K
-// fragments in registers (read from global memory one step ahead), and a "diag" run pipelines 4-bit tiles through
-// LDS and fetches its single 8-bit tile when it gets there.
+// MODE is compile-time: an all-4-bit run carries no 8-bit code, and a "diag" run pipelines 4-bit tiles through
+// LDS and fetches its single 8-bit tile straight from global memory when it gets there.  Runs with many 8-bit tiles
+// (all-8-bit, routed) stage them through LDS as well: an 8-bit K tile is as large as the two 4-bit buffers together,
+// so it has ONE buffer, and the registers that hold the coming step's fragments are its second one.  That takes a
+// second barrier per 8-bit step: barrier A publishes V(t) and K8(t+1); every wave pulls the K8(t+1) fragments into
+// registers; barrier B says that everyone has, and only then the loads of K8(t+2) go out.
 //
 // A "routed" run (MPSA_MODE_ROUTED) walks a visiting list made by the tile router (route.hip): the 4-bit tiles through
 // the LDS pipeline, then the 8-bit tiles with their K fragments prefetched from global memory; inside each precision
@@ -162,6 +169,21 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
         for (int c = 0; c < G::KI4; ++c) load16_to_lds_sv(koff[c], src, dst + (wu * G::KI4 + c) * 1024);
     };
+    uint32_t koff8[PRE8 ? G::KI8 : 1];                    // the same for an 8-bit K tile
+    if constexpr (PRE8) {
+#pragma unroll
+        for (int c = 0; c < G::KI8; ++c) {
+            const int p = (w * G::KI8 + c) * 64 + lane;
+            const int row = p / G::CPR8, slot = p % G::CPR8;
+            const int cb = slot ^ ((row >> G::SH8) & (G::CPR8 - 1));
+            koff8[c] = (uint32_t)(row * G::ROW8 + cb * 16);
+        }
+    }
+    auto issue_k8 = [&](int j) __attribute__((always_inline)) {           // 8-bit K tile j -> the K area (one buffer), swizzled rows
+        const uint8_t* src = a.k8 + (khead_row + (int64_t)j * TILE) * G::ROW8;
+#pragma unroll
+        for (int c = 0; c < (PRE8 ? G::KI8 : 0); ++c) load16_to_lds_sv(koff8[c], src, kbuf0 + (wu * G::KI8 + c) * 1024);
+    };
     auto issue_v = [&](int t, int j) __attribute__((always_inline)) {     // V tile j (step t) -> vbuf[t & 1], flat
         const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)j * TILE) * (D * 2);
         uint8_t* dst = vbuf0 + (t & 1) * G::V_BYTES;
@@ -195,17 +217,28 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
                 kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * G::ROW4 + (((2 * s + h) ^ f) * 16));
         }
     };
-    auto load_kf8 = [&](int j, v8i (&dstf)[G::KB][G::SST]) __attribute__((always_inline)) {
-        const uint8_t* src = a.k8 + (khead_row + (int64_t)j * TILE + r) * G::ROW8 + h * 16;
+    auto read_kf8 = [&]() __attribute__((always_inline)) {                // the staged 8-bit K tile -> fragments
 #pragma unroll
-        for (int kb = 0; kb < G::KB; ++kb)
+        for (int kb = 0; kb < (PRE8 ? G::KB : 0); ++kb) {
+            const int krow = 32 * kb + r;
+            const int f = (krow >> G::SH8) & (G::CPR8 - 1);
 #pragma unroll
             for (int s = 0; s < G::SST; ++s) {
                 // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
-                const v4i x0 = *reinterpret_cast<const v4i*>(src + kb * 32 * G::ROW8 + s * 64);
-                const v4i x1 = *reinterpret_cast<const v4i*>(src + kb * 32 * G::ROW8 + s * 64 + 32);
-                dstf[kb][s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+                const v4i x0 = *reinterpret_cast<const v4i*>(kbuf0 + krow * G::ROW8 + (((4 * s + h) ^ f) * 16));
+                const v4i x1 = *reinterpret_cast<const v4i*>(kbuf0 + krow * G::ROW8 + (((4 * s + h + 2) ^ f) * 16));
+                kf8[kb][s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
             }
+        }
+    };
+    // barrier B of an 8-bit step (and of the switch to 8-bit tiles): every wave has the staged tile's fragments in
+    // registers, so the one buffer may take the next tile
+    auto k8_handover = [&](bool more, int j_next) __attribute__((always_inline)) {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0xC07F);            // lgkmcnt(0): the fragment reads have arrived
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) issue_k8(j_next);
     };
 
     v16f acc[G::NDB];
@@ -231,14 +264,20 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         if (n_k4 > 0) issue_k4(0, tile_rel(0, R0{}));
         if (n_k4 > 1) issue_k4(1, tile_rel(0, R1{}));
     }
+    if constexpr (PRE8) {
+        if (!ROUTED || first8) issue_k8(tile_rel(0, R0{}));
+    }
     load_kscales(tile_rel(0, R0{}), first8);
     load_q(first8);
-    if constexpr (PRE8) {
-        if (!ROUTED || first8) load_kf8(tile_rel(0, R0{}), kf8);
-    }
     __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0)
     __syncthreads();
     if constexpr (HAS4) read_kf4(0);
+    if constexpr (PRE8) {
+        if (!ROUTED || first8) {
+            read_kf8();
+            k8_handover(nsteps > 1, tile_rel(0, R1{}));
+        }
+    }
 
     // One step = one key tile.  IS8 / MASKED are compile-time so the common step (4-bit, unmasked) carries no
     // branches or mask arithmetic.
@@ -372,6 +411,15 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
             if (t + 2 < n_k4) issue_k4(t + 2, tile_rel(t, R2{}));
         }
 
+        // 8-bit steps: the K8(t+1) fragments, published by this step's barrier, go into registers first (before the
+        // V fragments are fetched, so that the two sets are not in flight together); then barrier B and K8(t+2)
+        if constexpr (PREP && PRE8) {
+            if constexpr (IS8) {
+                read_kf8();
+                k8_handover(t + 2 < nsteps, tile_rel(t, R2{}));
+            }
+        }
+
         // ---- O^T += V^T P^T, V fragments prefetched PRE instructions ahead ----
         constexpr int PRE = 8;
         const uint8_t* vl = vbuf0 + (t & 1) * G::V_BYTES + lane * 16;
@@ -384,9 +432,6 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         // step this reads a valid but unused tile.
         if constexpr (PREP) {
             load_kscales(tile_rel(t, R1{}), IS8);
-            if constexpr (PRE8) {
-                if constexpr (IS8) load_kf8(tile_rel(t, R1{}), kf8);
-            }
             if constexpr (HAS4) {
                 if constexpr (!IS8) read_kf4(t + 1);
             }
@@ -417,9 +462,15 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         for (int t = 0; t < r4p; ++t) step(t, std::false_type{}, std::false_type{}, std::true_type{});
         for (int t = r4p; t < r4; ++t) step(t, std::false_type{}, std::true_type{}, std::true_type{});
         if (r4 > 0 && r4 < nsteps) {                   // otherwise the prologue already loaded the 8-bit operands
+            // the 4-bit buffers become the 8-bit tile's single buffer: nothing that matters is read from them any
+            // more (a slower wave may still fetch fragments of a 4-bit step that does not exist)
+            issue_k8(jq0);
             load_kscales(jq0, true);
             load_q(true);
-            load_kf8(jq0, kf8);
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+            read_kf8();
+            k8_handover(r4 + 1 < nsteps, jq1);
         }
         for (int t = r4; t < r8p; ++t) step(t, std::true_type{}, std::false_type{}, std::true_type{});
         for (int t = r8p; t < nsteps; ++t) step(t, std::true_type{}, std::true_type{}, std::true_type{});
