@@ -155,42 +155,45 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
 
     // ---- staging ----
     const int wu = __builtin_amdgcn_readfirstlane(w);    // the wave index, known to be uniform
-    uint32_t koff[G::KI4];                                // this lane's byte offsets into a 4-bit K tile (swizzled rows)
-#pragma unroll
-    for (int c = 0; c < G::KI4; ++c) {
-        const int p = (w * G::KI4 + c) * 64 + lane;
-        const int row = p / G::CPR4, slot = p % G::CPR4;
-        const int cb = slot ^ ((row >> G::SH4) & (G::CPR4 - 1));
-        koff[c] = (uint32_t)(row * G::ROW4 + cb * 16);
-    }
+    // Lane offsets of the staging loads are recomputed where they are used (a handful of integer instructions)
+    // from a lane index the compiler cannot see through: kept in registers across the loops of a routed run they
+    // get spilled, and a reload in front of a load instruction costs a memory round trip per step.
+    auto opaque_lane = [&]() __attribute__((always_inline)) {
+        int ln = lane;
+        if constexpr (ROUTED) asm volatile("" : "+v"(ln));
+        return ln;
+    };
     auto issue_k4 = [&](int t, int j) __attribute__((always_inline)) {    // 4-bit K tile j (step t) -> kbuf[t & 1], swizzled rows
         const uint8_t* src = a.k4 + (khead_row + (int64_t)j * TILE) * G::ROW4;
         uint8_t* dst = kbuf0 + (t & 1) * G::K_BYTES;
+        const int ln = opaque_lane();
 #pragma unroll
-        for (int c = 0; c < G::KI4; ++c) load16_to_lds_sv(koff[c], src, dst + (wu * G::KI4 + c) * 1024);
-    };
-    uint32_t koff8[PRE8 ? G::KI8 : 1];                    // the same for an 8-bit K tile
-    if constexpr (PRE8) {
-#pragma unroll
-        for (int c = 0; c < G::KI8; ++c) {
-            const int p = (w * G::KI8 + c) * 64 + lane;
-            const int row = p / G::CPR8, slot = p % G::CPR8;
-            const int cb = slot ^ ((row >> G::SH8) & (G::CPR8 - 1));
-            koff8[c] = (uint32_t)(row * G::ROW8 + cb * 16);
+        for (int c = 0; c < G::KI4; ++c) {
+            const int p = (wu * G::KI4 + c) * 64 + ln;
+            const int row = p / G::CPR4, slot = p % G::CPR4;
+            const int cb = slot ^ ((row >> G::SH4) & (G::CPR4 - 1));
+            load16_to_lds_sv((uint32_t)(row * G::ROW4 + cb * 16), src, dst + (wu * G::KI4 + c) * 1024);
         }
-    }
+    };
     auto issue_k8 = [&](int j) __attribute__((always_inline)) {           // 8-bit K tile j -> the K area (one buffer), swizzled rows
         const uint8_t* src = a.k8 + (khead_row + (int64_t)j * TILE) * G::ROW8;
+        const int ln = opaque_lane();
 #pragma unroll
-        for (int c = 0; c < (PRE8 ? G::KI8 : 0); ++c) load16_to_lds_sv(koff8[c], src, kbuf0 + (wu * G::KI8 + c) * 1024);
+        for (int c = 0; c < (PRE8 ? G::KI8 : 0); ++c) {
+            const int p = (wu * G::KI8 + c) * 64 + ln;
+            const int row = p / G::CPR8, slot = p % G::CPR8;
+            const int cb = slot ^ ((row >> G::SH8) & (G::CPR8 - 1));
+            load16_to_lds_sv((uint32_t)(row * G::ROW8 + cb * 16), src, kbuf0 + (wu * G::KI8 + c) * 1024);
+        }
     };
     auto issue_v = [&](int t, int j) __attribute__((always_inline)) {     // V tile j (step t) -> vbuf[t & 1], flat
         const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)j * TILE) * (D * 2);
         uint8_t* dst = vbuf0 + (t & 1) * G::V_BYTES;
+        const uint32_t lo = (uint32_t)opaque_lane() * 16u;
 #pragma unroll
         for (int c = 0; c < G::VI; ++c) {
             const int ci = wu * G::VI + c;
-            load16_to_lds_sv((uint32_t)lane * 16u, src + ci * 1024, dst + ci * 1024);
+            load16_to_lds_sv(lo, src + ci * 1024, dst + ci * 1024);
         }
     };
     // K operand of the coming step, in registers: 4-bit fragments come from LDS, 8-bit ones straight from global
@@ -422,7 +425,7 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
 
         // ---- O^T += V^T P^T, V fragments prefetched PRE instructions ahead ----
         constexpr int PRE = 8;
-        const uint8_t* vl = vbuf0 + (t & 1) * G::V_BYTES + lane * 16;
+        const uint8_t* vl = vbuf0 + (t & 1) * G::V_BYTES + opaque_lane() * 16;
         typename P::vec vf[PRE];
         if (keep) {
 #pragma unroll
