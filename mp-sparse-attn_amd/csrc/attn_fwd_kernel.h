@@ -156,11 +156,11 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     // ---- staging ----
     const int wu = __builtin_amdgcn_readfirstlane(w);    // the wave index, known to be uniform
     // Lane offsets of the staging loads are recomputed where they are used (a handful of integer instructions)
-    // from a lane index the compiler cannot see through: kept in registers across the loops of a routed run they
-    // get spilled, and a reload in front of a load instruction costs a memory round trip per step.
+    // from a lane index the compiler cannot see through in the variants that are short of registers: kept there
+    // across the loops they get spilled, and a reload in front of a load instruction costs a memory round trip per step.
     auto opaque_lane = [&]() __attribute__((always_inline)) {
         int ln = lane;
-        if constexpr (ROUTED) asm volatile("" : "+v"(ln));
+        if constexpr (ROUTED || SKIP || MODE == MPSA_MODE_MXFP8) asm volatile("" : "+v"(ln));
         return ln;
     };
     auto issue_k4 = [&](int t, int j) __attribute__((always_inline)) {    // 4-bit K tile j (step t) -> kbuf[t & 1], swizzled rows
