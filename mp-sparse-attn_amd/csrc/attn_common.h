@@ -74,15 +74,6 @@ __device__ __forceinline__ void load16_to_lds(const uint8_t* gsrc, uint8_t* lds_
                                      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
-// A wave-uniform pointer as a 64-bit value the compiler knows to be uniform (scalar registers).
-__device__ __forceinline__ uint64_t uniform_bits(const void* p) {
-    // the broadcast builtin returns a signed int: widen through uint32_t, or the low half sign-extends
-    const uint64_t v = (uint64_t)(uintptr_t)p;
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
-    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
-    return (uint64_t)lo | ((uint64_t)hi << 32);
-}
-
 // The same load with the address split into a wave-uniform 64-bit base (scalar registers) and the lane's unsigned
 // 32-bit byte offset: no per-lane 64-bit pointers to keep or to compute.  Written as assembly (the builtin only
 // takes a full per-lane pointer); the compiler does not count these loads, so the kernel waits for them itself

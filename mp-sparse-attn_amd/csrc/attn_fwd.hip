@@ -26,9 +26,9 @@
 // operand reads of 16 consecutive rows hit 16 distinct 4-bank groups.  Both are double-buffered and the loop
 // needs ONE barrier per tile: after the barrier of step t a wave issues the loads of V(t+1) and K(t+2), pulls the
 // K(t+1) fragments from LDS into registers and runs P.V of step t; the next step's score MFMAs then start from
-// registers.  8-bit K tiles (the diagonal tile of "diag" runs, every tile of "mxfp8" runs) bypass LDS: each lane
-// reads its fragments from global memory one step ahead.  K scales are read from global memory one step ahead
-// as well.  80 KiB of LDS and at most 256 registers per workgroup let two workgroups share a CU, so one's matrix
+// registers.  The single 8-bit K tile of a "diag" run bypasses LDS (each lane reads its fragments from global memory);
+// runs with many 8-bit tiles ("mxfp8", routed) stage them through the same LDS area, one buffer plus the fragment
+// registers (see attn_fwd_kernel.h).  K scales are read from global memory one step ahead.  80 KiB of LDS and at most 256 registers per workgroup let two workgroups share a CU, so one's matrix
 // instructions overlap the other's softmax VALU work.
 #include "attn_fwd_kernel.h"
 

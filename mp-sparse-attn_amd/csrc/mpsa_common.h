@@ -41,3 +41,12 @@ static inline hipError_t mpsa_reserve_lds(const void* kern, int bytes, bool* don
 
 __device__ __forceinline__ float mpsa_u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t mpsa_f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// A wave-uniform pointer as a 64-bit value the compiler knows to be uniform (scalar registers).
+__device__ __forceinline__ uint64_t uniform_bits(const void* p) {
+    // the broadcast builtin returns a signed int: widen through uint32_t, or the low half sign-extends
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return (uint64_t)lo | ((uint64_t)hi << 32);
+}
