@@ -82,7 +82,9 @@ template <> __device__ __forceinline__ OutE5M2 cvt_out<OutE5M2>(float v) {
 template <int BYTES>
 __device__ __forceinline__ void load_to_lds(uint32_t lane_off, const uint8_t* wave_base, uint8_t* lds_wave_base) {
     // address = wave-uniform base (scalar registers) + the lane's unsigned 32-bit byte offset
-    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds_wave_base);
+    // the low 32 bits of a generic pointer into LDS are the LDS byte address (a cast to the LDS address space
+    // would add a null check per load)
+    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_wave_base);
     const uint64_t gb = (uint64_t)(uintptr_t)wave_base;
     if constexpr (BYTES == 16)
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(base), "v"(lane_off), "s"(gb) : "memory", "m0");
