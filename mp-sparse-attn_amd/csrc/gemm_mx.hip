@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     uint8_t* const scg = smem + NSTAGE * STAGE_BYTES;  // wide path: [group parity][operand][row][16]
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the wave index, known to be uniform
     const int wm = wave >> 1, wn = wave & 1;
     const int h = lane >> 5, r = lane & 31;
 
