@@ -108,6 +108,38 @@ def test_routed_entry_point_and_sparsity():
         mxfp_attn(q.to(DEV), k.to(DEV), v.to(DEV), block_scale_type="mxfp4", route_thresh=0.5, smooth_k=False)
 
 
+def test_routed_e5m2_smooth_k_fp16_and_nhd_layout():
+    """The reference's own 8-bit format (E5M2), fp16 inputs, K smoothing and the "NHD" layout through the routed path."""
+    q, k, v = _inputs(1, 4, 2, 3 * 64 + 21, 64, seed=370)
+    q, k, v = q.to(torch.float16), k.to(torch.float16), v.to(torch.float16)
+    N = q.shape[2]
+    ks = O.smooth_k(k)
+    ops = prepare_operands(q.to(DEV), ks.to(DEV), v.to(DEV), 64, "routed_e5")
+    cls = route_tiles(ops, True, 0.5, 0.2)[0].cpu().numpy()
+    assert {1, 2} <= set(np.unique(cls).tolist())
+    want = O.attn_mx(q, ks, v, tile=64, causal=True, mode="routed", route=cls, fmt8=O.FMT_E5M2)
+    got = mxfp_attn_kernel(q.transpose(1, 2).contiguous().to(DEV), ks.transpose(1, 2).contiguous().to(DEV),
+                           v.transpose(1, 2).contiguous().to(DEV), is_causal=True, tensor_layout="NHD",
+                           output_dtype=torch.float16, block_scale_type="routed_e5", tile=64, route_thresh=0.5,
+                           skip_thresh=0.2)
+    assert got.shape == (1, N, 4, 64)
+    _compare(got.transpose(1, 2), want, "routed_e5 NHD")
+    # smoothing inside the wrapper: same map inputs up to the 16-bit mean's last place, so compare the output only
+    got2 = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=True, smooth_k=True, output_dtype=torch.float16,
+                            block_scale_type="routed_e5", tile=64, route_thresh=0.5, skip_thresh=None)
+    want2 = O.attn_mx(q, k, v, tile=64, causal=True, mode="routed", smooth_k=True, fmt8=O.FMT_E5M2,
+                      route=O.route_tiles(*_oracle_scales(q, O.smooth_k(k), 64), 64, True, 0.5, None))
+    _compare(got2, want2, "routed_e5 smooth_k")
+
+
+def _oracle_scales(q, k, tile):
+    """Padded 4-bit scale bytes of Q (with the softmax pre-scale) and K from the oracle's quantizer."""
+    def padded(x, pre):
+        sc = np.asarray(O.quantize_mx(x, pre, O.FMT_E2M1)[1])
+        return np.pad(sc, ((0, 0), (0, 0), (0, (-x.shape[2]) % tile), (0, 0)))
+    return padded(q, O.q_pre_scale(q.shape[-1], None)), padded(k, 1.0)
+
+
 @pytest.mark.parametrize("N", [512, 512 + 77])
 def test_routed_reproduces_fixed_modes_bit_for_bit(N):
     """Non-causal runs of the general kernel: thresholds off = every tile 4-bit = mode mxfp4; a hand-made list with
