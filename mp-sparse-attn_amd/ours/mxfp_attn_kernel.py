@@ -87,6 +87,8 @@ def attention_from_operands(ops, out, is_causal, skip_thresh=None, skipped=None,
     B, Hq, Hkv, Nq, N, D = ops["shape"]
     dev = out.device
     if ops["mode"] == _lib.MODE_ROUTED:
+        if route is None:
+            raise ValueError("routed operands need route=(cls, order, counts) from route_tiles()")
         _, order, counts = route
         with torch.cuda.device(dev):
             _lib.check(_lib.lib().mpsa_attn_fwd_routed(
