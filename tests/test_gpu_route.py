@@ -76,6 +76,30 @@ def test_route_many_key_tiles_and_thresholds():
         assert np.array_equal(order.cpu().numpy(), want_order), (hi, lo)
 
 
+def test_route_golden_vectors_on_gpu():
+    """The HIP router against the committed vectors (scale bytes in, class map / lists / run lengths out)."""
+    import os
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "route_vectors.npz"))
+    L = _lib.lib()
+    for name in "abcde":
+        tile, D, n_keys, causal = (int(x) for x in d[name + "_meta"])
+        hi, lo = (float(x) for x in d[name + "_thresh"])
+        qs, ks = torch.from_numpy(d[name + "_qs"]).to(DEV), torch.from_numpy(d[name + "_ks"]).to(DEV)
+        B, Hq, nq_pad, _ = qs.shape
+        Hkv, nk_pad = ks.shape[1], ks.shape[2]
+        nq = n_keys if nq_pad == nk_pad else nq_pad
+        ntq, ntk = nq_pad // tile, nk_pad // tile
+        work = torch.empty(L.mpsa_route_workspace(B, Hq, Hkv, nq, n_keys, D, tile), dtype=torch.uint8, device=DEV)
+        cls = torch.empty((B, Hq, ntq, ntk), dtype=torch.uint8, device=DEV)
+        order = torch.empty((B, Hq, ntq, ntk), dtype=torch.int32, device=DEV)
+        counts = torch.empty((B, Hq, ntq, 4), dtype=torch.int32, device=DEV)
+        _lib.check(L.mpsa_route_tiles(_lib.ptr(qs), _lib.ptr(ks), B, Hq, Hkv, nq, n_keys, D, tile, causal, hi, lo,
+                                      _lib.ptr(work), _lib.ptr(cls), _lib.ptr(order), _lib.ptr(counts), _lib.stream_ptr()))
+        assert np.array_equal(cls.cpu().numpy(), d[name + "_cls"]), name
+        assert np.array_equal(order.cpu().numpy(), d[name + "_order"]), name
+        assert np.array_equal(counts.cpu().numpy(), d[name + "_counts"]), name
+
+
 def _compare(got, want, what=""):
     m = O.precision_metric(got.cpu(), want)
     assert m["cos"] >= COS_MIN and m["max_abs"] <= MAXABS_MAX, f"{what}: {m}"

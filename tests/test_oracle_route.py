@@ -189,3 +189,18 @@ def test_routed_attention_all_skipped_row_is_zero():
     route = np.array([[[[FP4, FP4], [SKIP, SKIP]]]], dtype=np.uint8)
     out = O.attn_mx(q, k, v, tile=32, causal=False, mode="routed", route=route)
     assert (out[0, 0, 32:] == 0).all() and out[0, 0, :32].abs().max() > 0
+
+
+def test_route_golden_vectors():
+    """The committed vectors (tests/golden/route_vectors.npz, written by make_route_vectors.py) pin the rule."""
+    import os
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "route_vectors.npz"))
+    for name in "abcde":
+        tile, D, n_keys, causal = (int(x) for x in d[name + "_meta"])
+        hi, lo = (float(x) for x in d[name + "_thresh"])
+        cls = O.route_tiles(d[name + "_qs"], d[name + "_ks"], tile, bool(causal), hi, lo)
+        order, counts = O.route_order(cls, n_keys, tile, bool(causal))
+        assert np.array_equal(cls, d[name + "_cls"]), name
+        assert np.array_equal(order, d[name + "_order"]), name
+        assert np.array_equal(counts, d[name + "_counts"]), name
+
