@@ -36,8 +36,8 @@ Parity status of each restated function:
   of the statistic, the decisions and the restricted softmax
   (tests/test_oracle_gemm_attn.py).
 * ``route_tiles`` / ``route_order`` -- this build's own integer rule (the reference has no precision router);
-  pinned against a float64 evaluation of the score bound it stands for and hand-worked maps
-  (tests/test_oracle_route.py); ``attn_mx(mode="routed")`` is pinned against the dense float64 attention on the
+  pinned against an exact rational evaluation of the score bound it stands for, hand-worked maps and committed
+  golden vectors (tests/test_oracle_route.py, tests/golden/route_vectors.npz); ``attn_mx(mode="routed")`` is pinned against the dense float64 attention on the
   same map and must reproduce the fixed modes on the maps that describe them.
 * ``seq_mean`` / ``smooth_k`` -- the once-rounded mean is pinned against
   float64 arithmetic and exactly representable cases; the float32 summation
