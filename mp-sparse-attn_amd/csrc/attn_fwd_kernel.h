@@ -107,7 +107,9 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         if constexpr (ROUTED) return t < nsteps ? min(max(ord[t], 0), a.nt - 1) : 0;
         if (t < n_plain) return t + (t >= skip ? 1 : 0);
         if (tail_special && t == n_plain) return a.nt - 1;
-        return i;
+        // the diagonal tile (runs that have one have as many key tiles as query tiles) -- and, past the last step,
+        // any valid key tile: with more query tiles than key tiles (cross attention) i itself is not one
+        return min(i, a.nt - 1);
     };
     // routed: the key tiles of steps t, t+1, t+2 are kept in scalar registers and the list entry of step t+3 is
     // fetched a whole step before its first use -- a scalar load that is waited for in the middle of a step would

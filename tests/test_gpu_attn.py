@@ -162,7 +162,8 @@ def test_tiny_and_barely_ragged_lengths(N, tile, causal):
 
 
 @pytest.mark.parametrize("mode", ["mxfp4", "mxfp8"])
-@pytest.mark.parametrize("Nq,Nk,D,tile", [(300, 77, 128, 128), (64, 1000, 64, 64), (1024, 512, 128, 128), (130, 129, 64, 128)])
+@pytest.mark.parametrize("Nq,Nk,D,tile", [(300, 77, 128, 128), (64, 1000, 64, 64), (1024, 512, 128, 128), (130, 129, 64, 128),
+                                          (640, 64, 64, 128)])
 def test_cross_attention_different_query_and_key_lengths(mode, Nq, Nk, D, tile):
     """Non-causal attention of Nq queries over Nk keys (the reference's kernel takes M and N apart,
     ours/mxfp_attn_kernel.py:362-371), grouped-query heads, ragged on both sides; with tile skipping as well."""
