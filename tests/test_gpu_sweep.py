@@ -1,0 +1,88 @@
+"""Seeded random sweeps of the attention and matmul entry points against the CPU oracle: shapes, head grouping,
+ragged lengths, cross attention, every precision mode incl. routed, both 16-bit input types.  The fixed-shape tests
+name their cases; this one walks combinations nobody thought of (an earlier sweep of this kind found a look-ahead
+that read K scales out of bounds when a cross-attention run had more query tiles than key tiles)."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from conftest import make_qkv
+from ours.block_scaled_matmul import block_scaled_matmul, initialize_block_scaled_from_tensor
+from ours.mxfp_attn_kernel import prepare_operands, route_tiles, attention_from_operands, mxfp_attn_kernel
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _attention_case(rnd):
+    D = rnd.choice([64, 128]); tile = rnd.choice([64, 128])
+    Hkv = rnd.choice([1, 2]); Hq = Hkv * rnd.choice([1, 2, 4])
+    N = max(128, rnd.randint(1, 6) * tile - rnd.choice([0, 0, 1, 17, tile // 2, tile - 1]))
+    mode = rnd.choice(["mxfp4", "mxfp8", "diag", "routed", "routed", "mxfp8e5", "routed_e5"])
+    causal = rnd.random() < 0.5
+    cross = (not causal) and mode != "diag" and rnd.random() < 0.3
+    Nk = max(64, rnd.randint(1, 6) * tile - rnd.choice([0, 3, tile // 2])) if cross else N
+    dt = rnd.choice([torch.bfloat16, torch.float16])
+    return dict(D=D, tile=tile, Hq=Hq, Hkv=Hkv, N=N, Nk=Nk, mode=mode, causal=causal, cross=cross, dt=dt,
+                seed=rnd.randint(0, 10 ** 6), hi=rnd.choice([None, 0.3, 0.6, 0.9]), lo=rnd.choice([None, 0.05, 0.3]))
+
+
+@pytest.mark.parametrize("sweep_seed", [11, 12])
+def test_attention_sweep(sweep_seed):
+    rnd = random.Random(sweep_seed)
+    for c in range(40):
+        p = _attention_case(rnd)
+        what = f"sweep {sweep_seed} case {c}: {p}"
+        print(what, flush=True)
+        q, k, v = make_qkv(1, p["Hq"], p["Hkv"], p["N"], p["D"], seed=p["seed"], dtype=p["dt"])
+        if p["cross"]:
+            _, k, v = make_qkv(1, p["Hq"], p["Hkv"], p["Nk"], p["D"], seed=p["seed"] + 1, dtype=p["dt"])
+        g = torch.Generator().manual_seed(p["seed"] + 7)
+        for t in (q, k):                                   # magnitudes that differ from tile to tile
+            n = t.shape[2]
+            gain = torch.exp2(torch.randint(-3, 3, (1, t.shape[1], -(-n // 64), 1), generator=g).float())
+            t *= gain.repeat_interleave(64, dim=2)[:, :, :n].to(t.dtype)
+        fmt8 = O.FMT_E5M2 if p["mode"].endswith("e5") else O.FMT_E4M3
+        if p["mode"].startswith("routed"):
+            ops = prepare_operands(q.to(DEV), k.to(DEV), v.to(DEV), p["tile"], p["mode"])
+            route = route_tiles(ops, p["causal"], p["hi"], p["lo"])
+            cls = route[0].cpu().numpy()
+            want_cls = O.route_tiles(ops["qs4"].cpu().numpy(), ops["ks4"].cpu().numpy(), p["tile"], p["causal"], p["hi"], p["lo"])
+            assert np.array_equal(cls, want_cls), what
+            out = torch.empty((1, p["Hq"], p["N"], p["D"]), dtype=p["dt"], device=DEV)
+            attention_from_operands(ops, out, p["causal"], route=route)
+            want = O.attn_mx(q, k, v, tile=p["tile"], causal=p["causal"], mode="routed", route=cls, fmt8=fmt8)
+        else:
+            out = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=p["causal"], block_scale_type=p["mode"],
+                                   tile=p["tile"], output_dtype=p["dt"])
+            want = O.attn_mx(q, k, v, tile=p["tile"], causal=p["causal"], mode={"mxfp8e5": "mxfp8"}.get(p["mode"], p["mode"]),
+                             fmt8=fmt8)
+        m = O.precision_metric(out.cpu(), want)
+        assert m["cos"] >= 0.999 and m["max_abs"] <= 2e-2, f"{what}: {m}"
+
+
+def test_matmul_sweep():
+    rnd = random.Random(21)
+    types = {"mxfp4": O.FMT_E2M1, "mxfp8": O.FMT_E4M3, "mxfp8e5": O.FMT_E5M2}
+    for c in range(16):
+        M = 256 * rnd.randint(1, 3); N = 256 * rnd.randint(1, 4); K = 128 * rnd.randint(1, 20)
+        bst = rnd.choice(list(types)); fmt = types[bst]
+        dt = rnd.choice([torch.float32, torch.bfloat16, torch.float16])
+        what = f"case {c}: M={M} N={N} K={K} {bst} out={dt}"
+        print(what, flush=True)
+        g = torch.Generator().manual_seed(rnd.randint(0, 10 ** 6))
+        scale_a = torch.exp2(torch.randint(-4, 4, (M, K // 32), generator=g).float()).repeat_interleave(32, 1)
+        a = (torch.randn(M, K, generator=g) * scale_a).bfloat16()
+        b = torch.randn(N, K, generator=g).bfloat16()
+        ac, asc, bc, bsc, cfg = initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst)
+        got = block_scaled_matmul(ac, asc, bc, bsc, dt, M, N, K, cfg).cpu()
+        da = O.dequantize_mx(ac.cpu(), asc.cpu(), fmt, torch.float64)
+        db = O.dequantize_mx(bc.cpu(), bsc.cpu(), fmt, torch.float64)
+        want, mag = da @ db.T, da.abs() @ db.abs().T
+        out_rounding = {torch.float32: 0.0, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -10}[dt]
+        err = (got.double() - want).abs()
+        bound = (1e-7 * mag + out_rounding * want.abs()) if fmt == O.FMT_E2M1 else ((1e-3 + out_rounding) * want.abs() + 3e-5 * mag)
+        assert not (err > bound).any(), what
