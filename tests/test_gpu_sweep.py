@@ -12,6 +12,7 @@ import oracle as O
 from conftest import make_qkv
 from ours.block_scaled_matmul import block_scaled_matmul, initialize_block_scaled_from_tensor
 from ours.mxfp_attn_kernel import prepare_operands, route_tiles, attention_from_operands, mxfp_attn_kernel
+from ours.quant_mxint8 import quantize_mx, quantize_mx_dual
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -86,3 +87,35 @@ def test_matmul_sweep():
         err = (got.double() - want).abs()
         bound = (1e-7 * mag + out_rounding * want.abs()) if fmt == O.FMT_E2M1 else ((1e-3 + out_rounding) * want.abs() + 3e-5 * mag)
         assert not (err > bound).any(), what
+
+
+def test_quantizer_sweep():
+    """Codes and scale bytes bit-exact: random shapes, magnitudes over 40 binades, pre-scales, padding, strided
+    ("NHD") inputs, single and dual output."""
+    rnd = random.Random(31)
+    for c in range(30):
+        B, H = rnd.choice([1, 2]), rnd.choice([1, 3])
+        N = rnd.choice([1, 31, 64, 100, 257, 640]); D = rnd.choice([64, 128, 256])
+        dt = rnd.choice([torch.bfloat16, torch.float16])
+        pre = rnd.choice([1.0, 0.5, O.q_pre_scale(D), 0.1275, 3.0])
+        out_rows = N + rnd.choice([0, 0, 5, 128 - N % 128])
+        what = f"case {c}: B={B} H={H} N={N} D={D} {dt} pre={pre} out_rows={out_rows}"
+        print(what, flush=True)
+        g = torch.Generator().manual_seed(rnd.randint(0, 10 ** 6))
+        spread = 20 if dt == torch.bfloat16 else 6
+        mag = torch.exp2(torch.randint(-spread, spread, (B, H, N, D // 32), generator=g).float()).repeat_interleave(32, 3)
+        x = (torch.randn(B, H, N, D, generator=g) * mag).to(dt)
+        xd = x.to(DEV)
+        if rnd.random() < 0.5:                             # the same values behind "NHD" strides
+            xd = xd.transpose(1, 2).contiguous().transpose(1, 2)
+        for fmt in (O.FMT_E2M1, O.FMT_E4M3, O.FMT_E5M2):
+            codes, scales = quantize_mx(xd, pre, fmt, out_rows=out_rows)
+            want_c, want_s = O.quantize_mx(x, pre, fmt)
+            assert torch.equal(scales[:, :, :N].cpu(), want_s) and torch.equal(codes[:, :, :N].cpu(), want_c), f"{what} fmt {fmt}"
+            assert not scales[:, :, N:].any() and not codes[:, :, N:].any(), f"{what}: padding rows must be zero"
+        c4, s4, c8, s8 = quantize_mx_dual(xd, pre, out_rows=out_rows)
+        w4, ws4 = O.quantize_mx(x, pre, O.FMT_E2M1)
+        w8, ws8 = O.quantize_mx(x, pre, O.FMT_E4M3)
+        assert torch.equal(c4[:, :, :N].cpu(), w4) and torch.equal(s4[:, :, :N].cpu(), ws4), f"{what} dual 4-bit"
+        assert torch.equal(c8[:, :, :N].cpu(), w8) and torch.equal(s8[:, :, :N].cpu(), ws8), f"{what} dual 8-bit"
+
