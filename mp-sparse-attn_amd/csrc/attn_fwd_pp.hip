@@ -5,16 +5,21 @@
 // tile structure and the grouped-query head mapping).  What differs is the work split.  A workgroup of EIGHT waves
 // owns TWO adjacent query tiles: waves 0-3 ("X", tile 2I+1) and waves 4-7 ("Y", tile 2I); wave w and wave w+4 sit
 // on the same SIMD.  Both groups read the same K and V tiles from LDS, which halves the L2 -> LDS traffic per query
-// and the number of direct-to-LDS loads per CU.  Between two consecutive workgroup barriers X runs
-// P.V(t) -> S(t+1) -> softmax(t+1) while Y runs softmax(t) -> P.V(t) -> S(t+1), i.e. the two waves of a SIMD are in
-// opposite phases.  (Measured on MI355X this phase offset buys little: while one wave streams back-to-back matrix
-// instructions the other wave of the SIMD gets almost no vector issue slots, so matrix and vector phases of the two
-// waves still add up; the shared staging is what makes this kernel faster than the one-tile kernel.)
+// and the number of direct-to-LDS loads per CU.
+//
+// Step t of a wave (between workgroup barriers t and t+1) is software-pipelined inside the wave: first the score
+// instructions S(t+1), then the 32 matrix instructions of P.V(t) with the softmax of tile t+1 placed in the gaps
+// between them -- measured on MI355X, vector instructions of the *other* wave of a SIMD get almost no issue slots
+// while a wave streams matrix instructions, but a few vector instructions between a wave's own matrix instructions
+// are free.  The registers of a 16-key group of P(t) take the new P(t+1) as soon as the four instructions that
+// consume the group have been issued.  When the (lazy) running maximum has to move, the scores are rebased at once
+// and the output accumulators at the top of the next step, when P.V(t) -- relative to the old maximum -- is through.
+// The wave's diagonal tile runs as straight-line code after the loop; Y, one tile short of X, idles in the last step.
 //
 // Staging is the one of attn_fwd.hip: 4-bit K tiles (XOR-swizzled rows) and V tiles (operand order) arrive by
-// direct-to-LDS loads, double-buffered, one barrier per key tile; the K fragments of the next tile are pulled into
-// registers before the P.V instructions are issued; the single 8-bit (diagonal) tile of a "diag" run is read straight
-// from global memory.  The running maximum is lazy and rides in the score MFMA's C operand.
+// direct-to-LDS loads, one barrier per key tile; K has three buffers (the tile whose fragments are being pulled into
+// registers is two steps ahead of the P.V tile), V two; the single 8-bit (diagonal) tile of a "diag" run is read
+// straight from global memory.  The running maximum rides in the score MFMA's C operand.
 #include "attn_common.h"
 
 namespace {
@@ -24,7 +29,8 @@ constexpr int KB = TILE / 32, SST = D / 64, NDB = D / 32;
 constexpr int ROW4 = D / 2, ROW8 = D;
 constexpr int CPR4 = ROW4 / 16, SH4 = 2;
 constexpr int K_BYTES = TILE * ROW4, V_BYTES = TILE * D * 2;
-constexpr int SMEM = 2 * K_BYTES + 2 * V_BYTES;
+constexpr int NKBUF = 3;                        // K tiles in LDS: one being multiplied, two ahead
+constexpr int SMEM = NKBUF * K_BYTES + 2 * V_BYTES;
 constexpr int NWAVES = 8;
 constexpr int VI = V_BYTES / 1024 / NWAVES;     // direct-load instructions per wave for one V tile (4)
 constexpr int NV = KB * 2 * NDB;                // P.V matrix instructions per tile (32)
@@ -38,7 +44,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, w = tid >> 6;
     const int h = lane >> 5, r = lane & 31;
-    const int role = w >> 2;                     // 0 = X (matrix phase first), 1 = Y (vector phase first)
+    const int role = w >> 2;                     // 0 = X (tile 2I+1), 1 = Y (tile 2I)
     const int wq = w & 3;
 
     // ---- which (batch, kv head, query head, query-tile pair) -- XCD-aware, heavy pairs first ----
@@ -64,7 +70,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     const int64_t q_row = qhead_row + (int64_t)i * TILE + q_local;
 
     uint8_t* const kbuf0 = smem;
-    uint8_t* const vbuf0 = smem + 2 * K_BYTES;
+    uint8_t* const vbuf0 = smem + NKBUF * K_BYTES;
 
     // ---- operands in registers ----
     v8i qf[SST];
@@ -97,7 +103,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             ksc[kb] = (int)(*reinterpret_cast<const uint32_t*>(sp + kb * 32 * (D / 32)) >> (8 * h));
     };
     auto read_kf4 = [&](int t) __attribute__((always_inline)) {
-        const uint8_t* kl = kbuf0 + (t & 1) * K_BYTES;
+        const uint8_t* kl = kbuf0 + (t % NKBUF) * K_BYTES;
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
             const int krow = 32 * kb + r;
@@ -119,7 +125,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     }
     auto issue_k4 = [&](int t) __attribute__((always_inline)) {
         const uint8_t* src = a.k4 + (khead_row + (int64_t)t * TILE) * ROW4;
-        load16_to_lds_sv(koff, src, kbuf0 + (t & 1) * K_BYTES + wu * 1024);
+        load16_to_lds_sv(koff, src, kbuf0 + (t % NKBUF) * K_BYTES + wu * 1024);
     };
     auto issue_v = [&](int t) __attribute__((always_inline)) {
         const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)t * TILE) * (D * 2);
@@ -138,7 +144,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         if (t + 1 < nsteps) issue_v(t + 1);
-        if (t + 2 < nsteps) issue_k4(t + 2);
+        if (t + 3 < nsteps) issue_k4(t + 3);
     };
 
     // ---- per-query state ----
@@ -258,65 +264,127 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         }
     };
 
-    // ---- prologue (all waves): V(0), K(0), K(1) on their way; step-0 operands into registers ----
+    // P.V(t) with the softmax of tile t+1 (whose scores are in st) in the gaps between its matrix instructions: after the
+    // four instructions that consume one 16-key group of P(t), that group's registers take the new P(t+1)
+    float alpha_due = 1.0f;
+    bool rescale_due = false;
+    auto rescale = [&]() __attribute__((always_inline)) {
+        if (rescale_due) {
+#pragma unroll
+            for (int d = 0; d < NDB; ++d)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[d][e] *= alpha_due;
+            rescale_due = false;
+        }
+    };
+    auto pv_exp = [&](int t) __attribute__((always_inline)) {
+        constexpr int PRE = 8;
+        const uint8_t* vl = vbuf0 + (t & 1) * V_BYTES + lane * 16;
+        typename P::vec vf[PRE];
+#pragma unroll
+        for (int x = 0; x < PRE; ++x) vf[x] = *reinterpret_cast<const typename P::vec*>(vl + x * 1024);
+        auto mm = [&](int idx) __attribute__((always_inline)) {
+            const int d = idx % NDB, kc = idx / NDB;
+            const typename P::vec cur = vf[idx % PRE];
+            if (idx + PRE < NV) vf[idx % PRE] = *reinterpret_cast<const typename P::vec*>(vl + (idx + PRE) * 1024);
+            acc[d] = P::mfma(cur, __builtin_bit_cast(typename P::vec, pk[kc >> 1][kc & 1]), acc[d]);
+        };
+#pragma unroll
+        for (int idx = 0; idx < NDB; ++idx) mm(idx);
+        float mx = st[0][0];
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, st[kb][e]);
+        mx = max_lane_pair(mx);
+        float ps0 = 0.0f, ps1 = 0.0f;
+        auto ex = [&](int g, int j) __attribute__((always_inline)) {
+            const int kb = g >> 1, c = g & 1;
+            const float p0 = __builtin_amdgcn_exp2f(st[kb][8 * c + 2 * j]);
+            const float p1 = __builtin_amdgcn_exp2f(st[kb][8 * c + 2 * j + 1]);
+            const typename P::v2 pp = P::pack(p0, p1);
+            pk[kb][c][j] = __builtin_bit_cast(int, pp);
+            if (j & 1) ps1 = P::add2(pp, ps1); else ps0 = P::add2(pp, ps0);
+        };
+        const uint8_t* kl = kbuf0 + ((t + 2) % NKBUF) * K_BYTES;
+        auto kfrag = [&](int kb, int s) __attribute__((always_inline)) {
+            const int krow = 32 * kb + r;
+            const int f = (krow >> SH4) & (CPR4 - 1);
+            kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * ROW4 + (((2 * s + h) ^ f) * 16));
+        };
+        if (__any(mx > REBASE)) {
+            // rare: the running maximum moves.  P(t), whose P.V is under way, is relative to the old one: the output
+            // accumulators are rescaled once that is through (at the top of the next step)
+            const float delta = __builtin_fmaxf(mx, 0.0f);
+            alpha_due = __builtin_amdgcn_exp2f(-delta);
+            rescale_due = true;
+            m_run += delta;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) negm[e] = -m_run;
+            l_run *= alpha_due;
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) st[kb][e] -= delta;
+        }
+#pragma unroll
+        for (int kc = 1; kc < 2 * KB; ++kc)
+#pragma unroll
+            for (int d = 0; d < NDB; ++d) {
+                mm(kc * NDB + d);
+                ex(kc - 1, d);
+                if (kc >= KB && d < SST) kfrag(kc - KB, d);   // K fragments of tile t+2 (the score MFMAs are long gone)
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+            }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ex(2 * KB - 1, j);
+        l_run += ps0 + ps1;
+    };
+
+    // ---- prologue (all waves): V(0), K(0..2) on their way; Q into registers ----
     issue_v(0);
     issue_k4(0);
     issue_k4(1);
-    load_kscales(0, false);
+    if (nsteps > 2) issue_k4(2);
     load_q(false);
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    read_kf4(0);
 
-    if (role == 0) {
-        // ===== X: tile i = 2*pair+1 >= 1; between barriers: P.V(t) -> S(t+1) -> softmax(t+1) =====
+    // Step t (between barriers t and t+1): S(t+1), then P.V(t) with the softmax of t+1 in its gaps.  The wave's last
+    // key tile (the diagonal one, index i) gets straight-line code; Y, one tile short of X, idles through the last step.
+    const int last = i;
+    if (last == 0) {
+        prep_special(0);
+        s_special(0);
+        softmax(true, std::true_type{});
+    } else {
+        prep_plain(0);
         s_plain();
         softmax(true, std::false_type{});
-        for (int t = 0; t < nsteps - 2; ++t) {
-            sync_issue(t);
-            prep_plain(t + 1);
-            pv(t);
-            s_plain();
-            softmax(false, std::false_type{});
-        }
-        {
-            const int t = nsteps - 2;
-            sync_issue(t);
-            prep_special(t + 1);
-            pv(t);
-            s_special(t + 1);
-            softmax(false, std::true_type{});
-        }
-        sync_issue(nsteps - 1);
-        pv(nsteps - 1);
-    } else {
-        // ===== Y: tile i = 2*pair; between barriers: softmax(t) -> P.V(t) -> S(t+1); idle in the last step =====
-        if (i == 0) {
-            prep_special(0);
-            s_special(0);
-        } else {
-            s_plain();
-        }
-        for (int t = 0; t < i - 1; ++t) {
-            sync_issue(t);
-            softmax(t == 0, std::false_type{});
-            prep_plain(t + 1);
-            pv(t);
-            s_plain();
-        }
-        if (i >= 1) {
-            const int t = i - 1;
-            sync_issue(t);
-            softmax(t == 0, std::false_type{});
-            prep_special(t + 1);
-            pv(t);
-            s_special(t + 1);
-        }
-        sync_issue(i);
-        softmax(i == 0, std::true_type{});
-        pv(i);
-        sync_issue(i + 1);
+        if (last >= 2) prep_plain(1);
     }
+    for (int t = 0; t + 2 <= last; ++t) {
+        rescale();
+        sync_issue(t);
+        s_plain();
+        load_kscales(t + 2, false);
+        pv_exp(t);
+    }
+    rescale();
+    if (last >= 1) {
+        const int t = last - 1;
+        sync_issue(t);
+        prep_special(t + 1);
+        pv(t);
+        s_special(t + 1);
+        softmax(false, std::true_type{});
+    }
+    sync_issue(last);
+    pv(last);
+    if (role == 1) sync_issue(last + 1);
     __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
 
     // ---- epilogue: O = acc / l ; register e of lane (h, r): dim 32*db + 8*(e/4) + 4*h + e%4 of query r ----
