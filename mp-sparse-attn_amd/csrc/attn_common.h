@@ -28,6 +28,9 @@ template <> struct PV<MPSA_BF16> {
     static __device__ __forceinline__ float add2(v2 p, float c) { return __builtin_amdgcn_fdot2_f32_bf16(p, (v2){(__bf16)1.0f, (__bf16)1.0f}, c, false); }
     // P = exp2(S - m_run) may grow to 2^REBASE before the running maximum is moved: bf16 has float32's range
     static constexpr float REBASE = 60.0f;
+    // a lane's row sum of one tile at which a kernel that takes the exponentials first and looks afterwards does
+    // the tile again with the maximum pass (2^REBASE)
+    static constexpr float OPTIMISTIC_LIMIT = 1152921504606846976.0f;
 };
 template <> struct PV<MPSA_F16> {
     typedef v8h vec;
@@ -36,6 +39,7 @@ template <> struct PV<MPSA_F16> {
     static __device__ __forceinline__ v2 pack(float x, float y) { return (v2){(_Float16)x, (_Float16)y}; }
     static __device__ __forceinline__ float add2(v2 p, float c) { return __builtin_amdgcn_fdot2(p, (v2){(_Float16)1.0f, (_Float16)1.0f}, c, false); }
     static constexpr float REBASE = 12.0f;      // fp16 P must stay below 65504
+    static constexpr float OPTIMISTIC_LIMIT = 4096.0f;
 };
 
 // Exchange between the two lanes (l, l^32) that share one query.  v_permlane32_swap swaps lanes 32-63 of its first

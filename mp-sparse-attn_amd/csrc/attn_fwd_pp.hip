@@ -265,18 +265,11 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     };
 
     // P.V(t) with the softmax of tile t+1 (whose scores are in st) in the gaps between its matrix instructions: after the
-    // four instructions that consume one 16-key group of P(t), that group's registers take the new P(t+1)
-    float alpha_due = 1.0f;
-    bool rescale_due = false;
-    auto rescale = [&]() __attribute__((always_inline)) {
-        if (rescale_due) {
-#pragma unroll
-            for (int d = 0; d < NDB; ++d)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[d][e] *= alpha_due;
-            rescale_due = false;
-        }
-    };
+    // four instructions that consume one 16-key group of P(t), that group's registers take the new P(t+1).
+    // The exponentials are taken optimistically, without looking for the tile's maximum first: the running maximum
+    // only has to move when a score exceeds it by more than REBASE, and then the row sum shows it (it exceeds
+    // 2^REBASE or is not finite).  In that rare case the tile is done again the careful way, from its K fragments,
+    // which are still in LDS.
     auto pv_exp = [&](int t) __attribute__((always_inline)) {
         constexpr int PRE = 8;
         const uint8_t* vl = vbuf0 + (t & 1) * V_BYTES + lane * 16;
@@ -289,14 +282,6 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             if (idx + PRE < NV) vf[idx % PRE] = *reinterpret_cast<const typename P::vec*>(vl + (idx + PRE) * 1024);
             acc[d] = P::mfma(cur, __builtin_bit_cast(typename P::vec, pk[kc >> 1][kc & 1]), acc[d]);
         };
-#pragma unroll
-        for (int idx = 0; idx < NDB; ++idx) mm(idx);
-        float mx = st[0][0];
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, st[kb][e]);
-        mx = max_lane_pair(mx);
         float ps0 = 0.0f, ps1 = 0.0f;
         auto ex = [&](int g, int j) __attribute__((always_inline)) {
             const int kb = g >> 1, c = g & 1;
@@ -312,36 +297,56 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             const int f = (krow >> SH4) & (CPR4 - 1);
             kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * ROW4 + (((2 * s + h) ^ f) * 16));
         };
-        if (__any(mx > REBASE)) {
-            // rare: the running maximum moves.  P(t), whose P.V is under way, is relative to the old one: the output
-            // accumulators are rescaled once that is through (at the top of the next step)
-            const float delta = __builtin_fmaxf(mx, 0.0f);
-            alpha_due = __builtin_amdgcn_exp2f(-delta);
-            rescale_due = true;
-            m_run += delta;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) negm[e] = -m_run;
-            l_run *= alpha_due;
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) st[kb][e] -= delta;
-        }
-#pragma unroll
-        for (int kc = 1; kc < 2 * KB; ++kc)
+        for (int kc = 0; kc < 2 * KB; ++kc)
 #pragma unroll
             for (int d = 0; d < NDB; ++d) {
                 mm(kc * NDB + d);
-                ex(kc - 1, d);
+                if (kc > 0) ex(kc - 1, d);
                 if (kc >= KB && d < SST) kfrag(kc - KB, d);   // K fragments of tile t+2 (the score MFMAs are long gone)
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
-                __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+                if (kc > 0) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+                }
             }
 #pragma unroll
         for (int j = 0; j < 4; ++j) ex(2 * KB - 1, j);
-        l_run += ps0 + ps1;
+        float tot = ps0 + ps1;
+        if (__any(!(tot < P::OPTIMISTIC_LIMIT))) {
+            // the careful way: scores again, maximum, rebase (P.V(t) is through, the accumulators can be rescaled now)
+            prep_plain(t + 1);
+            s_plain();
+            float mx = st[0][0];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, st[kb][e]);
+            mx = max_lane_pair(mx);
+            const float delta = __builtin_fmaxf(mx, 0.0f);
+            const float alpha = __builtin_amdgcn_exp2f(-delta);
+            m_run += delta;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) negm[e] = -m_run;
+            l_run *= alpha;
+#pragma unroll
+            for (int d = 0; d < NDB; ++d)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[d][e] *= alpha;
+            ps0 = 0.0f;
+            ps1 = 0.0f;
+#pragma unroll
+            for (int g = 0; g < 2 * KB; ++g) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) st[g >> 1][8 * (g & 1) + e] -= delta;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) ex(g, j);
+            }
+            tot = ps0 + ps1;
+            prep_plain(t + 2);                             // back to the operands of the next step
+        }
+        l_run += tot;
     };
 
     // ---- prologue (all waves): V(0), K(0..2) on their way; Q into registers ----
@@ -367,13 +372,11 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         if (last >= 2) prep_plain(1);
     }
     for (int t = 0; t + 2 <= last; ++t) {
-        rescale();
         sync_issue(t);
         s_plain();
         load_kscales(t + 2, false);
         pv_exp(t);
     }
-    rescale();
     if (last >= 1) {
         const int t = last - 1;
         sync_issue(t);

@@ -57,6 +57,41 @@ def test_all_kernel_variants_gqa(D, tile, causal, N):
     _compare(got, want, f"D={D} tile={tile} causal={causal}")
 
 
+def _rising_qkv(N, D, step, seed, spike_tile=None, tile=128):
+    """Inputs whose scores climb along the key axis: q = u + noise, k[n] = g(n) u + noise with |u|^2 = D, so that a
+    score in log2 units is about 1.44 sqrt(D) g(n).  ``step`` is g's increase per key tile; with ``spike_tile`` g is
+    zero except on that tile (one tile far above all the others)."""
+    gen = torch.Generator().manual_seed(seed)
+    u = torch.sign(torch.randn(D, generator=gen))
+    n = torch.arange(N, dtype=torch.float32)
+    g = (n / tile) * step if spike_tile is None else ((n // tile) == spike_tile).float() * step
+    q = (u + 0.3 * torch.randn(1, 4, N, D, generator=gen)).to(torch.bfloat16)
+    k = (g[:, None] * u + 0.3 * torch.randn(1, 2, N, D, generator=gen)).to(torch.bfloat16)
+    v = torch.randn(1, 2, N, D, generator=gen).to(torch.bfloat16)
+    return q, k, v
+
+
+@pytest.mark.parametrize("pv", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal,N,tile", [(True, 1024, 128), (True, 1536, 128), (False, 1024, 128), (True, 640, 128), (True, 512, 64)])
+@pytest.mark.parametrize("shape", ["ramp", "spike"])
+def test_running_maximum_moves(shape, causal, N, tile, pv):
+    """Scores that rise by far more than the lazy maximum's threshold from one key tile to the next (bf16: 60, fp16: 12,
+    in log2 units), and a single tile towering over the rest: the running maximum has to move, in the paired-tile
+    kernel (causal, whole tile pairs), which takes the exponentials first and repeats a tile whose row sum shows that
+    the maximum must move, and in the general kernel."""
+    D = 128
+    if shape == "ramp":
+        q, k, v = _rising_qkv(N, D, step=5.0, seed=N + tile, tile=tile)          # ~80 log2 units per tile
+    else:
+        q, k, v = _rising_qkv(N, D, step=9.0, seed=N + tile + 1, spike_tile=2, tile=tile)
+    q, k, v = q.to(pv), k.to(pv), v.to(pv)
+    for mode in ("diag", "mxfp4"):
+        got = _run(q, k, v, is_causal=causal, block_scale_type=mode, tile=tile, output_dtype=torch.float32)
+        want = O.attn_mx(q, k, v, tile=tile, causal=causal, mode=mode, out_dtype=torch.float32)
+        assert torch.isfinite(got).all()
+        _compare(got, want, f"{shape} {mode} causal={causal} N={N} tile={tile} {pv}")
+
+
 def test_c3_llama_shape_one_kv_group_with_outliers():
     """B=1 Hq=32 Hkv=8 N=8192 D=128 causal, outlier channels, 128x128 tiles: the full problem runs on the GPU,
     the oracle checks query heads 4..7 (KV head 1) and head 31."""
