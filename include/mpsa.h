@@ -158,6 +158,20 @@ int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, const uint8_t* b, 
                          void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream);
 
 /*
+ * Both products with the scales in the reference's packed form [rows/128, K/128, 32, 4, 4] - what its wrappers build
+ * before calling the Triton kernel (ours/mxfp_attn_kernel.py:56-57, consumed at ours/block_scaled_matmul.py:207-216)
+ * and what mpsa_scales_to_5d produces: byte (r%32)*16 + (r/32 % 4)*4 + k of chunk (r/128, kb/4) is the scale of row r,
+ * K block kb = 4*(kb/4) + k.  The kernel fetches a 128-row x 128-element chunk as 512 contiguous bytes (a quarter of
+ * the cache lines the row-major layout costs) and reads a lane's scale words for four row blocks with one 128-bit
+ * LDS read.  Same results as the row-major entry points, bit for bit.  sa5, sb5: 16-byte aligned.
+ */
+int mpsa_gemm_mx_packed(const uint8_t* a, const uint8_t* sa5, const uint8_t* b, const uint8_t* sb5, int fmt,
+                        int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream);
+int mpsa_gemm_mx_batched_packed(const uint8_t* a, const uint8_t* sa5, const uint8_t* b, const uint8_t* sb5, int fmt,
+                                int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
+                                void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream);
+
+/*
  * Value-tile repack: v [B,H,N,D] (bf16 | f16, strided, last dim contiguous) -> v_tiles
  * [B,H,ceil(N/tile),tile*D] of the same dtype in matrix-core operand order, keys past N zero.
  * Replaces the dtype normalisation / .contiguous() of V in the reference wrapper

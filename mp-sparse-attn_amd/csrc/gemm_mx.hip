@@ -48,6 +48,7 @@ struct GemmArgs {
     void* c;
     int64_t ldc;
     int M, N, K;
+    int packed;                // scales in the packed [rows/128, K/128, 32, 4, 4] form instead of [rows, K/32]
     int heads_a, heads_b;      // batched runs: blockIdx.y = batch * heads_a + head; B's head is head / (heads_a / heads_b)
 };
 
@@ -92,8 +93,9 @@ __device__ __forceinline__ void load_to_lds(uint32_t lane_off, const uint8_t* wa
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(base), "v"(lane_off), "s"(gb) : "memory", "m0");
 }
 
-template <int FMT, typename OutT, bool WIDE>
+template <int FMT, typename OutT, bool WIDE, bool PK>
 __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
+    static_assert(!(WIDE && PK), "packed scales use the per-stage scale area");
     constexpr bool FP4 = (FMT == MPSA_FMT_E2M1);
     constexpr int STAGE_BYTES = stage_bytes<WIDE>();
     constexpr int GROUP = FP4 ? 4 : 8;                 // stages covered by 16 scale bytes of a row
@@ -153,6 +155,13 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     const uint8_t* const b_base = g.b + (int64_t)n0 * row_bytes;
     const uint8_t* const sa_base = g.sa + (int64_t)m0 * srow_bytes;
     const uint8_t* const sb_base = g.sb + (int64_t)n0 * srow_bytes;
+    // packed scales (the reference's [rows/128, K/128, 32, 4, 4] form, ours/mxfp_attn_kernel.py:56-57): the scale bytes
+    // of 128 rows x 128 elements of K are one 512-byte chunk, byte (row%32)*16 + (row/32)*4 + k.  A stage needs two
+    // chunks per operand: waves 0, 1 bring A's, waves 2, 3 B's, each with its first 32 lanes.
+    const int kchunks = g.K / 128;
+    const uint32_t pko = (uint32_t)((lane & 31) * 16);
+    const uint8_t* const s_pk = (wave < 2 ? g.sa + (int64_t)(m0 / 128) * kchunks * 512 : g.sb + (int64_t)(n0 / 128) * kchunks * 512) +
+                                (int64_t)(wave & 1) * kchunks * 512;
     // a stage's loads go out in four parts (two code instructions each, the narrow path's scale words with the
     // last) so that they can be spread between the matrix instructions of a step
     auto issue_part = [&](int kt, int part) __attribute__((always_inline)) {
@@ -160,7 +169,15 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         uint8_t* st = smem + (kt % NSTAGE) * STAGE_BYTES;
         load_to_lds<16>(lo[part], a_base + (int64_t)kc * ROWB, st + (wave * 4 + part) * 1024);
         load_to_lds<16>(lo[part], b_base + (int64_t)kc * ROWB, st + OP_BYTES + (wave * 4 + part) * 1024);
-        if constexpr (!WIDE) {
+        if constexpr (PK) {
+            // with 8-bit codes a chunk covers two stages and the odd stage's step takes its scale words from the
+            // even step's registers, so only even stages fetch (any two consecutive stages still issue the same
+            // number of loads, which is what the partial waits count)
+            if (part == 3 && (FP4 || (kt & 1) == 0)) {
+                const int64_t kb = FP4 ? kc : (kc >> 1);
+                if (lane < 32) load_to_lds<16>(pko, s_pk + kb * 512, st + 2 * OP_BYTES + wave * 512);
+            }
+        } else if constexpr (!WIDE) {
             if (part == 3) {
                 // four scale bytes per row: the stage's own with 4-bit codes; with 8-bit codes the aligned word
                 // that holds this stage's two bytes (the stage count is even, so the word is inside the row)
@@ -241,7 +258,16 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
                     if (isb) f.sb[i] = even.sb[i]; else f.sa[i] = even.sa[i];
                 }
             } else if (fresh) {
-                (isb ? f.rb[i] : f.ra[i]) = *reinterpret_cast<const uint32_t*>(sc + row * sstride);
+                if constexpr (PK) {
+                    // one conflict-free 128-bit read: the scale words of this lane's row in all four row blocks
+                    if (i == 0) {
+                        const v4i wsc = *reinterpret_cast<const v4i*>(sc + (isb ? wn : wm) * 512 + r * 16);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) (isb ? f.rb[q] : f.ra[q]) = (uint32_t)wsc[q];
+                    }
+                } else {
+                    (isb ? f.rb[i] : f.ra[i]) = *reinterpret_cast<const uint32_t*>(sc + row * sstride);
+                }
             } else {
                 if (isb) f.sb[i] = even.sb[i]; else f.sa[i] = even.sa[i];
             }
@@ -315,7 +341,7 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     // wide path although the two stages after a scale fetch amount to 18: waiting for two loads more than
     // needed is harmless and keeps the count a constant.)
     auto publish = [&]() __attribute__((always_inline)) {
-        constexpr int KEEP = 2 * (WIDE ? CODE_LOADS : CODE_LOADS + 2);
+        constexpr int KEEP = WIDE ? 2 * CODE_LOADS : PK ? (FP4 ? 2 * (CODE_LOADS + 1) : 2 * CODE_LOADS + 1) : 2 * (CODE_LOADS + 2);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(wait_imm(KEEP));
         __syncthreads();
@@ -324,7 +350,8 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
 
     Frag f0, f1;
     {
-        constexpr int KEEP = (NSTAGE - 1) * (WIDE ? CODE_LOADS : CODE_LOADS + 2);
+        // stages 1 .. NSTAGE-1 stay in flight (packed 8-bit: only stage 2 of them carries scale loads)
+        constexpr int KEEP = WIDE ? (NSTAGE - 1) * CODE_LOADS : PK ? (FP4 ? (NSTAGE - 1) * (CODE_LOADS + 1) : (NSTAGE - 1) * CODE_LOADS + 1) : (NSTAGE - 1) * (CODE_LOADS + 2);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(wait_imm(KEEP));
         __syncthreads();
@@ -382,10 +409,10 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         }
 }
 
-template <int FMT, typename OutT, bool WIDE>
+template <int FMT, typename OutT, bool WIDE, bool PK>
 void launch_kernel(const GemmArgs& g, dim3 grid, hipStream_t st) {
     static bool reserved[MPSA_MAX_DEVICES] = {};
-    auto kern = gemm_mx_kernel<FMT, OutT, WIDE>;
+    auto kern = gemm_mx_kernel<FMT, OutT, WIDE, PK>;
     // a failure here shows up as a launch error, which the caller reports
     (void)mpsa_reserve_lds(reinterpret_cast<const void*>(kern), smem_bytes<WIDE>(), reserved);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem_bytes<WIDE>(), st, g);
@@ -393,8 +420,9 @@ void launch_kernel(const GemmArgs& g, dim3 grid, hipStream_t st) {
 
 template <int FMT, typename OutT>
 void launch_one(const GemmArgs& g, dim3 grid, hipStream_t st) {
-    if (g.K % 512 == 0) launch_kernel<FMT, OutT, true>(g, grid, st);
-    else                launch_kernel<FMT, OutT, false>(g, grid, st);
+    if (g.packed)            launch_kernel<FMT, OutT, false, true>(g, grid, st);
+    else if (g.K % 512 == 0) launch_kernel<FMT, OutT, true, false>(g, grid, st);
+    else                     launch_kernel<FMT, OutT, false, false>(g, grid, st);
 }
 
 template <int FMT>
@@ -407,9 +435,9 @@ void launch_fmt(const GemmArgs& g, int c_dtype, dim3 grid, hipStream_t st) {
 
 }  // namespace
 
-extern "C" int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
-                                    int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
-                                    void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
+static int gemm_entry(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt, bool packed,
+                      int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
+                      void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
     if (!a || !sa || !b || !sb || !c) return mpsa_fail(MPSA_EINVAL, "gemm: null pointer");
     if (fmt != MPSA_FMT_E2M1 && fmt != MPSA_FMT_E4M3 && fmt != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "gemm: unknown format %d", fmt);
     if (c_dtype != MPSA_BF16 && c_dtype != MPSA_F16 && c_dtype != MPSA_F32 && c_dtype != MPSA_F8E5M2) return mpsa_fail(MPSA_EINVAL, "gemm: unsupported output dtype %d", c_dtype);
@@ -420,10 +448,12 @@ extern "C" int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, const u
         return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: shape too large");
     if (!mpsa_aligned16(a) || !mpsa_aligned16(b) || (reinterpret_cast<uintptr_t>(sa) & 3) || (reinterpret_cast<uintptr_t>(sb) & 3))
         return mpsa_fail(MPSA_EALIGN, "gemm: codes must be 16-byte and scales 4-byte aligned");
+    if (packed && (!mpsa_aligned16(sa) || !mpsa_aligned16(sb))) return mpsa_fail(MPSA_EALIGN, "gemm: packed scales must be 16-byte aligned");
     GemmArgs g;
     g.a = a; g.sa = sa; g.b = b; g.sb = sb; g.c = c; g.ldc = ldc;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.heads_a = (int)heads_a; g.heads_b = (int)heads_b;
+    g.packed = packed ? 1 : 0;
     dim3 grid((unsigned)((M / BM) * (N / BN)), (unsigned)(batch * heads_a));
     hipStream_t st = (hipStream_t)stream;
     if (fmt == MPSA_FMT_E2M1)      launch_fmt<MPSA_FMT_E2M1>(g, c_dtype, grid, st);
@@ -433,7 +463,24 @@ extern "C" int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, const u
     return MPSA_OK;
 }
 
+extern "C" int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
+                                    int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
+                                    void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
+    return gemm_entry(a, sa, b, sb, fmt, false, batch, heads_a, heads_b, M, N, K, c, c_dtype, ldc, stream);
+}
+
 extern "C" int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
                             int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
-    return mpsa_gemm_mx_batched(a, sa, b, sb, fmt, 1, 1, 1, M, N, K, c, c_dtype, ldc, stream);
+    return gemm_entry(a, sa, b, sb, fmt, false, 1, 1, 1, M, N, K, c, c_dtype, ldc, stream);
+}
+
+extern "C" int mpsa_gemm_mx_packed(const uint8_t* a, const uint8_t* sa5, const uint8_t* b, const uint8_t* sb5, int fmt,
+                                   int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
+    return gemm_entry(a, sa5, b, sb5, fmt, true, 1, 1, 1, M, N, K, c, c_dtype, ldc, stream);
+}
+
+extern "C" int mpsa_gemm_mx_batched_packed(const uint8_t* a, const uint8_t* sa5, const uint8_t* b, const uint8_t* sb5, int fmt,
+                                           int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
+                                           void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
+    return gemm_entry(a, sa5, b, sb5, fmt, true, batch, heads_a, heads_b, M, N, K, c, c_dtype, ldc, stream);
 }

@@ -38,6 +38,8 @@ SIGNATURES = {
                                      _vp, _vp, _vp, _vp, _i64, _vp]),
     "mpsa_gemm_mx": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
     "mpsa_gemm_mx_batched": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
+    "mpsa_gemm_mx_packed": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
+    "mpsa_gemm_mx_batched_packed": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
     "mpsa_v_tiles": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _int, _vp, _vp]),
     "mpsa_attn_prepare": (_int, [_vp, _p64, _vp, _p64, _vp, _p64, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int,
                                  _f32, _vp] + [_vp] * 9 + [_vp]),

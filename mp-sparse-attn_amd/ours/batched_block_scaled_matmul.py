@@ -21,10 +21,12 @@ def block_scaled_batched_matmul(a, a_scale, b, b_scale, dtype_dst, B, H, M, N, K
         raise ValueError(f"Unsupported dtype: {dtype_dst}")
     fmt = _fmt_of(configs)
     _lib.require_device(a, a_scale, b, b_scale)
-    if a_scale.dim() == 7:
-        a_scale = unpack_scale_5d(a_scale)
-    if b_scale.dim() == 7:
-        b_scale = unpack_scale_5d(b_scale)
+    packed = a_scale.dim() == 7 and b_scale.dim() == 7      # both packed: the kernel takes them as they are
+    if not packed:
+        if a_scale.dim() == 7:
+            a_scale = unpack_scale_5d(a_scale)
+        if b_scale.dim() == 7:
+            b_scale = unpack_scale_5d(b_scale)
     width = K // 2 if fmt == _lib.FMT_E2M1 else K
     a = a.view(torch.uint8).contiguous()
     b = b.view(torch.uint8).contiguous()
@@ -33,10 +35,14 @@ def block_scaled_batched_matmul(a, a_scale, b, b_scale, dtype_dst, B, H, M, N, K
     Hb = b.shape[1]
     assert a.shape == (B, H, M, width) and b.shape == (B, Hb, N, width), "operand shapes do not match B, H, M, N, K"
     assert H % Hb == 0, "heads of A must be a multiple of heads of B"
-    assert a_scale.shape == (B, H, M, K // VEC_SIZE) and b_scale.shape == (B, Hb, N, K // VEC_SIZE), "scales must be [B, H, rows, K/32]"
+    if packed:
+        assert a_scale.shape == (B, H, M // 128, K // 128, 32, 4, 4) and b_scale.shape == (B, Hb, N // 128, K // 128, 32, 4, 4), \
+            "packed scales must be [B, H, rows/128, K/128, 32, 4, 4]"
+    else:
+        assert a_scale.shape == (B, H, M, K // VEC_SIZE) and b_scale.shape == (B, Hb, N, K // VEC_SIZE), "scales must be [B, H, rows, K/32]"
     out = torch.empty((B, H, M, N), dtype=dtype_dst, device=a.device)
+    entry = _lib.lib().mpsa_gemm_mx_batched_packed if packed else _lib.lib().mpsa_gemm_mx_batched
     with torch.cuda.device(a.device):
-        _lib.check(_lib.lib().mpsa_gemm_mx_batched(_lib.ptr(a), _lib.ptr(a_scale), _lib.ptr(b), _lib.ptr(b_scale), fmt,
-                                                   B, H, Hb, M, N, K, _lib.ptr(out), _lib.dtype_id(dtype_dst), N,
-                                                   _lib.stream_ptr(a.device)))
+        _lib.check(entry(_lib.ptr(a), _lib.ptr(a_scale), _lib.ptr(b), _lib.ptr(b_scale), fmt,
+                         B, H, Hb, M, N, K, _lib.ptr(out), _lib.dtype_id(dtype_dst), N, _lib.stream_ptr(a.device)))
     return out

@@ -3,7 +3,8 @@
 ``block_scaled_matmul(a, a_scale, b, b_scale, dtype_dst, M, N, K, configs)`` keeps the reference
 signature (ours/block_scaled_matmul.py:271).  Operands are what the quantizer emits: row-major codes
 (``[M, K/2]`` packed E2M1 or ``[M, K]`` 8-bit) and linear E8M0 scales ``[M, K/32]`` (the reference's 5-D packed
-scales ``[M/128, K/128, 32, 4, 4]`` are accepted too and re-laid out first); B is ``[N, K]``
+scales ``[M/128, K/128, 32, 4, 4]`` are accepted too: given for both operands they go to the kernel as they are,
+which is its faster path); B is ``[N, K]``
 (NT product).  The element format is read from ``configs["ELEM_PER_BYTE_A"]`` (2 = E2M1) and, for
 8-bit, ``configs.get("FMT8", "e4m3")``.
 """
@@ -71,33 +72,43 @@ def block_scaled_matmul(a, a_scale, b, b_scale, dtype_dst, M, N, K, configs):
         raise ValueError(f"Unsupported dtype: {dtype_dst}")
     fmt = _fmt_of(configs)
     _lib.require_device(a, a_scale, b, b_scale)
-    if a_scale.dim() == 5:                       # the reference's packed scale layout
-        a_scale = unpack_scale_5d(a_scale)
-    if b_scale.dim() == 5:
-        b_scale = unpack_scale_5d(b_scale)
+    # the reference's packed scale layout goes to the kernel as it is when both operands come that way
+    packed = a_scale.dim() == 5 and b_scale.dim() == 5
+    if not packed:
+        if a_scale.dim() == 5:
+            a_scale = unpack_scale_5d(a_scale)
+        if b_scale.dim() == 5:
+            b_scale = unpack_scale_5d(b_scale)
     width = K // 2 if fmt == _lib.FMT_E2M1 else K
     a = a.view(torch.uint8).contiguous()
     b = b.view(torch.uint8).contiguous()
     a_scale = a_scale.contiguous()
     b_scale = b_scale.contiguous()
     assert a.shape == (M, width) and b.shape == (N, width), "operand shapes do not match M, N, K"
-    assert a_scale.shape == (M, K // VEC_SIZE) and b_scale.shape == (N, K // VEC_SIZE), "scales must be [rows, K/32]"
+    if packed:
+        assert a_scale.shape == (M // 128, K // 128, 32, 4, 4) and b_scale.shape == (N // 128, K // 128, 32, 4, 4), \
+            "packed scales must be [rows/128, K/128, 32, 4, 4]"
+    else:
+        assert a_scale.shape == (M, K // VEC_SIZE) and b_scale.shape == (N, K // VEC_SIZE), "scales must be [rows, K/32]"
     out = torch.empty((M, N), dtype=dtype_dst, device=a.device)
+    entry = _lib.lib().mpsa_gemm_mx_packed if packed else _lib.lib().mpsa_gemm_mx
     with torch.cuda.device(a.device):
-        _lib.check(_lib.lib().mpsa_gemm_mx(_lib.ptr(a), _lib.ptr(a_scale), _lib.ptr(b), _lib.ptr(b_scale), fmt,
-                                           M, N, K, _lib.ptr(out), _lib.dtype_id(dtype_dst), N,
-                                           _lib.stream_ptr(a.device)))
+        _lib.check(entry(_lib.ptr(a), _lib.ptr(a_scale), _lib.ptr(b), _lib.ptr(b_scale), fmt,
+                         M, N, K, _lib.ptr(out), _lib.dtype_id(dtype_dst), N, _lib.stream_ptr(a.device)))
     return out
 
 
-def initialize_block_scaled_from_tensor(a_tensor, b_tensor, block_scale_type="mxfp4"):
+def initialize_block_scaled_from_tensor(a_tensor, b_tensor, block_scale_type="mxfp4", packed_scales=False):
     """Quantize bf16/fp16 ``A [M,K]`` and ``B [N,K]`` per 32 along K and package them for
     :func:`block_scaled_matmul`: returns ``(a, a_scale, b, b_scale, configs)``.
 
     Counterpart of the reference's operand packaging (ours/block_scaled_matmul.py:299-406) chained after
-    the quantizer as in test_quant.py:296-350; scales stay in the linear ``[rows, K/32]`` layout."""
+    the quantizer as in test_quant.py:296-350; scales stay in the linear ``[rows, K/32]`` layout unless
+    ``packed_scales`` asks for the reference's packed one."""
     configs = make_configs(block_scale_type)
     fmt = _fmt_of(configs)
     a, sa = quantize_mx(a_tensor[None, None], 1.0, fmt)
     b, sb = quantize_mx(b_tensor[None, None], 1.0, fmt)
+    if packed_scales:                            # the reference packs them at this point (ours/block_scaled_matmul.py:299-406)
+        return a[0, 0], pack_scale_5d(sa[0, 0]), b[0, 0], pack_scale_5d(sb[0, 0]), configs
     return a[0, 0], sa[0, 0], b[0, 0], sb[0, 0], configs

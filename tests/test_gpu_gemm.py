@@ -148,6 +148,29 @@ def test_scale_5d_layout_and_matmul_with_packed_scales():
         pack_scale_5d(lin[:, :, :100].contiguous().to(DEV))
 
 
+@pytest.mark.parametrize("bst", ["mxfp4", "mxfp8", "mxfp8e5"])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 768, 384), (256, 512, 640), (768, 256, 1024), (512, 512, 2048)])
+def test_packed_scale_kernel_path_equals_the_row_major_one(bst, M, N, K):
+    """Both operands' scales in the reference's packed form go to the kernel as they are (512-byte chunks fetched
+    whole, one 128-bit LDS read per lane and stage): every output bit equals the row-major path's, for every format,
+    several tiles per dimension, K that is and is not a multiple of 512 (the row-major path then takes its own two
+    variants), odd and even stage counts, and each output dtype."""
+    from ours.block_scaled_matmul import pack_scale_5d
+    g = torch.Generator().manual_seed(M + N + K)
+    a = (torch.randn(M, K, generator=g) * torch.exp2(torch.randint(-6, 6, (M, 1), generator=g).float())).bfloat16()
+    b = (torch.randn(N, K, generator=g) * torch.exp2(torch.randint(-6, 6, (1, K), generator=g).float())).bfloat16()
+    ac, asc, bc, bsc, cfg = initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst)
+    assert asc.unique().numel() > 4                               # scales that differ: a mixed-up byte would show
+    a5, b5 = pack_scale_5d(asc), pack_scale_5d(bsc)
+    for dt in (torch.float32, torch.bfloat16, torch.float16, torch.float8_e5m2):
+        c_lin = block_scaled_matmul(ac, asc, bc, bsc, dt, M, N, K, cfg)
+        c_pk = block_scaled_matmul(ac, a5, bc, b5, dt, M, N, K, cfg)
+        assert torch.equal(c_lin.view(torch.uint8) if dt == torch.float8_e5m2 else c_lin,
+                           c_pk.view(torch.uint8) if dt == torch.float8_e5m2 else c_pk), f"{bst} {M}x{N}x{K} {dt}"
+    ac2, a52, bc2, b52, _ = initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst, packed_scales=True)
+    assert torch.equal(a52, a5) and torch.equal(b52, b5) and torch.equal(ac2, ac)
+
+
 def test_e5m2_output_dtype():
     """The reference's third output dtype (ours/block_scaled_matmul.py:185-190): every byte equals torch's own
     float32 -> float8_e5m2 cast of the kernel's float32 result, overflow to infinity included."""
