@@ -12,8 +12,10 @@
 // between them -- measured on MI355X, vector instructions of the *other* wave of a SIMD get almost no issue slots
 // while a wave streams matrix instructions, but a few vector instructions between a wave's own matrix instructions
 // are free.  The registers of a 16-key group of P(t) take the new P(t+1) as soon as the four instructions that
-// consume the group have been issued.  When the (lazy) running maximum has to move, the scores are rebased at once
-// and the output accumulators at the top of the next step, when P.V(t) -- relative to the old maximum -- is through.
+// consume the group have been issued.  The exponentials are taken without a maximum pass: the (lazy) running maximum
+// only has to move when a score exceeds it by more than a threshold, which the tile's row sum then shows; the wave
+// does such a tile again the careful way (scores from the K tile still in LDS, maximum, rebase of row sum and output
+// accumulators -- P.V(t), relative to the old maximum, is through by then -- and exponentials).
 // The wave's diagonal tile runs as straight-line code after the loop; Y, one tile short of X, idles in the last step.
 //
 // Staging is the one of attn_fwd.hip: 4-bit K tiles (XOR-swizzled rows) and V tiles (operand order) arrive by
