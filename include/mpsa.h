@@ -136,7 +136,7 @@ int mpsa_seq_mean(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, i
  * and its Triton kernel (ours/block_scaled_matmul.py:271-296, :154-267).
  *
  *   a, b     packed codes [M,K/2] / [N,K/2] (E2M1) or [M,K] / [N,K] (8-bit), row-major, contiguous
- *   sa, sb   E8M0 bytes [M,K/32] / [N,K/32], row-major (the linear layout, not the 5-D packed one)
+ *   sa, sb   E8M0 bytes [M,K/32] / [N,K/32], row-major (the linear layout; mpsa_gemm_mx_packed below takes the 5-D packed one)
  *   fmt      element format of both operands
  *   c        [M,N] of c_dtype (MPSA_BF16 | MPSA_F16 | MPSA_F32 | MPSA_F8E5M2: one E5M2 byte per element, round to
  *            nearest even, overflow to infinity - the reference's output dtypes are f32, f16 and e5m2,

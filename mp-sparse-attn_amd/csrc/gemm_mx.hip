@@ -25,6 +25,9 @@
 // the codes themselves.  When K is a multiple of 512 the kernel instead fetches 16 scale bytes per row at a
 // time (a "group" of 4 stages of 4-bit codes, 8 stages of 8-bit codes) into a double-buffered LDS area, one
 // group ahead.  Other K fall back to one 4-byte scale load per row per stage.
+// With the scales in the reference's packed form [rows/128, K/128, 32, 4, 4] (ours/mxfp_attn_kernel.py:56-57) the
+// scale bytes of 128 rows x 128 elements of K are one contiguous 512-byte chunk: a stage's scales are four chunks,
+// one 32-lane load per wave, and a lane reads its scale words for all four row blocks with one 128-bit LDS read.
 #include "mpsa_common.h"
 
 namespace {
