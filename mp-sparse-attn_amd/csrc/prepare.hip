@@ -15,12 +15,11 @@ struct PrepArgs {
     VTArgs v;
     uint32_t bq, bk, bv;          // workgroups per (batch, head) of each job
     uint32_t hq, hkv;
-    uint32_t q_total, k_total;    // workgroups of the Q job, of the K job
+    uint32_t q_total, k_total, v_total;    // blocks of the Q job, of the K job, of the V job
 };
 
 template <int XDT, bool DO4, bool DO8, int FMT8, int TILE, int D>
-__global__ __launch_bounds__(256) void prepare_kernel(PrepArgs p) {
-    uint32_t blk = blockIdx.x;
+__device__ __forceinline__ void prepare_block(const PrepArgs& p, uint32_t blk) {
     if (blk < p.q_total) {
         const uint32_t head = blk / p.bq;
         quantize_block<XDT, DO4, DO8, FMT8, false>(p.q, blk - head * p.bq, head % p.hq, head / p.hq, p.hq);
@@ -33,8 +32,16 @@ __global__ __launch_bounds__(256) void prepare_kernel(PrepArgs p) {
         return;
     }
     blk -= p.k_total;
+    if (blk >= p.v_total) return;
     const uint32_t head = blk / p.bv;
     v_tiles_block<TILE, D>(p.v, blk - head * p.bv, head % p.hkv, head / p.hkv, p.hkv);
+}
+
+// two blocks of work per workgroup (measured on the stand-alone quantizer: 8-13 % more bandwidth than one)
+template <int XDT, bool DO4, bool DO8, int FMT8, int TILE, int D>
+__global__ __launch_bounds__(256) void prepare_kernel(PrepArgs p) {
+    prepare_block<XDT, DO4, DO8, FMT8, TILE, D>(p, 2 * blockIdx.x);
+    prepare_block<XDT, DO4, DO8, FMT8, TILE, D>(p, 2 * blockIdx.x + 1);
 }
 
 template <int XDT, bool DO4, bool DO8, int FMT8>
@@ -94,9 +101,10 @@ extern "C" int mpsa_attn_prepare(const void* q, const int64_t q_strides[4], cons
     if (total >= (int64_t(1) << 31)) return mpsa_fail(MPSA_EUNSUPPORTED, "prepare: problem too large for one launch");
     p.bq = bq; p.bk = bk; p.bv = bv; p.hq = (uint32_t)Hq; p.hkv = (uint32_t)Hkv;
     p.q_total = (uint32_t)((int64_t)bq * Hq * B); p.k_total = (uint32_t)((int64_t)bk * Hkv * B);
+    p.v_total = (uint32_t)((int64_t)bv * Hkv * B);
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == MPSA_BF16) launch_mode<MPSA_BF16>(p, mode, fmt8, tile, (int)D, (unsigned)total, st);
-    else                    launch_mode<MPSA_F16>(p, mode, fmt8, tile, (int)D, (unsigned)total, st);
+    if (dtype == MPSA_BF16) launch_mode<MPSA_BF16>(p, mode, fmt8, tile, (int)D, (unsigned)((total + 1) / 2), st);
+    else                    launch_mode<MPSA_F16>(p, mode, fmt8, tile, (int)D, (unsigned)((total + 1) / 2), st);
     MPSA_CHECK_LAUNCH("prepare");
     return MPSA_OK;
 }

@@ -110,7 +110,7 @@ int quantize_common(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N,
     unsigned blocks = 0;
     const int rc = mpsa_quantize_setup(x, x_dtype, B, H, N, D, xs, sub, pre, do4, emax4, do8, fmt8, emax8, c4, s4, c8, s8, out_rows, &a, &blocks);
     if (rc != MPSA_OK || blocks == 0) return rc;
-    dim3 grid(blocks, (unsigned)H, (unsigned)B);
+    dim3 grid((blocks + 1) / 2, (unsigned)H, (unsigned)B);     // the kernel takes two blocks of chunks per workgroup
     if (x_dtype == MPSA_BF16) {
         if (do4 && do8) launch<MPSA_BF16, true, true>(a, fmt8, grid, st);
         else if (do4)   launch<MPSA_BF16, true, false>(a, fmt8, grid, st);

@@ -193,7 +193,9 @@ __device__ __forceinline__ void quantize_block(const QuantArgs& a, uint32_t bx, 
 
 template <int XDT, bool DO4, bool DO8, int FMT8, bool SW8>
 __global__ __launch_bounds__(256) void quantize_kernel(QuantArgs a) {
-    quantize_block<XDT, DO4, DO8, FMT8, SW8>(a, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y);
+    // two 256-chunk blocks per workgroup: both loads are in flight before either block is converted
+    quantize_block<XDT, DO4, DO8, FMT8, SW8>(a, 2 * blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y);
+    quantize_block<XDT, DO4, DO8, FMT8, SW8>(a, 2 * blockIdx.x + 1, blockIdx.y, blockIdx.z, gridDim.y);
 }
 
 }  // namespace
