@@ -132,6 +132,21 @@ int mpsa_seq_mean(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, i
                   const int64_t x_strides[4], float* workspace, void* mean, mpsa_stream_t stream);
 
 /*
+ * mpsa_seq_mean without a workspace argument, for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid allocation).  It has no counterpart in the reference.  The
+ * float32 partial sums go to a device array built into the library (MPSA_SEQ_MEAN_STATIC_BYTES per GPU, held until
+ * the process ends); the call allocates and frees nothing.  Same kernels, same bits as mpsa_seq_mean.
+ *   - mpsa_seq_mean_workspace(B,H,N,D) must not exceed MPSA_SEQ_MEAN_STATIC_BYTES (e.g. B*H = 8 heads of D = 128 up to
+ *     N = 262144), else MPSA_EUNSUPPORTED;
+ *   - all calls on one GPU share the array: calls that overlap on one GPU (different streams or host threads) race;
+ *     calls ordered on one stream are safe.  Nothing needs clearing between calls (every partial sum read was
+ *     written by the same call).
+ */
+#define MPSA_SEQ_MEAN_STATIC_BYTES 4194304
+int mpsa_seq_mean_static(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                         const int64_t x_strides[4], void* mean, mpsa_stream_t stream);
+
+/*
  * Block-scaled matmul  C[M,N] = (A o 2^(sa-127)) (B o 2^(sb-127))^T.  Replaces block_scaled_matmul
  * and its Triton kernel (ours/block_scaled_matmul.py:271-296, :154-267).
  *

@@ -17,6 +17,7 @@
 // 2 B/element in, 0.5 (+1) B/element of codes and 1/32 (x2) B/element of scales out.
 #include "quantize_kernel.h"
 #include <cstring>
+#include <mutex>
 
 namespace {
 
@@ -186,8 +187,10 @@ extern "C" int64_t mpsa_seq_mean_workspace(int64_t B, int64_t H, int64_t N, int6
     return B * H * ((N + MEAN_ROWS - 1) / MEAN_ROWS) * D * (int64_t)sizeof(float);
 }
 
-extern "C" int mpsa_seq_mean(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
-                             const int64_t x_strides[4], float* workspace, void* mean, mpsa_stream_t stream) {
+namespace {
+
+int seq_mean_common(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                    const int64_t x_strides[4], float* workspace, void* mean, hipStream_t st) {
     if (!x || !x_strides || !workspace || !mean) return mpsa_fail(MPSA_EINVAL, "seq_mean: null pointer");
     if (x_dtype != MPSA_BF16 && x_dtype != MPSA_F16) return mpsa_fail(MPSA_EINVAL, "seq_mean: x_dtype must be bf16 or f16");
     if (B <= 0 || H <= 0 || N <= 0) return mpsa_fail(MPSA_EINVAL, "seq_mean: bad shape");
@@ -199,7 +202,6 @@ extern "C" int mpsa_seq_mean(const void* x, int x_dtype, int64_t B, int64_t H, i
     a.x = x; a.sb = x_strides[0]; a.sh = x_strides[1]; a.sn = x_strides[2];
     a.n = (int)N; a.d = (int)D; a.nchunk = (int)((N + MEAN_ROWS - 1) / MEAN_ROWS);
     a.partial = workspace; a.mean = mean; a.inv_n = 1.0f / (float)N;
-    hipStream_t st = (hipStream_t)stream;
     dim3 grid((unsigned)a.nchunk, (unsigned)H, (unsigned)B);
     if (x_dtype == MPSA_BF16) {
         hipLaunchKernelGGL(seq_mean_kernel<MPSA_BF16>, grid, dim3(256), 0, st, a);
@@ -210,4 +212,52 @@ extern "C" int mpsa_seq_mean(const void* x, int x_dtype, int64_t B, int64_t H, i
     }
     MPSA_CHECK_LAUNCH("seq_mean");
     return MPSA_OK;
+}
+
+}  // namespace
+
+extern "C" int mpsa_seq_mean(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                             const int64_t x_strides[4], float* workspace, void* mean, mpsa_stream_t stream) {
+    return seq_mean_common(x, x_dtype, B, H, N, D, x_strides, workspace, mean, (hipStream_t)stream);
+}
+
+// ---- the same mean for callers that cannot allocate: the partial sums live in a device array of this library ----
+// Every GPU the library runs on holds its own copy of the array (at its own address) until the process ends.  The
+// name `scratch` is a host-side handle, not a device address: host code asks the runtime for the address once per
+// device and passes that pointer on.
+static __device__ __align__(256) float scratch[MPSA_SEQ_MEAN_STATIC_BYTES / sizeof(float)];
+
+namespace {
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[MPSA_MAX_DEVICES] = {};
+
+// device address of `scratch` on the current device (resolved on the first call per device)
+int scratch_for_current_device(float** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "seq_mean_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= MPSA_MAX_DEVICES) return mpsa_fail(MPSA_EUNSUPPORTED, "seq_mean_static: device index %d beyond %d", dev, MPSA_MAX_DEVICES - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        float* p = nullptr;
+        e = hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return mpsa_fail(MPSA_ELAUNCH, "seq_mean_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return MPSA_OK;
+}
+}  // namespace
+
+extern "C" int mpsa_seq_mean_static(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
+                                    const int64_t x_strides[4], void* mean, mpsa_stream_t stream) {
+    const int64_t need = mpsa_seq_mean_workspace(B, H, N, D);
+    if (need > (int64_t)MPSA_SEQ_MEAN_STATIC_BYTES)
+        return mpsa_fail(MPSA_EUNSUPPORTED, "seq_mean_static: B*H*ceil(N/256)*D*4 = %lld bytes of partial sums exceed the built-in %lld; use mpsa_seq_mean with a workspace",
+                         (long long)need, (long long)MPSA_SEQ_MEAN_STATIC_BYTES);
+    float* ws = nullptr;
+    const int rc = scratch_for_current_device(&ws);
+    if (rc != MPSA_OK) return rc;
+    // nothing to clear: the first kernel writes every partial sum the second one reads
+    return seq_mean_common(x, x_dtype, B, H, N, D, x_strides, ws, mean, (hipStream_t)stream);
 }

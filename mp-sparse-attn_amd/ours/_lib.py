@@ -34,6 +34,7 @@ SIGNATURES = {
     "mpsa_quantize_mx": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _vp, _f32, _int, _int, _vp, _vp, _i64, _vp]),
     "mpsa_seq_mean_workspace": (_i64, [_i64, _i64, _i64, _i64]),
     "mpsa_seq_mean": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _vp, _vp, _vp]),
+    "mpsa_seq_mean_static": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _vp, _vp]),
     "mpsa_quantize_mx_dual": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _vp, _f32, _int, _int, _int,
                                      _vp, _vp, _vp, _vp, _i64, _vp]),
     "mpsa_gemm_mx": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
