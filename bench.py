@@ -8,8 +8,8 @@ MX-quantize Q and K (E2M1 + E4M3 in one pass each), repack V, fused attention (d
 off-diagonal MXFP4, causal, GQA).  Prints ONE JSON line: whole-step attention TFLOP/s
 (FlashAttention convention 2*B*Hq*N^2*D for causal), the roofline of the dominant kernel (the fused
 attention kernel, timed alone with HIP events on its launch stream), secondary figures for the
-quantizer and the standalone block-scaled GEMM, and the CPU oracle timed on the host cores on a bounded
-sample of the same workload.
+quantizer and the standalone block-scaled GEMM and for the long-context configuration (N = 131072), and the CPU
+oracle timed on the host cores on a bounded sample of the same workload.
 """
 import argparse
 import json
@@ -30,10 +30,27 @@ PEAK_FP8_TFLOPS = 5000.0
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 
-# HBM-side bytes per launch of the fused attention kernel (L2 <-> fabric), from rocprofv3 --pmc FETCH_SIZE and
+# HBM-side bytes per launch of the fused attention kernel (L2 <-> fabric) come from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of `bench.py --only attn`, each scaled by the same counter's reading for a 1 GiB copy
-# (`bench.py --only copy`): FETCH_SIZE x 2.0 KiB, WRITE_SIZE x 1.0 KiB.  Summary: profiles/attn_c3_hbm_traffic.txt
-MEASURED_ATTN_TRAFFIC_BYTES = {"c3": 110.2e6 + 67.1e6}
+# (`bench.py --only copy`).  The summary file carries them in lines of the form
+#   #@ traffic workload=c3 mode=diag read_bytes=... write_bytes=... commit=...
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "attn_c3_hbm_traffic.txt")
+
+
+def measured_traffic(workload, mode):
+    """(bytes per launch, commit it was measured at) from the profile summary, or (None, None)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                if not line.startswith("#@ traffic"):
+                    continue
+                kv = dict(item.split("=", 1) for item in line.split()[2:])
+                if kv.get("workload") == workload and kv.get("mode") == mode:
+                    return float(kv["read_bytes"]) + float(kv["write_bytes"]), kv.get("commit")
+    except (OSError, ValueError, KeyError):
+        pass
+    return None, None
+
 
 WORKLOADS = {
     # name: (B, Hq, Hkv, N, D, tile, seed, description)
@@ -89,10 +106,33 @@ def time_events(fn, iters):
     return start.elapsed_time(stop) / iters
 
 
+def wait_for_device():
+    """Spin on an event until the stream has drained, then synchronize: the host does not sleep, so its wake-up
+    latency (about a tenth of a millisecond) stays out of short timed regions."""
+    ev = torch.cuda.Event()
+    ev.record()
+    while not ev.query():
+        pass
+    torch.cuda.synchronize()
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(q, k, v, tile, D, causal=True):
     """The CPU oracle (a port of the reference's fake-quant path) on the first 8192 positions of the workload
-    (all of it for C1/C3), every head."""
+    (all of it for C1/C3), every head, on the host threads this process may use."""
     import oracle as O
+    threads = max(1, min(int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)), os.cpu_count() or 1))
+    torch.set_num_threads(threads)
     Hq, Hkv = q.shape[1], k.shape[1]
     group = Hq
     n = min(q.shape[2], 8192)
@@ -105,9 +145,51 @@ def cpu_baseline(q, k, v, tile, D, causal=True):
     flops = (2.0 if causal else 4.0) * qs.shape[0] * group * n * n * D
     return {
         "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "cpu_model": cpu_model(),
         "sample": f"oracle.attn_mx (quantize+dequantize+tiled attention, torch CPU) on {group} query heads / {Hkv} KV heads, "
                   f"N={n}, D={D}, {'causal' if causal else 'non-causal'}, diag mode: {dt:.2f} s",
         "seconds": dt,
+    }
+
+
+def secondary_c4(device):
+    """The long-context configuration (N = 131072) next to the headline line: fused attention kernel, whole step, and
+    the operand preparation on 2.9 GB of traffic -- far beyond the 256 MB last-level cache, i.e. the quantizer's
+    out-of-cache bandwidth."""
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands
+    B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS["c4"]
+    q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device)
+    out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
+    ops = prepare_operands(q, k, v, tile, "diag")
+    attention_from_operands(ops, out, True)
+    torch.cuda.synchronize()
+    iters = 10
+    attn_ms = time_events(lambda: attention_from_operands(ops, out, True), iters)
+    prep_ms = time_events(lambda: prepare_operands(q, k, v, tile, "diag", reuse=ops), iters)
+
+    def step():
+        attention_from_operands(prepare_operands(q, k, v, tile, "diag", reuse=ops), out, True)
+
+    step()
+    wait_for_device()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        step()
+    wait_for_device()
+    step_ms = (time.perf_counter() - t0) * 1e3 / iters
+    flops = 2.0 * B * Hq * N * N * D
+    comp = composite_peak_tflops(N // tile, True)
+    # the preparation reads q, k, v (2 B/elem) and writes both code sets + scales of q and k and the V tiles
+    prep_bytes = (q.numel() + k.numel()) * (2 + 0.5 + 1 + 2 / 32) + v.numel() * 4
+    ktf, stf = flops / attn_ms / 1e9, flops / step_ms / 1e9
+    return {
+        "workload": desc, "steps": iters,
+        "kernel_ms": round(attn_ms, 3), "kernel_TFLOP/s": round(ktf, 1), "kernel_frac_mxfp4_peak": round(ktf / PEAK_FP4_TFLOPS, 5),
+        "kernel_frac_composite": round(ktf / comp, 5),
+        "ms_per_step": round(step_ms, 3), "TFLOP/s": round(stf, 1), "frac_mxfp4_peak": round(stf / PEAK_FP4_TFLOPS, 5),
+        "frac_composite": round(stf / comp, 5),
+        "prepare_ms": round(prep_ms, 4), "prepare_GB/s": round(prep_bytes / prep_ms / 1e6, 1),
+        "prepare_frac_hbm": round(prep_bytes / prep_ms / 1e6 / PEAK_HBM_GBS, 4), "prepare_bytes": prep_bytes,
     }
 
 
@@ -202,6 +284,8 @@ def main():
     ap.add_argument("--skip-thresh", type=float, default=None, help="routed: skipped below this share")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--no-c4", action="store_true", help="leave the long-context figures out of `secondary`")
+    ap.add_argument("--eager", action="store_true", help="time plain launches instead of replaying the step as a HIP graph")
     ap.add_argument("--linear-scales", action="store_true",
                     help="with --only gemm4/gemm8: row-major [rows, K/32] scales instead of the reference's packed form")
     ap.add_argument("--only", default=None, choices=["attn", "copy", "quant", "gemm4", "gemm8"],
@@ -237,18 +321,42 @@ def main():
 
     routed = args.mode == "routed"
 
+    # The secondary figures run first: they are not part of the timed region, and a few hundred milliseconds of
+    # matrix work before it bring the GPU's clocks up, which `--warmup` steps of a fraction of a millisecond do not.
+    second = None
+    if not args.no_secondary:
+        second = secondary(device, quick=args.steps < 10)
+
+    state = {"ops": prepare_operands(q, k, v, tile, args.mode)}
+
     def step():
-        ops = prepare_operands(q, k, v, tile, args.mode)
+        ops = prepare_operands(q, k, v, tile, args.mode, reuse=state["ops"])
         route = route_tiles(ops, causal, args.route_thresh, args.skip_thresh) if routed else None
         attention_from_operands(ops, out, causal, route=route)
 
+    # One step = two kernel launches on a stream.  A serving loop replays them as a HIP graph (the library neither
+    # allocates nor synchronises, so the whole step captures); --eager times plain launches instead.
+    launch = "eager"
+    run_step = step
+    if not args.eager and not routed:
+        try:
+            step()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            run_step, launch = graph.replay, "hip graph replay"
+        except Exception as e:                                    # capture is an optimisation, not a requirement
+            print(f"bench: graph capture failed ({e}); timing eager launches", file=sys.stderr)
+            run_step, launch = step, "eager"
+
     for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
+        run_step()
+    wait_for_device()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
+        run_step()
+    wait_for_device()
     dt = time.perf_counter() - t0
     ms_per_step = dt * 1e3 / args.steps
     flops = (2.0 if causal else 4.0) * B * Hq * N * N * D
@@ -261,15 +369,16 @@ def main():
     torch.cuda.synchronize()
     k_iters = max(5, args.steps)
     attn_ms = time_events(lambda: attention_from_operands(ops, out, causal, route=route), k_iters)
-    prep_ms = time_events(lambda: prepare_operands(q, k, v, tile, args.mode), k_iters)
+    prep_ms = time_events(lambda: prepare_operands(q, k, v, tile, args.mode, reuse=ops), k_iters)
     achieved = flops / (attn_ms * 1e-3) / 1e12
     nt = (N + tile - 1) // tile
     comp = composite_peak_tflops(nt, causal)
+    traffic, traffic_commit = measured_traffic(args.workload, args.mode)
     paired = causal and D == 128 and tile == 128 and N % 256 == 0 and args.mode in ("diag", "mxfp4")
     roofline = {
         "bound": "mfma", "kernel": ("attn_pp_kernel" if paired else "attn_fwd_kernel") + " (fused attention)", "achieved": round(achieved, 2), "peak": PEAK_FP4_TFLOPS,
         "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP4_TFLOPS, 5),
-        "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get(args.workload) if args.mode == "diag" else None,
+        "traffic": traffic, "traffic_measured_at": traffic_commit,
         "kernel_ms": round(attn_ms, 4), "prepare_ms": round(prep_ms, 4),
         "composite_peak": round(comp, 1), "frac_composite": round(achieved / comp, 5),
         "flops_per_launch": flops,
@@ -288,12 +397,17 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "mxfp4/mxfp8 scores (E2M1/E4M3 + E8M0), bf16 P.V, f32 accumulate", "data": "synthetic",
         "config": {"workload": desc, "B": B, "Hq": Hq, "Hkv": Hkv, "N": N, "D": D, "tile": tile, "mode": args.mode,
-                   "step": "quantize Q,K (dual) + V repack + " + ("tile router + " if routed else "") + "fused attention"},
+                   "step": "quantize Q,K (dual) + V repack + " + ("tile router + " if routed else "") + "fused attention",
+                   "launch": launch},
         "frac_mxfp4_peak": round(tflops / PEAK_FP4_TFLOPS, 5),
         "roofline": roofline,
     }
-    if not args.no_secondary:
-        result["secondary"] = secondary(device, quick=args.steps < 10)
+    if second is not None:
+        result["secondary"] = second
+        if args.workload == "c3" and args.mode == "diag" and not args.no_c4:
+            del ops, route
+            state.clear()
+            result["secondary"]["c4"] = secondary_c4(device)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(q, k, v, tile, D, causal)
     else:

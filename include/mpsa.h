@@ -39,6 +39,8 @@ typedef void* mpsa_stream_t;
 #define MPSA_MODE_MXFP8 1   /* every tile 8-bit */
 #define MPSA_MODE_DIAG  2   /* tile j == i 8-bit, all others 4-bit */
 #define MPSA_MODE_ROUTED 3  /* per-tile precision from a visiting list (mpsa_route_tiles, mpsa_attn_fwd_routed) */
+#define MPSA_MODE_MIXED  4  /* every tile: 8-bit Q x 4-bit K - the reference's "mixed" type (ELEM_PER_BYTE_A = 1,
+                               ELEM_PER_BYTE_B = 2, ours/mxfp_attn_kernel.py:264-269, :448-449) */
 
 #define MPSA_OK             0
 #define MPSA_EINVAL        -1   /* null pointer, bad enum, bad shape */
@@ -48,6 +50,15 @@ typedef void* mpsa_stream_t;
 
 int mpsa_version(void);
 const char* mpsa_last_error(void);
+
+/*
+ * One-time set-up of the CURRENT device: raises the dynamic-LDS limit of every kernel variant that needs it and
+ * resolves the address of the library's built-in device array (mpsa_seq_mean_static).  The launchers do this by
+ * themselves on a device's first use; a caller that captures its very first call into a HIP graph calls mpsa_init()
+ * beforehand, once per device, because function attributes cannot be set during capture.  Idempotent, thread-safe.
+ * (The reference has no counterpart: Triton sets such limits when it loads a kernel.)
+ */
+int mpsa_init(void);
 
 /*
  * Elementwise format conversions behind the MXFP4Tensor / MXScaleTensor helper classes; contiguous
@@ -63,6 +74,15 @@ int mpsa_e2m1_encode(const float* x, int64_t n, uint8_t* codes, mpsa_stream_t st
 int mpsa_e2m1_decode(const uint8_t* codes, int64_t n, float* out, mpsa_stream_t stream);
 int mpsa_e8m0_encode(const float* x, int64_t n, uint8_t* codes, mpsa_stream_t stream);
 int mpsa_e8m0_decode(const uint8_t* codes, int64_t n, float* out, mpsa_stream_t stream);
+
+/*
+ * float32 -> one FP8 byte per element, fmt MPSA_FMT_E5M2 | MPSA_FMT_E4M3: the elementwise cast the reference's operand
+ * packaging applies to its 8-bit operands, a_tensor.to(torch.float8_e5m2) (ours/block_scaled_matmul.py:334-336,
+ * :349-351; ours/mxfp_attn_kernel.py:467-469, :479-481): round to nearest even, no saturation (E5M2 overflows to
+ * infinity, E4M3 - which has no infinity - to NaN), NaN stays NaN.  No block scale is derived here: this is not the
+ * MX quantizer.
+ */
+int mpsa_fp8_encode(const float* x, int64_t n, int fmt, uint8_t* codes, mpsa_stream_t stream);
 
 /*
  * Nibble packing of E2M1 codes along one dimension of a contiguous tensor seen as [outer, n, inner]:
@@ -152,13 +172,16 @@ int mpsa_seq_mean_static(const void* x, int x_dtype, int64_t B, int64_t H, int64
  *
  *   a, b     packed codes [M,K/2] / [N,K/2] (E2M1) or [M,K] / [N,K] (8-bit), row-major, contiguous
  *   sa, sb   E8M0 bytes [M,K/32] / [N,K/32], row-major (the linear layout; mpsa_gemm_mx_packed below takes the 5-D packed one)
- *   fmt      element format of both operands
+ *   fmt_a, fmt_b   element format of each operand (MPSA_FMT_*); they may differ - the reference's "mixed" type is an
+ *            8-bit A with a 4-bit B (ELEM_PER_BYTE_A / ELEM_PER_BYTE_B, ours/block_scaled_matmul.py:318-324, :252-257)
  *   c        [M,N] of c_dtype (MPSA_BF16 | MPSA_F16 | MPSA_F32 | MPSA_F8E5M2: one E5M2 byte per element, round to
  *            nearest even, overflow to infinity - the reference's output dtypes are f32, f16 and e5m2,
  *            ours/block_scaled_matmul.py:185-190, :273-280), leading dimension ldc elements
- *   M % 256 == 0, N % 256 == 0, K % 128 == 0
+ *   M, N >= 1 (edge tiles are masked, as in the reference's kernel), K % 64 == 0.  Equal formats with M % 256 == 0,
+ *   N % 256 == 0 and K % 128 == 0 run on the LDS-staged 256 x 256 kernel, every other case on a 128 x 128 kernel
+ *   that reads its operands straight from L2 (same results; MPSA_GEMM_GENERAL=1 in the environment forces it).
  */
-int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
+int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, int fmt_a, const uint8_t* b, const uint8_t* sb, int fmt_b,
                  int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream);
 
 /*
@@ -168,7 +191,7 @@ int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const ui
  * Triton kernel (ours/batched_block_scaled_matmul.py:183-236, :43-180) - the batched Q.K^T of the reference's
  * mxfp_attn (ours/mxfp_attn.py:64-66) - with the 2-D kernel's semantics.
  */
-int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
+int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, int fmt_a, const uint8_t* b, const uint8_t* sb, int fmt_b,
                          int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
                          void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream);
 
@@ -178,11 +201,12 @@ int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, const uint8_t* b, 
  * and what mpsa_scales_to_5d produces: byte (r%32)*16 + (r/32 % 4)*4 + k of chunk (r/128, kb/4) is the scale of row r,
  * K block kb = 4*(kb/4) + k.  The kernel fetches a 128-row x 128-element chunk as 512 contiguous bytes (a quarter of
  * the cache lines the row-major layout costs) and reads a lane's scale words for four row blocks with one 128-bit
- * LDS read.  Same results as the row-major entry points, bit for bit.  sa5, sb5: 16-byte aligned.
+ * LDS read.  Same results as the row-major entry points, bit for bit.  sa5, sb5: 16-byte aligned; M, N and K in
+ * multiples of 128 (the layout's chunk).
  */
-int mpsa_gemm_mx_packed(const uint8_t* a, const uint8_t* sa5, const uint8_t* b, const uint8_t* sb5, int fmt,
+int mpsa_gemm_mx_packed(const uint8_t* a, const uint8_t* sa5, int fmt_a, const uint8_t* b, const uint8_t* sb5, int fmt_b,
                         int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream);
-int mpsa_gemm_mx_batched_packed(const uint8_t* a, const uint8_t* sa5, const uint8_t* b, const uint8_t* sb5, int fmt,
+int mpsa_gemm_mx_batched_packed(const uint8_t* a, const uint8_t* sa5, int fmt_a, const uint8_t* b, const uint8_t* sb5, int fmt_b,
                                 int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
                                 void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream);
 
@@ -203,7 +227,7 @@ int mpsa_v_tiles(const void* v, int v_dtype, int64_t B, int64_t H, int64_t N, in
  *
  *   q [B,Hq,Nq,D], k and v [B,Hkv,Nk,D] of dtype (MPSA_BF16 | MPSA_F16), element strides as for mpsa_quantize_mx
  *   mode       MPSA_MODE_MXFP4: only the 4-bit outputs are written (8-bit pointers may be null),
- *              MPSA_MODE_MXFP8: only the 8-bit ones, MPSA_MODE_DIAG / MPSA_MODE_ROUTED: both
+ *              MPSA_MODE_MXFP8: only the 8-bit ones, MPSA_MODE_DIAG / MPSA_MODE_ROUTED / MPSA_MODE_MIXED: both
  *   k_sub      NULL or [B,Hkv,D] (smooth-K mean from mpsa_seq_mean)
  *   outputs    as the inputs of mpsa_attn_fwd
  */
@@ -222,7 +246,8 @@ int mpsa_attn_prepare(const void* q, const int64_t q_strides[4], const void* k, 
  *   q4,qs4 / q8,qs8   Q codes + scales from the quantizer, rows padded to nq_pad per head:
  *                     [B,Hq,nq_pad,D/2],[B,Hq,nq_pad,D/32] and [B,Hq,nq_pad,D],[B,Hq,nq_pad,D/32]
  *   k4,ks4 / k8,ks8   same for K with Hkv heads and nk_pad rows
- *                     (the 4-bit set may be null in MPSA_MODE_MXFP8, the 8-bit set in MPSA_MODE_MXFP4)
+ *                     (the 4-bit set may be null in MPSA_MODE_MXFP8, the 8-bit set in MPSA_MODE_MXFP4;
+ *                     MPSA_MODE_MIXED reads q8, qs8, k4, ks4 only)
  *   fmt8              MPSA_FMT_E4M3 | MPSA_FMT_E5M2
  *   v_tiles           output of mpsa_v_tiles for the same tile, pv_dtype (MPSA_BF16 | MPSA_F16);
  *                     P is rounded to that dtype before P.V

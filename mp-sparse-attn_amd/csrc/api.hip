@@ -1,5 +1,8 @@
 // Version and error reporting of libmpsa.
 #include "mpsa_common.h"
+#include <atomic>
+#include <mutex>
+#include <vector>
 
 static thread_local char g_err[512] = "";
 
@@ -13,3 +16,39 @@ int mpsa_fail(int code, const char* fmt, ...) {
 
 extern "C" int mpsa_version(void) { return 100; }
 extern "C" const char* mpsa_last_error(void) { return g_err; }
+
+namespace {
+struct LdsEntry { const void* kern; int bytes; };
+std::vector<LdsEntry>& lds_registry() { static std::vector<LdsEntry> r; return r; }
+std::mutex& init_mutex() { static std::mutex m; return m; }
+std::atomic<bool> g_device_ready[MPSA_MAX_DEVICES];
+}  // namespace
+
+bool mpsa_register_lds_kernel(const void* kern, int bytes) {
+    std::lock_guard<std::mutex> lock(init_mutex());
+    lds_registry().push_back({kern, bytes});
+    return true;
+}
+
+extern "C" int mpsa_init(void) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "init: hipGetDevice: %s", hipGetErrorString(e));
+    {
+        std::lock_guard<std::mutex> lock(init_mutex());
+        for (const LdsEntry& k : lds_registry()) {
+            e = hipFuncSetAttribute(k.kern, hipFuncAttributeMaxDynamicSharedMemorySize, k.bytes);
+            if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "init: cannot reserve %d bytes of LDS for a kernel: %s", k.bytes, hipGetErrorString(e));
+        }
+    }
+    const int rc = mpsa_seq_mean_static_resolve();
+    if (rc != MPSA_OK) return rc;
+    if (dev >= 0 && dev < MPSA_MAX_DEVICES) g_device_ready[dev].store(true, std::memory_order_release);
+    return MPSA_OK;
+}
+
+int mpsa_ensure_init() {
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < MPSA_MAX_DEVICES && g_device_ready[dev].load(std::memory_order_acquire)) return MPSA_OK;
+    return mpsa_init();
+}

@@ -67,6 +67,12 @@ __device__ __forceinline__ v16f score_mfma8(v8i k, v8i q, v16f c, int sel, int k
     if (sel == 0) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, FMT8, FMT8, 0, ks, 0, qs);
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, FMT8, FMT8, 2, ks, 2, qs);
 }
+// 4-bit K operand x 8-bit Q operand ("mixed"): each operand's registers follow its own format's layout
+template <int FMT8>
+__device__ __forceinline__ v16f score_mfma48(v8i k, v8i q, v16f c, int sel, int ks, int qs) {
+    if (sel == 0) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, 4, FMT8, 0, ks, 0, qs);
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, 4, FMT8, 2, ks, 2, qs);
+}
 __device__ __forceinline__ v16f score_mfma4(v8i k, v8i q, v16f c, int sel, int ks, int qs) {
     if (sel == 0) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, 4, 4, 0, ks, 0, qs);
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(k, q, c, 4, 4, 2, ks, 2, qs);

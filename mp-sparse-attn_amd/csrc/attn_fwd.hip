@@ -37,6 +37,9 @@ namespace {
 template <int D, int TILE, int PVT>
 int launch_mode(const AttnArgs& a, hipStream_t st) {
     if (a.mode == MPSA_MODE_MXFP4) return launch_one<D, TILE, PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP4>(a, st);
+    if (a.mode == MPSA_MODE_MIXED)
+        return a.fmt8 == MPSA_FMT_E5M2 ? launch_one<D, TILE, PVT, MPSA_FMT_E5M2, MPSA_MODE_MIXED>(a, st)
+                                       : launch_one<D, TILE, PVT, MPSA_FMT_E4M3, MPSA_MODE_MIXED>(a, st);
     if (a.mode == MPSA_MODE_MXFP8)
         return a.fmt8 == MPSA_FMT_E5M2 ? launch_one<D, TILE, PVT, MPSA_FMT_E5M2, MPSA_MODE_MXFP8>(a, st)
                                        : launch_one<D, TILE, PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP8>(a, st);
@@ -58,13 +61,18 @@ static int attn_entry(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, 
                       int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal, int mode,
                       bool skip, float skip_thresh, int32_t* skipped, const int32_t* order, const int32_t* counts,
                       mpsa_stream_t stream) {
-    if (mode != MPSA_MODE_MXFP4 && mode != MPSA_MODE_MXFP8 && mode != MPSA_MODE_DIAG && mode != MPSA_MODE_ROUTED) return mpsa_fail(MPSA_EINVAL, "attn: unknown mode %d", mode);
+    if (mode != MPSA_MODE_MXFP4 && mode != MPSA_MODE_MXFP8 && mode != MPSA_MODE_DIAG && mode != MPSA_MODE_ROUTED && mode != MPSA_MODE_MIXED) return mpsa_fail(MPSA_EINVAL, "attn: unknown mode %d", mode);
     const bool routed = mode == MPSA_MODE_ROUTED;
     if (routed && (!order || !counts)) return mpsa_fail(MPSA_EINVAL, "attn: a routed run needs the visiting lists (order, counts)");
     if (routed && ((reinterpret_cast<uintptr_t>(order) | reinterpret_cast<uintptr_t>(counts)) & 3)) return mpsa_fail(MPSA_EALIGN, "attn: order and counts must be 4-byte aligned");
+    const bool mixed = mode == MPSA_MODE_MIXED;
     const bool need4 = mode != MPSA_MODE_MXFP8, need8 = mode != MPSA_MODE_MXFP4;
-    if (need4 && (!q4 || !qs4 || !k4 || !ks4)) return mpsa_fail(MPSA_EINVAL, "attn: 4-bit operands missing");
-    if (need8 && (!q8 || !qs8 || !k8 || !ks8)) return mpsa_fail(MPSA_EINVAL, "attn: 8-bit operands missing");
+    if (mixed) {
+        if (!q8 || !qs8 || !k4 || !ks4) return mpsa_fail(MPSA_EINVAL, "attn: the mixed mode needs 8-bit Q and 4-bit K operands");
+    } else {
+        if (need4 && (!q4 || !qs4 || !k4 || !ks4)) return mpsa_fail(MPSA_EINVAL, "attn: 4-bit operands missing");
+        if (need8 && (!q8 || !qs8 || !k8 || !ks8)) return mpsa_fail(MPSA_EINVAL, "attn: 8-bit operands missing");
+    }
     if (!v_tiles || !o || !o_strides) return mpsa_fail(MPSA_EINVAL, "attn: null pointer");
     if (need8 && fmt8 != MPSA_FMT_E4M3 && fmt8 != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "attn: 8-bit format must be E4M3 or E5M2");
     if (pv_dtype != MPSA_BF16 && pv_dtype != MPSA_F16) return mpsa_fail(MPSA_EINVAL, "attn: pv_dtype must be bf16 or f16");
@@ -92,22 +100,17 @@ static int attn_entry(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, 
     hipStream_t st = (hipStream_t)stream;
     if (routed) return attn_routed_launch(a, pv_dtype, st);
     if (skip) {
+        if (mixed) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: tile skipping is built for the mxfp4 and mxfp8 modes only");
         if (mode == MPSA_MODE_DIAG) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: tile skipping needs a single-precision mode (mxfp4 or mxfp8): the rule's reference tile is the first key tile, which a diag run visits last for query tile 0");
         if (!(skip_thresh == skip_thresh)) return mpsa_fail(MPSA_EINVAL, "attn: skip_thresh is NaN");
         if (skipped && (reinterpret_cast<uintptr_t>(skipped) & 3)) return mpsa_fail(MPSA_EALIGN, "attn: skipped must be 4-byte aligned");
         return attn_skip_launch(a, pv_dtype, st);
     }
     if (attn_pp_supported(a, pv_dtype)) return attn_pp_launch(a, pv_dtype, st);
-#ifdef MPSA_ATTN_ONLY_128
-    if (D == 128 && tile == 128 && pv_dtype == MPSA_BF16 && fmt8 == MPSA_FMT_E4M3 && mode == MPSA_MODE_DIAG)
-        return launch_one<128, 128, MPSA_BF16, MPSA_FMT_E4M3, MPSA_MODE_DIAG>(a, st);
-    return mpsa_fail(MPSA_EUNSUPPORTED, "attn: development build with a single variant");
-#else
     if (D == 128 && tile == 128) return launch_dt<128, 128>(a, pv_dtype, st);
     if (D == 64 && tile == 64)   return launch_dt<64, 64>(a, pv_dtype, st);
     if (D == 128 && tile == 64)  return launch_dt<128, 64>(a, pv_dtype, st);
     return launch_dt<64, 128>(a, pv_dtype, st);
-#endif
 }
 
 extern "C" int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,

@@ -81,6 +81,7 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     // treatment go LAST: first every plain tile (main precision, no mask) in one tight loop, then the tile that
     // holds the sequence tail (masked) if there is one, then the diagonal tile i (causal mask and / or 8-bit).
     constexpr bool ROUTED = MODE == MPSA_MODE_ROUTED;
+    constexpr bool MIXED = MODE == MPSA_MODE_MIXED;       // every tile: 8-bit Q against 4-bit K
     constexpr bool HAS4 = MODE != MPSA_MODE_MXFP8;        // 4-bit tiles exist (LDS pipeline in use)
     constexpr bool PRE8 = MODE == MPSA_MODE_MXFP8 || ROUTED;   // 8-bit K fragments are prefetched one step ahead
     const bool tail = a.n < a.n_pad;
@@ -273,7 +274,7 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         if (!ROUTED || first8) issue_k8(tile_rel(0, R0{}));
     }
     load_kscales(tile_rel(0, R0{}), first8);
-    load_q(first8);
+    load_q(first8 || MIXED);
     __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0)
     __syncthreads();
     if constexpr (HAS4) read_kf4(0);
@@ -317,7 +318,8 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
                 for (int s = 0; s < G::SST; ++s) {
                     const v4i x = kf4[kb][s];
                     const v8i k8v = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
-                    st[kb] = score_mfma4(k8v, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
+                    if constexpr (MIXED) st[kb] = score_mfma48<FMT8>(k8v, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
+                    else                 st[kb] = score_mfma4(k8v, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
                 }
             }
         }
@@ -555,16 +557,22 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     }
 }
 
+template <int D, int TILE, int PVT, int FMT8, int MODE, bool SKIP>
+struct AttnLds {
+    static constexpr int smem = Geom<D, TILE>::SMEM + (SKIP ? 2 * Geom<D, TILE>::NW * (int)sizeof(float) : 0);
+    static inline const bool registered =
+        mpsa_register_lds_kernel(reinterpret_cast<const void*>(attn_fwd_kernel<D, TILE, PVT, FMT8, MODE, SKIP>), smem);
+};
+
 template <int D, int TILE, int PVT, int FMT8, int MODE, bool SKIP = false>
 int launch_one(const AttnArgs& a, hipStream_t st) {
     typedef Geom<D, TILE> G;
-    constexpr int smem = G::SMEM + (SKIP ? 2 * G::NW * (int)sizeof(float) : 0);
-    static bool reserved[MPSA_MAX_DEVICES] = {};
-    auto kern = attn_fwd_kernel<D, TILE, PVT, FMT8, MODE, SKIP>;
-    const hipError_t e = mpsa_reserve_lds(reinterpret_cast<const void*>(kern), smem, reserved);
-    if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "attn: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
+    typedef AttnLds<D, TILE, PVT, FMT8, MODE, SKIP> L;
+    if (!L::registered) return mpsa_fail(MPSA_ELAUNCH, "attn: kernel not registered");
+    const int rc = mpsa_ensure_init();
+    if (rc != MPSA_OK) return rc;
     dim3 grid((unsigned)(a.B * a.Hq * a.ntq));
-    hipLaunchKernelGGL(kern, grid, dim3(G::NT), smem, st, a);
+    hipLaunchKernelGGL((attn_fwd_kernel<D, TILE, PVT, FMT8, MODE, SKIP>), grid, dim3(G::NT), L::smem, st, a);
     MPSA_CHECK_LAUNCH("attn");
     return MPSA_OK;
 }

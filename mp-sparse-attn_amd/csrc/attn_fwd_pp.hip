@@ -452,13 +452,17 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
 }
 
 template <int PVT, int FMT8, int MODE>
+struct PpLds {
+    static inline const bool registered = mpsa_register_lds_kernel(reinterpret_cast<const void*>(attn_pp_kernel<PVT, FMT8, MODE>), SMEM);
+};
+
+template <int PVT, int FMT8, int MODE>
 int launch_pp(const AttnArgs& a, hipStream_t st) {
-    static bool reserved[MPSA_MAX_DEVICES] = {};
-    auto kern = attn_pp_kernel<PVT, FMT8, MODE>;
-    const hipError_t e = mpsa_reserve_lds(reinterpret_cast<const void*>(kern), SMEM, reserved);
-    if (e != hipSuccess) return mpsa_fail(MPSA_ELAUNCH, "attn: cannot reserve %d bytes of LDS: %s", SMEM, hipGetErrorString(e));
+    if (!PpLds<PVT, FMT8, MODE>::registered) return mpsa_fail(MPSA_ELAUNCH, "attn: kernel not registered");
+    const int rc = mpsa_ensure_init();
+    if (rc != MPSA_OK) return rc;
     dim3 grid((unsigned)(a.B * a.Hq * (a.nt / 2)));
-    hipLaunchKernelGGL(kern, grid, dim3(512), SMEM, st, a);
+    hipLaunchKernelGGL((attn_pp_kernel<PVT, FMT8, MODE>), grid, dim3(512), SMEM, st, a);
     MPSA_CHECK_LAUNCH("attn(pp)");
     return MPSA_OK;
 }

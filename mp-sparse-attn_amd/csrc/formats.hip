@@ -60,6 +60,42 @@ __global__ __launch_bounds__(256) void e8m0_decode_kernel(const uint8_t* c, int6
     out[i] = e == 255u ? mpsa_u2f(0x7FC00000u) : (e == 0u ? mpsa_u2f(0x00400000u) : mpsa_u2f(e << 23));
 }
 
+// float32 -> one FP8 byte, the cast torch performs for x.to(torch.float8_e5m2) / x.to(torch.float8_e4m3fn): round to
+// nearest even, no saturation.  E5M2 overflows to infinity (0x7C) and keeps NaN (0x7F); E4M3 ("fn": no infinities)
+// turns everything that rounds beyond 448 into NaN (0x7F).  The reference's operand packaging casts its 8-bit
+// operands this way (ours/block_scaled_matmul.py:334-336, :349-351).
+template <int FMT>
+__global__ __launch_bounds__(256) void fp8_encode_kernel(const float* x, int64_t n, uint8_t* out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t u = mpsa_f2u(x[i]);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    uint32_t a = u & 0x7FFFFFFFu;
+    uint32_t code;
+    if (a > 0x7F800000u) {
+        code = 0x7Fu;
+    } else if constexpr (FMT == MPSA_FMT_E5M2) {
+        if (a >= 0x38800000u) {                       // |x| >= 2^-14: normal
+            a += 0xFFFFFu + ((a >> 21) & 1u);
+            code = (a >> 21) - (112u << 2);
+            code = code > 0x7Cu ? 0x7Cu : code;
+        } else {                                      // subnormal, unit 2^-16
+            code = mpsa_f2u(mpsa_u2f(a) + 128.0f) - 0x43000000u;
+        }
+    } else {
+        if (a >= 0x43F00000u) {                       // |x| >= 480 (incl. infinity)
+            code = 0x7Fu;
+        } else if (a >= 0x3C800000u) {                // |x| >= 2^-6: normal
+            a += 0x7FFFFu + ((a >> 20) & 1u);
+            code = (a >> 20) - (120u << 3);
+            code = code > 0x7Fu ? 0x7Fu : code;
+        } else {                                      // subnormal, unit 2^-9
+            code = mpsa_f2u(mpsa_u2f(a) + 16384.0f) - 0x46800000u;
+        }
+    }
+    out[i] = (uint8_t)(sign | code);
+}
+
 template <typename K, typename... A>
 int run(const char* what, K kern, int64_t n, hipStream_t st, A... args) {
     if (n < 0) return mpsa_fail(MPSA_EINVAL, "%s: negative length", what);
@@ -167,4 +203,10 @@ extern "C" int mpsa_e8m0_encode(const float* x, int64_t n, uint8_t* codes, mpsa_
 extern "C" int mpsa_e8m0_decode(const uint8_t* codes, int64_t n, float* out, mpsa_stream_t stream) {
     if (n > 0 && (!codes || !out)) return mpsa_fail(MPSA_EINVAL, "e8m0_decode: null pointer");
     return run("e8m0_decode", e8m0_decode_kernel, n, (hipStream_t)stream, codes, n, out);
+}
+extern "C" int mpsa_fp8_encode(const float* x, int64_t n, int fmt, uint8_t* codes, mpsa_stream_t stream) {
+    if (fmt != MPSA_FMT_E4M3 && fmt != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "fp8_encode: format must be E4M3 or E5M2");
+    if (n > 0 && (!x || !codes)) return mpsa_fail(MPSA_EINVAL, "fp8_encode: null pointer");
+    if (fmt == MPSA_FMT_E5M2) return run("fp8_encode", fp8_encode_kernel<MPSA_FMT_E5M2>, n, (hipStream_t)stream, x, n, codes);
+    return run("fp8_encode", fp8_encode_kernel<MPSA_FMT_E4M3>, n, (hipStream_t)stream, x, n, codes);
 }

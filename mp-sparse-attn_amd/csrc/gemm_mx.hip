@@ -412,13 +412,148 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
         }
 }
 
+// ---- general kernel: any M and N (edge tiles masked), operands of different element formats ----
+// The reference's kernel tiles 128 x 256 with masked edges (ours/block_scaled_matmul.py:154-267) and takes the two
+// operands' element widths separately (ELEM_PER_BYTE_A / ELEM_PER_BYTE_B, "mixed" = 8-bit A x 4-bit B,
+// ours/block_scaled_matmul.py:318-324).  This kernel covers what the 256 x 256 kernel above does not: a workgroup of
+// four waves owns a 128 x 128 tile, a wave 64 x 64 (2 x 2 accumulators); operand fragments and scale bytes come
+// straight from global memory (L2), one 64-element step ahead of the matrix instructions.  Rows past M or N are
+// read from the last valid row and never stored.  Each operand's registers follow its own format's layout (4-bit:
+// the lane half's registers are MX block h of the step; 8-bit: registers 0-3 of both halves are block 0, 4-7 block 1).
+template <int FMT>
+__device__ __forceinline__ v8i load_frag(const uint8_t* row_ptr, int ks, int h) {
+    if constexpr (FMT == MPSA_FMT_E2M1) {
+        const v4i x = *reinterpret_cast<const v4i*>(row_ptr + ks * 32 + h * 16);
+        return (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+    } else {
+        const v4i x0 = *reinterpret_cast<const v4i*>(row_ptr + ks * 64 + h * 16);
+        const v4i x1 = *reinterpret_cast<const v4i*>(row_ptr + ks * 64 + h * 16 + 32);
+        return (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+    }
+}
+
+// scale byte of row `row`, MX block kb: row-major [rows, K/32] or the packed [rows/128, K/128, 32, 4, 4] form
+__device__ __forceinline__ int load_scale(const uint8_t* s, int row, int kb, int kblocks, bool packed) {
+    if (!packed) return s[(int64_t)row * kblocks + kb];
+    const int64_t chunk = (int64_t)(row >> 7) * (kblocks >> 2) + (kb >> 2);
+    return s[chunk * 512 + (row & 31) * 16 + ((row >> 5) & 3) * 4 + (kb & 3)];
+}
+
+template <int FA, int FB, typename OutT>
+__global__ __launch_bounds__(256) void gemm_mx_general_kernel(GemmArgs g) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int h = lane >> 5, r = lane & 31;
+    const int rowb_a = FA == MPSA_FMT_E2M1 ? g.K / 2 : g.K;
+    const int rowb_b = FB == MPSA_FMT_E2M1 ? g.K / 2 : g.K;
+    const int kblocks = g.K / 32;
+    const int tiles_n = (g.N + 127) / 128;
+    const int m0 = (blockIdx.x / tiles_n) * 128 + wm * 64;
+    const int n0 = (blockIdx.x % tiles_n) * 128 + wn * 64;
+    const int bz = blockIdx.y;
+    const int bb = bz / g.heads_a, ha = bz - bb * g.heads_a;
+    const int64_t zb = (int64_t)bb * g.heads_b + ha / (g.heads_a / g.heads_b);
+    // scale rows per matrix: the packed form pads nothing (rows % 128 == 0 is required for it)
+    const uint8_t* a = g.a + (int64_t)bz * g.M * rowb_a;
+    const uint8_t* b = g.b + zb * g.N * rowb_b;
+    const uint8_t* sa = g.sa + (int64_t)bz * g.M * kblocks;
+    const uint8_t* sb = g.sb + zb * g.N * kblocks;
+    int ra[2], rb[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        ra[i] = min(m0 + i * 32 + r, g.M - 1);
+        rb[i] = min(n0 + i * 32 + r, g.N - 1);
+    }
+    v16f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    const int steps = g.K / 64;
+    v8i fa[2], fb[2];
+    int ca[2], cb[2];
+    auto fetch = [&](int ks, v8i (&xa)[2], v8i (&xb)[2], int (&ya)[2], int (&yb)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            xa[i] = load_frag<FA>(a + (int64_t)ra[i] * rowb_a, ks, h);
+            xb[i] = load_frag<FB>(b + (int64_t)rb[i] * rowb_b, ks, h);
+            ya[i] = load_scale(sa, ra[i], 2 * ks + h, kblocks, g.packed != 0);
+            yb[i] = load_scale(sb, rb[i], 2 * ks + h, kblocks, g.packed != 0);
+        }
+    };
+    fetch(0, fa, fb, ca, cb);
+    for (int ks = 0; ks < steps; ++ks) {
+        v8i na[2], nb[2];
+        int da[2], db[2];
+        fetch(ks + 1 < steps ? ks + 1 : ks, na, nb, da, db);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], FA, FB, 0, ca[i], 0, cb[j]);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) { fa[i] = na[i]; fb[i] = nb[i]; ca[i] = da[i]; cb[i] = db[i]; }
+    }
+
+    // accumulator register e of lane (h, r) is C[8*(e/4) + 4*h + e%4][r] of its 32 x 32 block
+    OutT* c = static_cast<OutT*>(g.c) + (int64_t)bz * g.M * g.ldc;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = n0 + j * 32 + r;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int row = m0 + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+                if (row < g.M && col < g.N) c[(int64_t)row * g.ldc + col] = cvt_out<OutT>(acc[i][j][e]);
+            }
+        }
+}
+
+template <int FA, int FB>
+void launch_general_out(const GemmArgs& g, int c_dtype, dim3 grid, hipStream_t st) {
+    if (c_dtype == MPSA_BF16)        hipLaunchKernelGGL((gemm_mx_general_kernel<FA, FB, __bf16>), grid, dim3(256), 0, st, g);
+    else if (c_dtype == MPSA_F8E5M2) hipLaunchKernelGGL((gemm_mx_general_kernel<FA, FB, OutE5M2>), grid, dim3(256), 0, st, g);
+    else if (c_dtype == MPSA_F16)    hipLaunchKernelGGL((gemm_mx_general_kernel<FA, FB, _Float16>), grid, dim3(256), 0, st, g);
+    else                             hipLaunchKernelGGL((gemm_mx_general_kernel<FA, FB, float>), grid, dim3(256), 0, st, g);
+}
+
+template <int FA>
+void launch_general_b(const GemmArgs& g, int fmt_b, int c_dtype, dim3 grid, hipStream_t st) {
+    if (fmt_b == MPSA_FMT_E2M1)      launch_general_out<FA, MPSA_FMT_E2M1>(g, c_dtype, grid, st);
+    else if (fmt_b == MPSA_FMT_E4M3) launch_general_out<FA, MPSA_FMT_E4M3>(g, c_dtype, grid, st);
+    else                             launch_general_out<FA, MPSA_FMT_E5M2>(g, c_dtype, grid, st);
+}
+
+void launch_general(const GemmArgs& g, int fmt_a, int fmt_b, int c_dtype, dim3 grid, hipStream_t st) {
+    if (fmt_a == MPSA_FMT_E2M1)      launch_general_b<MPSA_FMT_E2M1>(g, fmt_b, c_dtype, grid, st);
+    else if (fmt_a == MPSA_FMT_E4M3) launch_general_b<MPSA_FMT_E4M3>(g, fmt_b, c_dtype, grid, st);
+    else                             launch_general_b<MPSA_FMT_E5M2>(g, fmt_b, c_dtype, grid, st);
+}
+
+// MPSA_GEMM_GENERAL=1 in the environment sends every shape to the general kernel (cross-checking)
+bool force_general() {
+    static const bool on = [] {
+        const char* v = getenv("MPSA_GEMM_GENERAL");
+        return v && v[0] == '1';
+    }();
+    return on;
+}
+
+template <int FMT, typename OutT, bool WIDE, bool PK>
+struct GemmLds {
+    static inline const bool registered =
+        mpsa_register_lds_kernel(reinterpret_cast<const void*>(gemm_mx_kernel<FMT, OutT, WIDE, PK>), smem_bytes<WIDE>());
+};
+
 template <int FMT, typename OutT, bool WIDE, bool PK>
 void launch_kernel(const GemmArgs& g, dim3 grid, hipStream_t st) {
-    static bool reserved[MPSA_MAX_DEVICES] = {};
-    auto kern = gemm_mx_kernel<FMT, OutT, WIDE, PK>;
-    // a failure here shows up as a launch error, which the caller reports
-    (void)mpsa_reserve_lds(reinterpret_cast<const void*>(kern), smem_bytes<WIDE>(), reserved);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem_bytes<WIDE>(), st, g);
+    if (!GemmLds<FMT, OutT, WIDE, PK>::registered) return;
+    hipLaunchKernelGGL((gemm_mx_kernel<FMT, OutT, WIDE, PK>), grid, dim3(256), smem_bytes<WIDE>(), st, g);
 }
 
 template <int FMT, typename OutT>
@@ -438,16 +573,19 @@ void launch_fmt(const GemmArgs& g, int c_dtype, dim3 grid, hipStream_t st) {
 
 }  // namespace
 
-static int gemm_entry(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt, bool packed,
+static bool known_fmt(int f) { return f == MPSA_FMT_E2M1 || f == MPSA_FMT_E4M3 || f == MPSA_FMT_E5M2; }
+
+static int gemm_entry(const uint8_t* a, const uint8_t* sa, int fmt_a, const uint8_t* b, const uint8_t* sb, int fmt_b, bool packed,
                       int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
                       void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
     if (!a || !sa || !b || !sb || !c) return mpsa_fail(MPSA_EINVAL, "gemm: null pointer");
-    if (fmt != MPSA_FMT_E2M1 && fmt != MPSA_FMT_E4M3 && fmt != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "gemm: unknown format %d", fmt);
+    if (!known_fmt(fmt_a) || !known_fmt(fmt_b)) return mpsa_fail(MPSA_EINVAL, "gemm: unknown format %d / %d", fmt_a, fmt_b);
     if (c_dtype != MPSA_BF16 && c_dtype != MPSA_F16 && c_dtype != MPSA_F32 && c_dtype != MPSA_F8E5M2) return mpsa_fail(MPSA_EINVAL, "gemm: unsupported output dtype %d", c_dtype);
     if (M <= 0 || N <= 0 || K <= 0 || ldc < N) return mpsa_fail(MPSA_EINVAL, "gemm: bad shape");
     if (batch <= 0 || heads_a <= 0 || heads_b <= 0 || heads_a % heads_b) return mpsa_fail(MPSA_EINVAL, "gemm: bad batch shape (batch=%lld heads_a=%lld heads_b=%lld)", (long long)batch, (long long)heads_a, (long long)heads_b);
-    if (M % BM || N % BN || K % 128) return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: M,N must be multiples of 256 and K of 128 (got %lld,%lld,%lld)", (long long)M, (long long)N, (long long)K);
-    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 24) || (M / BM) * (N / BN) > (int64_t(1) << 30) || batch * heads_a > 65535)
+    if (K % 64) return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: K must be a multiple of 64 (got %lld)", (long long)K);
+    if (packed && (M % 128 || N % 128 || K % 128)) return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: packed scales need M, N and K in multiples of 128 (got %lld,%lld,%lld)", (long long)M, (long long)N, (long long)K);
+    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 24) || ((M + 127) / 128) * ((N + 127) / 128) > (int64_t(1) << 30) || batch * heads_a > 65535)
         return mpsa_fail(MPSA_EUNSUPPORTED, "gemm: shape too large");
     if (!mpsa_aligned16(a) || !mpsa_aligned16(b) || (reinterpret_cast<uintptr_t>(sa) & 3) || (reinterpret_cast<uintptr_t>(sb) & 3))
         return mpsa_fail(MPSA_EALIGN, "gemm: codes must be 16-byte and scales 4-byte aligned");
@@ -457,33 +595,41 @@ static int gemm_entry(const uint8_t* a, const uint8_t* sa, const uint8_t* b, con
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.heads_a = (int)heads_a; g.heads_b = (int)heads_b;
     g.packed = packed ? 1 : 0;
-    dim3 grid((unsigned)((M / BM) * (N / BN)), (unsigned)(batch * heads_a));
     hipStream_t st = (hipStream_t)stream;
-    if (fmt == MPSA_FMT_E2M1)      launch_fmt<MPSA_FMT_E2M1>(g, c_dtype, grid, st);
-    else if (fmt == MPSA_FMT_E4M3) launch_fmt<MPSA_FMT_E4M3>(g, c_dtype, grid, st);
-    else                           launch_fmt<MPSA_FMT_E5M2>(g, c_dtype, grid, st);
+    const int rc = mpsa_ensure_init();
+    if (rc != MPSA_OK) return rc;
+    // whole 256 x 256 tiles of one element format: the LDS-staged kernel; everything else: the general one
+    if (fmt_a == fmt_b && M % BM == 0 && N % BN == 0 && K % 128 == 0 && !force_general()) {
+        dim3 grid((unsigned)((M / BM) * (N / BN)), (unsigned)(batch * heads_a));
+        if (fmt_a == MPSA_FMT_E2M1)      launch_fmt<MPSA_FMT_E2M1>(g, c_dtype, grid, st);
+        else if (fmt_a == MPSA_FMT_E4M3) launch_fmt<MPSA_FMT_E4M3>(g, c_dtype, grid, st);
+        else                             launch_fmt<MPSA_FMT_E5M2>(g, c_dtype, grid, st);
+    } else {
+        dim3 grid((unsigned)(((M + 127) / 128) * ((N + 127) / 128)), (unsigned)(batch * heads_a));
+        launch_general(g, fmt_a, fmt_b, c_dtype, grid, st);
+    }
     MPSA_CHECK_LAUNCH("gemm");
     return MPSA_OK;
 }
 
-extern "C" int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
+extern "C" int mpsa_gemm_mx_batched(const uint8_t* a, const uint8_t* sa, int fmt_a, const uint8_t* b, const uint8_t* sb, int fmt_b,
                                     int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
                                     void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
-    return gemm_entry(a, sa, b, sb, fmt, false, batch, heads_a, heads_b, M, N, K, c, c_dtype, ldc, stream);
+    return gemm_entry(a, sa, fmt_a, b, sb, fmt_b, false, batch, heads_a, heads_b, M, N, K, c, c_dtype, ldc, stream);
 }
 
-extern "C" int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, const uint8_t* b, const uint8_t* sb, int fmt,
+extern "C" int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, int fmt_a, const uint8_t* b, const uint8_t* sb, int fmt_b,
                             int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
-    return gemm_entry(a, sa, b, sb, fmt, false, 1, 1, 1, M, N, K, c, c_dtype, ldc, stream);
+    return gemm_entry(a, sa, fmt_a, b, sb, fmt_b, false, 1, 1, 1, M, N, K, c, c_dtype, ldc, stream);
 }
 
-extern "C" int mpsa_gemm_mx_packed(const uint8_t* a, const uint8_t* sa5, const uint8_t* b, const uint8_t* sb5, int fmt,
+extern "C" int mpsa_gemm_mx_packed(const uint8_t* a, const uint8_t* sa5, int fmt_a, const uint8_t* b, const uint8_t* sb5, int fmt_b,
                                    int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
-    return gemm_entry(a, sa5, b, sb5, fmt, true, 1, 1, 1, M, N, K, c, c_dtype, ldc, stream);
+    return gemm_entry(a, sa5, fmt_a, b, sb5, fmt_b, true, 1, 1, 1, M, N, K, c, c_dtype, ldc, stream);
 }
 
-extern "C" int mpsa_gemm_mx_batched_packed(const uint8_t* a, const uint8_t* sa5, const uint8_t* b, const uint8_t* sb5, int fmt,
+extern "C" int mpsa_gemm_mx_batched_packed(const uint8_t* a, const uint8_t* sa5, int fmt_a, const uint8_t* b, const uint8_t* sb5, int fmt_b,
                                            int64_t batch, int64_t heads_a, int64_t heads_b, int64_t M, int64_t N, int64_t K,
                                            void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream) {
-    return gemm_entry(a, sa5, b, sb5, fmt, true, batch, heads_a, heads_b, M, N, K, c, c_dtype, ldc, stream);
+    return gemm_entry(a, sa5, fmt_a, b, sb5, fmt_b, true, batch, heads_a, heads_b, M, N, K, c, c_dtype, ldc, stream);
 }

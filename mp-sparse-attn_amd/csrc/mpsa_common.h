@@ -19,19 +19,14 @@ int mpsa_fail(int code, const char* fmt, ...);
 
 static inline bool mpsa_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Kernels that need more dynamic LDS than the default limit get the function attribute once per device (the
-// attribute is per device); `done` is a per-kernel array of MPSA_MAX_DEVICES flags.  A race only repeats the call.
+// Kernels that need more dynamic LDS than the default limit carry a function attribute, which is per device and
+// cannot be set while a stream is being captured.  Every such kernel instantiation registers itself at library load
+// (LdsKernel<...>::registered, a static initialiser); mpsa_init() sets the attribute of all of them on the current
+// device, and the launchers call mpsa_ensure_init(), which does that on a device's first use if the caller has not.
 #define MPSA_MAX_DEVICES 64
-static inline hipError_t mpsa_reserve_lds(const void* kern, int bytes, bool* done) {
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= MPSA_MAX_DEVICES) return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (done[dev]) return hipSuccess;
-    e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e == hipSuccess) done[dev] = true;
-    return e;
-}
+bool mpsa_register_lds_kernel(const void* kern, int bytes);      // api.hip; always returns true
+int mpsa_ensure_init();                                          // api.hip; MPSA_OK or the failure of mpsa_init()
+int mpsa_seq_mean_static_resolve();                              // quantize.hip; address of the built-in partial-sum array
 
 #define MPSA_CHECK_LAUNCH(what)                                                        \
     do {                                                                               \

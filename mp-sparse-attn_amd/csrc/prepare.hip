@@ -72,7 +72,7 @@ extern "C" int mpsa_attn_prepare(const void* q, const int64_t q_strides[4], cons
                                  float pre_scale_q, const void* k_sub,
                                  uint8_t* q4, uint8_t* qs4, uint8_t* q8, uint8_t* qs8,
                                  uint8_t* k4, uint8_t* ks4, uint8_t* k8, uint8_t* ks8, void* v_tiles, mpsa_stream_t stream) {
-    if (mode == MPSA_MODE_ROUTED) mode = MPSA_MODE_DIAG;          // both operand sets, like a diag run
+    if (mode == MPSA_MODE_ROUTED || mode == MPSA_MODE_MIXED) mode = MPSA_MODE_DIAG;   // both operand sets, like a diag run
     if (mode != MPSA_MODE_MXFP4 && mode != MPSA_MODE_MXFP8 && mode != MPSA_MODE_DIAG) return mpsa_fail(MPSA_EINVAL, "prepare: unknown mode %d", mode);
     if (tile != 64 && tile != 128) return mpsa_fail(MPSA_EUNSUPPORTED, "prepare: tile must be 64 or 128 (got %d)", tile);
     if (B <= 0 || Hq <= 0 || Hkv <= 0 || Nq <= 0 || Nk <= 0 || Hq % Hkv) return mpsa_fail(MPSA_EINVAL, "prepare: bad shape (B=%lld Hq=%lld Hkv=%lld Nq=%lld Nk=%lld)", (long long)B, (long long)Hq, (long long)Hkv, (long long)Nq, (long long)Nk);

@@ -249,6 +249,11 @@ int scratch_for_current_device(float** out) {
 }
 }  // namespace
 
+int mpsa_seq_mean_static_resolve() {
+    float* p = nullptr;
+    return scratch_for_current_device(&p);
+}
+
 extern "C" int mpsa_seq_mean_static(const void* x, int x_dtype, int64_t B, int64_t H, int64_t N, int64_t D,
                                     const int64_t x_strides[4], void* mean, mpsa_stream_t stream) {
     const int64_t need = mpsa_seq_mean_workspace(B, H, N, D);

@@ -11,7 +11,7 @@ import torch
 
 BF16, F16, F32, F8E5M2 = 0, 1, 2, 3
 FMT_E4M3, FMT_E5M2, FMT_E2M1 = 0, 1, 4
-MODE_MXFP4, MODE_MXFP8, MODE_DIAG, MODE_ROUTED = 0, 1, 2, 3
+MODE_MXFP4, MODE_MXFP8, MODE_DIAG, MODE_ROUTED, MODE_MIXED = 0, 1, 2, 3, 4
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("MPSA_LIB_PATH") or os.path.join(os.path.dirname(_HERE), "lib", "libmpsa.so")
@@ -23,10 +23,12 @@ _p64 = ctypes.POINTER(ctypes.c_int64)
 SIGNATURES = {
     "mpsa_version": (_int, []),
     "mpsa_last_error": (ctypes.c_char_p, []),
+    "mpsa_init": (_int, []),
     "mpsa_e2m1_encode": (_int, [_vp, _i64, _vp, _vp]),
     "mpsa_e2m1_decode": (_int, [_vp, _i64, _vp, _vp]),
     "mpsa_e8m0_encode": (_int, [_vp, _i64, _vp, _vp]),
     "mpsa_e8m0_decode": (_int, [_vp, _i64, _vp, _vp]),
+    "mpsa_fp8_encode": (_int, [_vp, _i64, _int, _vp, _vp]),
     "mpsa_e2m1_pack": (_int, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "mpsa_e2m1_unpack": (_int, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "mpsa_scales_to_5d": (_int, [_vp, _i64, _i64, _i64, _vp, _vp]),
@@ -37,10 +39,10 @@ SIGNATURES = {
     "mpsa_seq_mean_static": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _vp, _vp]),
     "mpsa_quantize_mx_dual": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _vp, _f32, _int, _int, _int,
                                      _vp, _vp, _vp, _vp, _i64, _vp]),
-    "mpsa_gemm_mx": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
-    "mpsa_gemm_mx_batched": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
-    "mpsa_gemm_mx_packed": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
-    "mpsa_gemm_mx_batched_packed": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
+    "mpsa_gemm_mx": (_int, [_vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
+    "mpsa_gemm_mx_batched": (_int, [_vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
+    "mpsa_gemm_mx_packed": (_int, [_vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
+    "mpsa_gemm_mx_batched_packed": (_int, [_vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _int, _i64, _vp]),
     "mpsa_v_tiles": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _p64, _int, _vp, _vp]),
     "mpsa_attn_prepare": (_int, [_vp, _p64, _vp, _p64, _vp, _p64, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int,
                                  _f32, _vp] + [_vp] * 9 + [_vp]),
@@ -79,6 +81,14 @@ def lib():
             fn.restype = res
             fn.argtypes = args
         _lib = handle
+        # per-device set-up up front, so that even a caller's first launch can be captured into a HIP graph
+        # (no device here means no set-up: the entry points report their own errors)
+        if torch.cuda.is_available():
+            for dev in range(torch.cuda.device_count()):
+                with torch.cuda.device(dev):
+                    status = handle.mpsa_init()
+                if status != 0:
+                    raise MpsaError(status, handle.mpsa_last_error().decode("utf-8", "replace"))
     return _lib
 
 

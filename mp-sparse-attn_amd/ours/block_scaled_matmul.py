@@ -1,40 +1,51 @@
-"""Block-scaled matmul entry point -- the reference's ``ours/block_scaled_matmul.py`` surface.
+"""Block-scaled matmul entry points -- the reference's ``ours/block_scaled_matmul.py`` surface.
 
-``block_scaled_matmul(a, a_scale, b, b_scale, dtype_dst, M, N, K, configs)`` keeps the reference
-signature (ours/block_scaled_matmul.py:271).  Operands are what the quantizer emits: row-major codes
-(``[M, K/2]`` packed E2M1 or ``[M, K]`` 8-bit) and linear E8M0 scales ``[M, K/32]`` (the reference's 5-D packed
-scales ``[M/128, K/128, 32, 4, 4]`` are accepted too: given for both operands they go to the kernel as they are,
-which is its faster path); B is ``[N, K]``
-(NT product).  The element format is read from ``configs["ELEM_PER_BYTE_A"]`` (2 = E2M1) and, for
-8-bit, ``configs.get("FMT8", "e4m3")``.
+``block_scaled_matmul(a, a_scale, b, b_scale, dtype_dst, M, N, K, configs)`` keeps the reference signature
+(ours/block_scaled_matmul.py:271) and ``initialize_block_scaled_from_tensor(a_tensor, b_tensor, a_scale, b_scale,
+block_scale_type, compute_reference)`` the reference's operand packaging (ours/block_scaled_matmul.py:299-406).
+Operands are row-major codes (``[M, K/2]`` packed E2M1 or ``[M, K]`` 8-bit) with E8M0 scales, either linear
+``[M, K/32]`` (what the quantizer emits) or in the reference's 5-D packed form ``[M/128, K/128, 32, 4, 4]``; given
+packed for both operands they go to the kernel as they are, which is its faster path.  B is ``[N, K]`` (NT product).
+Element formats come from ``configs["ELEM_PER_BYTE_A"]`` / ``configs["ELEM_PER_BYTE_B"]`` (2 = E2M1, 1 = 8-bit; they
+may differ: the reference's ``"mixed"`` type) and, for 8-bit operands, ``configs.get("FMT8", "e4m3")``.
 """
 
 import torch
 
 from . import _lib
+from .mxfp import MXFP4Tensor, MXScaleTensor
 from .quant_mxint8 import quantize_mx
 
 VEC_SIZE = 32
 
+# block_scale_type -> (elements per byte of A, of B, 8-bit format).  As everywhere in this package "mxfp8" is E4M3;
+# the reference's own 8-bit format, E5M2 (a_tensor.to(torch.float8_e5m2), ours/block_scaled_matmul.py:334-336), is
+# spelled "mxfp8e5".  "mixed" is the reference's 8-bit A x 4-bit B.
+_TYPES = {
+    "mxfp4": (2, 2, "e4m3"), "mxfp8": (1, 1, "e4m3"), "mixed": (1, 2, "e4m3"),
+    "mxfp8e5": (1, 1, "e5m2"), "mixed_e5": (1, 2, "e5m2"),
+}
 
-def make_configs(block_scale_type="mxfp4"):
-    """The ``configs`` dict of the reference (ours/block_scaled_matmul.py:394-402) for this build's kernel."""
-    if block_scale_type not in ("mxfp4", "mxfp8", "mxfp8e5"):
+
+def make_configs(block_scale_type="mxfp4", fmt8=None):
+    """The ``configs`` dict of the reference (ours/block_scaled_matmul.py:394-402) for this build's kernels.
+    ``fmt8`` overrides the 8-bit element format (``"e4m3"`` | ``"e5m2"``)."""
+    if block_scale_type not in _TYPES:
         raise ValueError(f"Invalid block scale type: {block_scale_type}")
-    fp4 = block_scale_type == "mxfp4"
+    epb_a, epb_b, f8 = _TYPES[block_scale_type]
     return {
-        "BLOCK_SIZE_M": 256, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 128 if fp4 else 64, "num_stages": 2,
-        "ELEM_PER_BYTE_A": 2 if fp4 else 1, "ELEM_PER_BYTE_B": 2 if fp4 else 1, "VEC_SIZE": VEC_SIZE,
-        "FMT8": "e5m2" if block_scale_type == "mxfp8e5" else "e4m3",
+        "BLOCK_SIZE_M": 256, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 128 if epb_a == 2 else 64, "num_stages": 4,
+        "ELEM_PER_BYTE_A": epb_a, "ELEM_PER_BYTE_B": epb_b, "VEC_SIZE": VEC_SIZE, "FMT8": fmt8 or f8,
     }
 
 
-def _fmt_of(configs):
-    if configs["ELEM_PER_BYTE_A"] != configs["ELEM_PER_BYTE_B"]:
-        raise ValueError("mixed 8-bit x 4-bit operands are not supported")
-    if configs["ELEM_PER_BYTE_A"] == 2:
-        return _lib.FMT_E2M1
-    return _lib.FMT_E5M2 if configs.get("FMT8", "e4m3") == "e5m2" else _lib.FMT_E4M3
+def _fmts_of(configs):
+    """(fmt_a, fmt_b) of a configs dict."""
+    f8 = _lib.FMT_E4M3 if configs.get("FMT8", "e4m3") == "e4m3" else _lib.FMT_E5M2
+    pick = lambda epb: _lib.FMT_E2M1 if epb == 2 else f8
+    if configs["ELEM_PER_BYTE_A"] not in (1, 2) or configs["ELEM_PER_BYTE_B"] not in (1, 2):
+        raise ValueError("ELEM_PER_BYTE_A / ELEM_PER_BYTE_B must be 1 or 2")
+    return pick(configs["ELEM_PER_BYTE_A"]), pick(configs["ELEM_PER_BYTE_B"])
 
 
 def pack_scale_5d(scale):
@@ -70,7 +81,7 @@ def block_scaled_matmul(a, a_scale, b, b_scale, dtype_dst, M, N, K, configs):
     Reference: ours/block_scaled_matmul.py:271-296 (ValueError for an unsupported output dtype, :280)."""
     if dtype_dst not in (torch.float32, torch.float16, torch.bfloat16, torch.float8_e5m2):
         raise ValueError(f"Unsupported dtype: {dtype_dst}")
-    fmt = _fmt_of(configs)
+    fmt_a, fmt_b = _fmts_of(configs)
     _lib.require_device(a, a_scale, b, b_scale)
     # the reference's packed scale layout goes to the kernel as it is when both operands come that way
     packed = a_scale.dim() == 5 and b_scale.dim() == 5
@@ -79,12 +90,13 @@ def block_scaled_matmul(a, a_scale, b, b_scale, dtype_dst, M, N, K, configs):
             a_scale = unpack_scale_5d(a_scale)
         if b_scale.dim() == 5:
             b_scale = unpack_scale_5d(b_scale)
-    width = K // 2 if fmt == _lib.FMT_E2M1 else K
+    width_a = K // 2 if fmt_a == _lib.FMT_E2M1 else K
+    width_b = K // 2 if fmt_b == _lib.FMT_E2M1 else K
     a = a.view(torch.uint8).contiguous()
     b = b.view(torch.uint8).contiguous()
     a_scale = a_scale.contiguous()
     b_scale = b_scale.contiguous()
-    assert a.shape == (M, width) and b.shape == (N, width), "operand shapes do not match M, N, K"
+    assert a.shape == (M, width_a) and b.shape == (N, width_b), "operand shapes do not match M, N, K"
     if packed:
         assert a_scale.shape == (M // 128, K // 128, 32, 4, 4) and b_scale.shape == (N // 128, K // 128, 32, 4, 4), \
             "packed scales must be [rows/128, K/128, 32, 4, 4]"
@@ -93,22 +105,83 @@ def block_scaled_matmul(a, a_scale, b, b_scale, dtype_dst, M, N, K, configs):
     out = torch.empty((M, N), dtype=dtype_dst, device=a.device)
     entry = _lib.lib().mpsa_gemm_mx_packed if packed else _lib.lib().mpsa_gemm_mx
     with torch.cuda.device(a.device):
-        _lib.check(entry(_lib.ptr(a), _lib.ptr(a_scale), _lib.ptr(b), _lib.ptr(b_scale), fmt,
+        _lib.check(entry(_lib.ptr(a), _lib.ptr(a_scale), fmt_a, _lib.ptr(b), _lib.ptr(b_scale), fmt_b,
                          M, N, K, _lib.ptr(out), _lib.dtype_id(dtype_dst), N, _lib.stream_ptr(a.device)))
     return out
 
 
-def initialize_block_scaled_from_tensor(a_tensor, b_tensor, block_scale_type="mxfp4", packed_scales=False):
-    """Quantize bf16/fp16 ``A [M,K]`` and ``B [N,K]`` per 32 along K and package them for
-    :func:`block_scaled_matmul`: returns ``(a, a_scale, b, b_scale, configs)``.
+def fp8_cast(x, fmt8):
+    """Elementwise float -> FP8 byte (``x.to(torch.float8_e5m2)`` / ``float8_e4m3fn``) through ``mpsa_fp8_encode``."""
+    _lib.require_device(x)
+    x = x.to(torch.float32).contiguous()
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().mpsa_fp8_encode(_lib.ptr(x), x.numel(), fmt8, _lib.ptr(out), _lib.stream_ptr(x.device)))
+    return out
 
-    Counterpart of the reference's operand packaging (ours/block_scaled_matmul.py:299-406) chained after
-    the quantizer as in test_quant.py:296-350; scales stay in the linear ``[rows, K/32]`` layout unless
-    ``packed_scales`` asks for the reference's packed one."""
+
+def _package_operand(t, four_bit, fmt8):
+    """One operand of the reference's packaging: 8-bit -> the elementwise FP8 cast (ours/block_scaled_matmul.py:334-336);
+    4-bit -> ``MXFP4Tensor`` codes packed two per byte along K (:338-345; uint8 input is taken as ready-made codes, one
+    per byte, which is what the reference's constructor call accepts; float input is encoded first)."""
+    if not four_bit:
+        if t.dtype in (torch.float8_e5m2, torch.float8_e4m3fn, torch.uint8):
+            return t.view(torch.uint8)
+        return fp8_cast(t, fmt8)
+    codes = MXFP4Tensor(data=t, dtype=torch.uint8) if t.dtype == torch.uint8 else MXFP4Tensor(data=t.to(torch.float32))
+    return codes.to_packed_tensor(dim=t.dim() - 1)
+
+
+def _package_scale(s):
+    """Float scale factors -> E8M0 bytes through ``MXScaleTensor`` (ours/block_scaled_matmul.py:370-374); uint8 input
+    is taken as ready-made E8M0 bytes (ours/mxfp_attn_kernel.py:505-506)."""
+    if s.dtype == torch.uint8:
+        return s
+    return MXScaleTensor(s.to(torch.float32)).data
+
+
+def initialize_block_scaled_from_tensor(a_tensor, b_tensor, a_scale, b_scale, block_scale_type="mxfp4", compute_reference=False):
+    """Operand packaging with the reference's signature (ours/block_scaled_matmul.py:299-406).
+
+    ``a_tensor [M,K]``, ``b_tensor [N,K]``: values to cast element by element (no block scale is derived from them);
+    ``a_scale``, ``b_scale``: caller-supplied scale factors in the packed ``[rows/128, K/128, 32, 4, 4]`` layout, float
+    (encoded to E8M0 with ``MXScaleTensor``) or uint8.  ``block_scale_type``: ``"mxfp4"``, ``"mxfp8"`` (E4M3),
+    ``"mixed"`` (8-bit A x 4-bit B), ``"mxfp8e5"`` / ``"mixed_e5"`` (E5M2, the reference's cast).  ``"nvfp4"`` (16-element
+    blocks with FP8 scales) has no counterpart on the CDNA4 scaled matrix cores and raises.
+    Returns ``(a, a_scale, b, b_scale, configs, None)``; ``compute_reference=True`` raises -- the library carries no
+    second implementation to compare with."""
+    if block_scale_type == "nvfp4":
+        raise NotImplementedError("nvfp4 (16-element blocks, FP8 scale factors) is not available: the gfx950 scaled matrix "
+                                  "instructions take one E8M0 scale per 32 elements")
+    assert block_scale_type in _TYPES, f"Invalid block scale type: {block_scale_type}"
+    if compute_reference:
+        raise NotImplementedError("compute_reference is not available: use the test-suite's CPU oracle")
+    M, K = a_tensor.shape
+    N, K_b = b_tensor.shape
+    assert K == K_b, f"matrix dimensions do not match: A.shape[1]={K} != B.shape[1]={K_b}"
+    expected_a = (M // 128, K // VEC_SIZE // 4, 32, 4, 4)
+    expected_b = (N // 128, K // VEC_SIZE // 4, 32, 4, 4)
+    assert tuple(a_scale.shape) == expected_a, f"a_scale shape mismatch: expected {expected_a}, got {tuple(a_scale.shape)}"
+    assert tuple(b_scale.shape) == expected_b, f"b_scale shape mismatch: expected {expected_b}, got {tuple(b_scale.shape)}"
     configs = make_configs(block_scale_type)
-    fmt = _fmt_of(configs)
+    fmt_a, fmt_b = _fmts_of(configs)
+    f8 = fmt_a if fmt_a != _lib.FMT_E2M1 else _lib.FMT_E4M3
+    a = _package_operand(a_tensor, fmt_a == _lib.FMT_E2M1, f8)
+    b = _package_operand(b_tensor, fmt_b == _lib.FMT_E2M1, f8)
+    return a, _package_scale(a_scale), b, _package_scale(b_scale), configs, None
+
+
+def quantize_block_scaled_from_tensor(a_tensor, b_tensor, block_scale_type="mxfp4", packed_scales=False):
+    """MX-quantize bf16/fp16 ``A [M,K]`` and ``B [N,K]`` per 32 along K (scales derived from the data, as the attention
+    path does) and package them for :func:`block_scaled_matmul`: returns ``(a, a_scale, b, b_scale, configs)``.
+    ``block_scale_type``: ``"mxfp4"``, ``"mxfp8"`` (E4M3), ``"mxfp8e5"`` (E5M2).
+    Scales stay in the linear ``[rows, K/32]`` layout unless ``packed_scales`` asks for the reference's packed one."""
+    if block_scale_type not in ("mxfp4", "mxfp8", "mxfp8e5"):
+        raise ValueError(f"Invalid block scale type: {block_scale_type}")
+    configs = make_configs(block_scale_type)
+    fmt, _ = _fmts_of(configs)
     a, sa = quantize_mx(a_tensor[None, None], 1.0, fmt)
     b, sb = quantize_mx(b_tensor[None, None], 1.0, fmt)
-    if packed_scales:                            # the reference packs them at this point (ours/block_scaled_matmul.py:299-406)
+    if packed_scales:
         return a[0, 0], pack_scale_5d(sa[0, 0]), b[0, 0], pack_scale_5d(sb[0, 0]), configs
     return a[0, 0], sa[0, 0], b[0, 0], sb[0, 0], configs

@@ -13,13 +13,15 @@ from . import _lib
 from .quant_mxint8 import seq_mean, pre_scale_q, _as_bhnd, _check_input
 
 _MODES = {"mxfp4": _lib.MODE_MXFP4, "mxfp8": _lib.MODE_MXFP8, "mxfp8e5": _lib.MODE_MXFP8, "diag": _lib.MODE_DIAG,
-          "diag_e5": _lib.MODE_DIAG, "routed": _lib.MODE_ROUTED, "routed_e5": _lib.MODE_ROUTED}
+          "diag_e5": _lib.MODE_DIAG, "routed": _lib.MODE_ROUTED, "routed_e5": _lib.MODE_ROUTED,
+          "mixed": _lib.MODE_MIXED, "mixed_e5": _lib.MODE_MIXED}
 
 
-def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False):
+def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False, reuse=None):
     """Quantize Q/K (K minus its mean over the sequence if ``smooth_k``) and repack V for one attention call.
     q ``[B,Hq,Nq,D]``, k/v ``[B,Hkv,Nk,D]`` of one 16-bit dtype.  Returns a dict of device tensors (rows padded to
-    whole tiles) the launcher consumes."""
+    whole tiles) the launcher consumes.  ``reuse``: the dict a previous call returned for the same shapes, dtype, tile
+    and type -- its buffers are written again instead of allocating new ones (a serving loop's steady state)."""
     if block_scale_type not in _MODES:
         raise ValueError(f"Invalid block scale type: {block_scale_type}")
     mode = _MODES[block_scale_type]
@@ -30,21 +32,26 @@ def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False
     n_pad = nt * tile
     nq_pad = (Nq + tile - 1) // tile * tile
     pre = pre_scale_q(D, scale)
-    ops = {"mode": mode, "fmt8": fmt8, "tile": tile, "n": N, "q4": None, "qs4": None, "q8": None, "qs8": None,
-           "k4": None, "ks4": None, "k8": None, "ks8": None}
+    key = (mode, fmt8, tile, tuple(q.shape), tuple(k.shape), q.dtype, v.dtype, q.device)
     # smooth-K (ours/mxfp_attn_kernel.py:33-34): the mean over the sequence is subtracted inside the K quantizer
     kmean = seq_mean(k) if smooth_k else None
     q, k = _check_input(q), _check_input(k)
     dev = q.device
-    need4, need8 = mode != _lib.MODE_MXFP8, mode != _lib.MODE_MXFP4
-    u8 = lambda *shape: torch.empty(shape, dtype=torch.uint8, device=dev)
-    if need4:
-        ops["q4"], ops["qs4"] = u8(B, Hq, nq_pad, D // 2), u8(B, Hq, nq_pad, D // 32)
-        ops["k4"], ops["ks4"] = u8(B, Hkv, n_pad, D // 2), u8(B, Hkv, n_pad, D // 32)
-    if need8:
-        ops["q8"], ops["qs8"] = u8(B, Hq, nq_pad, D), u8(B, Hq, nq_pad, D // 32)
-        ops["k8"], ops["ks8"] = u8(B, Hkv, n_pad, D), u8(B, Hkv, n_pad, D // 32)
-    v_tiles = torch.empty((B, Hkv, nt, tile * D), dtype=v.dtype, device=v.device)
+    if reuse is not None and reuse.get("key") == key:
+        ops = reuse
+        v_tiles = ops["v_tiles"]
+    else:
+        ops = {"mode": mode, "fmt8": fmt8, "tile": tile, "n": N, "q4": None, "qs4": None, "q8": None, "qs8": None,
+               "k4": None, "ks4": None, "k8": None, "ks8": None, "key": key}
+        need4, need8 = mode != _lib.MODE_MXFP8, mode != _lib.MODE_MXFP4
+        u8 = lambda *shape: torch.empty(shape, dtype=torch.uint8, device=dev)
+        if need4:
+            ops["q4"], ops["qs4"] = u8(B, Hq, nq_pad, D // 2), u8(B, Hq, nq_pad, D // 32)
+            ops["k4"], ops["ks4"] = u8(B, Hkv, n_pad, D // 2), u8(B, Hkv, n_pad, D // 32)
+        if need8:
+            ops["q8"], ops["qs8"] = u8(B, Hq, nq_pad, D), u8(B, Hq, nq_pad, D // 32)
+            ops["k8"], ops["ks8"] = u8(B, Hkv, n_pad, D), u8(B, Hkv, n_pad, D // 32)
+        v_tiles = torch.empty((B, Hkv, nt, tile * D), dtype=v.dtype, device=v.device)
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().mpsa_attn_prepare(
             _lib.ptr(q), _lib.strides4(q), _lib.ptr(k), _lib.strides4(k), _lib.ptr(v), _lib.strides4(v),
@@ -114,6 +121,96 @@ def attention_from_operands(ops, out, is_causal, skip_thresh=None, skipped=None,
             _lib.ptr(ops["v_tiles"]), _lib.dtype_id(ops["v_tiles"].dtype), _lib.ptr(out), _lib.dtype_id(out.dtype),
             _lib.strides4(out), B, Hq, Hkv, Nq, N, D, ops["tile"], 1 if is_causal else 0, ops["mode"],
             _lib.stream_ptr(dev)))
+    return out
+
+
+def initialize_block_scaled_batched_from_tensor(a_tensor, b_tensor, a_scale, b_scale, block_scale_type="mxfp4", compute_reference=False):
+    """Operand packaging of the fused attention with the reference's signature (ours/mxfp_attn_kernel.py:426-553).
+
+    ``a_tensor [B,H,M,K]`` (Q) and ``b_tensor [B,Hkv,N,K]`` (K): uint8 codes as the quantizer leaves them (one E2M1
+    code per byte, or FP8 bytes) or float values, which are cast element by element; ``a_scale`` / ``b_scale``:
+    ``[B,H,rows/128,K/128,32,4,4]`` scale factors, uint8 E8M0 bytes (taken as they are, :505-506) or float (encoded
+    with ``MXScaleTensor``).  4-bit codes are packed two per byte along K (the last dim).  Returns
+    ``(a, a_scale, b, b_scale, configs, (None, None, None))``; ``compute_reference=True`` raises."""
+    from .block_scaled_matmul import _TYPES, _fmts_of, _package_operand, _package_scale, make_configs, VEC_SIZE
+    if block_scale_type == "nvfp4":
+        raise NotImplementedError("nvfp4 (16-element blocks, FP8 scale factors) is not available: the gfx950 scaled matrix "
+                                  "instructions take one E8M0 scale per 32 elements")
+    assert block_scale_type in _TYPES, f"Invalid block scale type: {block_scale_type}"
+    if compute_reference:
+        raise NotImplementedError("compute_reference is not available: use the test-suite's CPU oracle")
+    B, H, M, K = a_tensor.shape
+    B_b, H_b, N, K_b = b_tensor.shape
+    assert B == B_b, f"batch sizes do not match: A.shape[0]={B} != B.shape[0]={B_b}"
+    assert H % H_b == 0, f"head counts do not match: A.shape[1]={H}, B.shape[1]={H_b}"
+    assert K == K_b, f"matrix dimensions do not match: A.shape[3]={K} != B.shape[3]={K_b}"
+    expected_a = (B, H, M // 128, K // VEC_SIZE // 4, 32, 4, 4)
+    expected_b = (B, H_b, N // 128, K // VEC_SIZE // 4, 32, 4, 4)
+    assert tuple(a_scale.shape) == expected_a, f"a_scale shape mismatch: expected {expected_a}, got {tuple(a_scale.shape)}"
+    assert tuple(b_scale.shape) == expected_b, f"b_scale shape mismatch: expected {expected_b}, got {tuple(b_scale.shape)}"
+    configs = make_configs(block_scale_type)
+    configs["BLOCK_SIZE_M"] = configs["BLOCK_SIZE_N"] = 128
+    fmt_a, fmt_b = _fmts_of(configs)
+    f8 = fmt_a if fmt_a != _lib.FMT_E2M1 else _lib.FMT_E4M3
+    a = _package_operand(a_tensor, fmt_a == _lib.FMT_E2M1, f8)
+    b = _package_operand(b_tensor, fmt_b == _lib.FMT_E2M1, f8)
+    return a, _package_scale(a_scale), b, _package_scale(b_scale), configs, (None, None, None)
+
+
+def block_scaled_batched_attn(a_desc, a_scale, b_desc, b_scale, v_ori, dtype_dst, B, H, M, N, K, configs, STAGE=1, skip_thresh=None):
+    """Fused attention on packaged operands -- the reference's launcher (ours/mxfp_attn_kernel.py:362-423).
+
+    ``a_desc`` / ``b_desc``: Q ``[B,H,M,K']`` and K ``[B,Hkv,N,K']`` codes (``K' = K/2`` packed E2M1 or ``K`` FP8 bytes)
+    with ``sm_scale*log2(e)`` already folded into Q; ``a_scale`` / ``b_scale``: E8M0 bytes, packed
+    ``[B,H,rows/128,K/128,32,4,4]`` or linear ``[B,H,rows,K/32]``; ``v_ori [B,Hkv,N,K]`` bf16/fp16.  The precision comes
+    from ``configs`` (``ELEM_PER_BYTE_A`` / ``_B``: 2,2 = mxfp4; 1,1 = mxfp8; 1,2 = mixed).  ``STAGE``: 1 = every key
+    tile (what the reference's kernel does), 3 = causal.  Returns ``[B,H,M,K]`` of ``dtype_dst``."""
+    from .block_scaled_matmul import _fmts_of, unpack_scale_5d
+    if dtype_dst not in (torch.float32, torch.float16, torch.bfloat16):
+        raise ValueError(f"Unsupported dtype: {dtype_dst}")            # ours/mxfp_attn_kernel.py:389
+    if STAGE not in (1, 3):
+        raise ValueError(f"STAGE must be 1 (all key tiles) or 3 (causal), got {STAGE}")
+    _lib.require_device(a_desc, a_scale, b_desc, b_scale, v_ori)
+    fmt_a, fmt_b = _fmts_of(configs)
+    if fmt_a == _lib.FMT_E2M1 and fmt_b != _lib.FMT_E2M1:
+        raise ValueError("a 4-bit Q with an 8-bit K is not a type of the reference (mixed is 8-bit Q x 4-bit K)")
+    mode = _lib.MODE_MXFP4 if fmt_a == _lib.FMT_E2M1 else (_lib.MODE_MXFP8 if fmt_b != _lib.FMT_E2M1 else _lib.MODE_MIXED)
+    fmt8 = fmt_a if fmt_a != _lib.FMT_E2M1 else _lib.FMT_E4M3
+    Hkv = b_desc.shape[1]
+    tile = 128
+    assert M % tile == 0 and N % tile == 0, "M and N must be multiples of 128 (the packaged scale layout's chunk)"
+    assert K in [64, 128], "headdim should be in [64, 128]."
+    a_desc, b_desc = a_desc.view(torch.uint8).contiguous(), b_desc.view(torch.uint8).contiguous()
+    if a_scale.dim() == 7:
+        a_scale = unpack_scale_5d(a_scale)
+    if b_scale.dim() == 7:
+        b_scale = unpack_scale_5d(b_scale)
+    a_scale, b_scale = a_scale.contiguous(), b_scale.contiguous()
+    wa = K // 2 if fmt_a == _lib.FMT_E2M1 else K
+    wb = K // 2 if fmt_b == _lib.FMT_E2M1 else K
+    assert a_desc.shape == (B, H, M, wa) and b_desc.shape == (B, Hkv, N, wb), "operand shapes do not match B, H, M, N, K"
+    assert a_scale.shape == (B, H, M, K // 32) and b_scale.shape == (B, Hkv, N, K // 32), "scale shapes do not match"
+    assert v_ori.shape == (B, Hkv, N, K) and v_ori.dtype in (torch.float16, torch.bfloat16), "v must be [B,Hkv,N,K] bf16/fp16"
+    if v_ori.stride(-1) != 1:
+        v_ori = v_ori.contiguous()
+    dev = a_desc.device
+    v_tiles = torch.empty((B, Hkv, N // tile, tile * K), dtype=v_ori.dtype, device=dev)
+    out = torch.empty((B, H, M, K), dtype=dtype_dst, device=dev)
+    q4 = a_desc if fmt_a == _lib.FMT_E2M1 else None
+    q8 = a_desc if fmt_a != _lib.FMT_E2M1 else None
+    k4 = b_desc if fmt_b == _lib.FMT_E2M1 else None
+    k8 = b_desc if fmt_b != _lib.FMT_E2M1 else None
+    common = (_lib.ptr(q4), _lib.ptr(a_scale if q4 is not None else None), _lib.ptr(q8), _lib.ptr(a_scale if q8 is not None else None),
+              _lib.ptr(k4), _lib.ptr(b_scale if k4 is not None else None), _lib.ptr(k8), _lib.ptr(b_scale if k8 is not None else None), fmt8,
+              _lib.ptr(v_tiles), _lib.dtype_id(v_ori.dtype), _lib.ptr(out), _lib.dtype_id(dtype_dst), _lib.strides4(out),
+              B, H, Hkv, M, N, K, tile, 1 if STAGE == 3 else 0, mode)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mpsa_v_tiles(_lib.ptr(v_ori), _lib.dtype_id(v_ori.dtype), B, Hkv, N, K, _lib.strides4(v_ori), tile,
+                                           _lib.ptr(v_tiles), _lib.stream_ptr(dev)))
+        if skip_thresh is not None:
+            _lib.check(_lib.lib().mpsa_attn_fwd_skip(*common, float(skip_thresh), None, _lib.stream_ptr(dev)))
+        else:
+            _lib.check(_lib.lib().mpsa_attn_fwd(*common, _lib.stream_ptr(dev)))
     return out
 
 

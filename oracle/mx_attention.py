@@ -17,7 +17,7 @@ import torch.nn.functional as Fnn
 
 from .mx_quantize import FMT_E2M1, FMT_E4M3, quantize_mx, dequantize_mx, q_pre_scale, smooth_k as _smooth_k
 
-MODES = ("mxfp4", "mxfp8", "diag", "routed")
+MODES = ("mxfp4", "mxfp8", "diag", "routed", "mixed")
 
 
 def _tile_is_8bit(mode: str, i: int, j: int, route=None) -> bool:
@@ -32,6 +32,15 @@ def _tile_is_8bit(mode: str, i: int, j: int, route=None) -> bool:
     raise ValueError(f"unknown block_scale_type {mode}")
 
 
+def _tile_tags(mode: str, i: int, j: int, route=None):
+    """(precision of the Q operand, of the K operand) for tile (i, j).  ``"mixed"`` is the reference's 8-bit Q against
+    4-bit K on every tile (ELEM_PER_BYTE_A = 1, ELEM_PER_BYTE_B = 2: ours/mxfp_attn_kernel.py:264-269, :448-449)."""
+    if mode == "mixed":
+        return "8", "4"
+    tag = "8" if _tile_is_8bit(mode, i, j, route) else "4"
+    return tag, tag
+
+
 def _prepare(q, k, mode, scale, fmt8):
     """Quantize + dequantize Q and K in the formats the mode needs (float32 fake-quant)."""
     D = q.shape[-1]
@@ -39,9 +48,11 @@ def _prepare(q, k, mode, scale, fmt8):
     ops = {}
     if mode in ("mxfp4", "diag", "routed"):
         ops["q4"] = dequantize_mx(*quantize_mx(q, pre, FMT_E2M1), FMT_E2M1)
+    if mode in ("mxfp4", "diag", "routed", "mixed"):
         ops["k4"] = dequantize_mx(*quantize_mx(k, 1.0, FMT_E2M1), FMT_E2M1)
-    if mode in ("mxfp8", "diag", "routed"):
+    if mode in ("mxfp8", "diag", "routed", "mixed"):
         ops["q8"] = dequantize_mx(*quantize_mx(q, pre, fmt8), fmt8)
+    if mode in ("mxfp8", "diag", "routed"):
         ops["k8"] = dequantize_mx(*quantize_mx(k, 1.0, fmt8), fmt8)
     return ops
 
@@ -103,9 +114,9 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
                     c0, c1 = j * tile, min((j + 1) * tile, Nk)
                     if mode == "routed" and int(route[b, h, i, j]) not in (1, 2):
                         continue
-                    tag = "8" if _tile_is_8bit(mode, i, j, None if route is None else route[b, h]) else "4"
-                    qt = ops["q" + tag][b, hi_, r0:r1]
-                    kt = ops["k" + tag][b, kvh, c0:c1]
+                    qtag, ktag = _tile_tags(mode, i, j, None if route is None else route[b, h])
+                    qt = ops["q" + qtag][b, hi_, r0:r1]
+                    kt = ops["k" + ktag][b, kvh, c0:c1]
                     s = qt @ kt.T                                    # float32, already in log2 units
                     if causal and j == i:
                         rr = torch.arange(r0, r1).unsqueeze(1)
@@ -159,10 +170,10 @@ def attn_dense_f64(q, k, v, tile=128, causal=True, mode="diag", scale=None, smoo
                 for j in range((i if causal else nt - 1) + 1):
                     if mode == "routed" and int(route[b, h, i, j]) not in (1, 2):
                         continue                                     # skipped: the tile's scores stay -inf
-                    tag = "8" if _tile_is_8bit(mode, i, j, None if route is None else route[b, h]) else "4"
+                    qtag, ktag = _tile_tags(mode, i, j, None if route is None else route[b, h])
                     r = slice(i * tile, min((i + 1) * tile, N))
                     c = slice(j * tile, min((j + 1) * tile, N))
-                    s[r, c] = ops["q" + tag][b, hi_, r] @ ops["k" + tag][b, kvh, c].T
+                    s[r, c] = ops["q" + qtag][b, hi_, r] @ ops["k" + ktag][b, kvh, c].T
             if causal:
                 s = s.masked_fill(torch.ones(N, N, dtype=torch.bool).triu(1), float("-inf"))
             p = torch.exp2(s - s.amax(dim=1, keepdim=True))

@@ -44,8 +44,13 @@ def test_host_side_argument_validation():
     assert L.mpsa_seq_mean_workspace(2, 3, 1000, 64) == 2 * 3 * 4 * 64 * 4
     assert L.mpsa_seq_mean(one, 0, 1, 1, 8, 64, st_ok, null, one, null) == -1                      # no workspace
     assert L.mpsa_seq_mean(one, 0, 1, 1, 8, 96, st_ok, one, one, null) == -3                       # D = 96
-    assert L.mpsa_gemm_mx(one, one, one, one, 4, 100, 256, 128, one, 0, 256, null) == -3           # M % 256
-    assert L.mpsa_gemm_mx(one, one, one, one, 4, 256, 256, 128, one, 7, 256, null) == -1           # bad dtype
+    assert L.mpsa_gemm_mx(one, one, 4, one, one, 4, 100, 256, 96, one, 0, 256, null) == -3         # K % 64
+    assert L.mpsa_gemm_mx(one, one, 4, one, one, 4, 256, 256, 128, one, 7, 256, null) == -1        # bad dtype
+    assert L.mpsa_gemm_mx(one, one, 4, one, one, 3, 256, 256, 128, one, 0, 256, null) == -1        # bad format of B
+    assert L.mpsa_gemm_mx_packed(one, one, 4, one, one, 4, 100, 256, 128, one, 0, 256, null) == -3  # packed: M % 128
+    assert L.mpsa_fp8_encode(null, 4, 0, one, null) == -1
+    assert L.mpsa_fp8_encode(one, 4, 4, one, null) == -1                                           # E2M1 is not an FP8 format
+    assert L.mpsa_seq_mean_static(one, 0, 1, 64, 262144, 128, st_ok, one, null) == -3              # beyond the built-in array
     assert L.mpsa_v_tiles(one, 0, 1, 1, 128, 96, st_ok, 128, one, null) == -3                      # D = 96
     so = (ctypes.c_int64 * 4)(128 * 128, 128 * 128, 128, 1)
     args = [one] * 8 + [0, one, 0, one, 0, so, 1, 4, 3, 128, 128, 128, 128, 1, 2, null]
@@ -84,6 +89,7 @@ def test_python_entry_points_refuse_cpu_tensors_and_bad_arguments():
         block_scaled_matmul(x, x, x, x, torch.int8, 256, 256, 128, make_configs("mxfp4"))
     with pytest.raises(ValueError, match="Invalid block scale type"):
         make_configs("nvfp4")
+    assert make_configs("mixed")["ELEM_PER_BYTE_A"] == 1 and make_configs("mixed")["ELEM_PER_BYTE_B"] == 2
     t = MXFP4Tensor(data=torch.arange(16, dtype=torch.uint8).reshape(2, 8), dtype=torch.uint8)
     with pytest.raises(RuntimeError, match="no CPU"):
         t.to_packed_tensor(dim=1)

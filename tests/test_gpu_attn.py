@@ -24,6 +24,20 @@ def _compare(got, want, what=""):
     return m
 
 
+def _compare_16bit(got16, got32, want32, what=""):
+    """A 16-bit output against the oracle.  The 2e-2 bar is a bar on the arithmetic, checked on the float32 outputs;
+    rounding an output of magnitude 4 or more to bf16 can by itself move it by 2^-5 = 0.031 when the two float32
+    values straddle a rounding boundary, so the 16-bit output is checked as what it is: the kernel's own float32
+    result rounded once (bit for bit), hence within the bar plus half a 16-bit unit of the oracle."""
+    m = _compare(got32, want32, what + " (float32 outputs)")
+    assert torch.equal(got16.cpu(), got32.cpu().to(got16.dtype)), f"{what}: the 16-bit output is not the rounded float32 output"
+    w = want32.double()
+    half_ulp = torch.exp2(torch.floor(torch.log2(w.abs().clamp_min(1e-30))) - (8 if got16.dtype == torch.bfloat16 else 11))
+    err = (got16.cpu().double() - w).abs()
+    assert (err <= MAXABS_MAX + half_ulp).all(), f"{what}: 16-bit output off by {(err - half_ulp).max().item():.4f} beyond rounding"
+    return m
+
+
 def _run(q, k, v, **kw):
     return mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), **kw)
 
@@ -92,16 +106,19 @@ def test_running_maximum_moves(shape, causal, N, tile, pv):
         _compare(got, want, f"{shape} {mode} causal={causal} N={N} tile={tile} {pv}")
 
 
-def test_c3_llama_shape_one_kv_group_with_outliers():
-    """B=1 Hq=32 Hkv=8 N=8192 D=128 causal, outlier channels, 128x128 tiles: the full problem runs on the GPU,
-    the oracle checks query heads 4..7 (KV head 1) and head 31."""
+def test_c3_llama_shape_all_heads_with_outliers():
+    """B=1 Hq=32 Hkv=8 N=8192 D=128 causal, outlier channels, 128x128 tiles: the full problem on the GPU and in the
+    oracle, all 32 query heads.  The bar is checked on float32 outputs (see _compare_16bit for why the bf16 output is
+    checked as the rounding of that)."""
     q, k, v = make_qkv(1, 32, 8, 8192, 128, seed=2, outliers=True)
-    got = _run(q, k, v, is_causal=True, block_scale_type="diag", tile=128, output_dtype=torch.bfloat16)
-    heads = [4, 5, 6, 7, 31]
-    want = O.attn_mx(q, k, v, tile=128, causal=True, mode="diag", heads=heads)
-    m = _compare(got[:, heads], want, "C3 heads")
-    assert m["cos"] > 0.99999 and m["max_abs"] < 1.6e-2, m          # well inside the bar on this workload
-    assert torch.isfinite(got.float()).all()
+    got16 = _run(q, k, v, is_causal=True, block_scale_type="diag", tile=128, output_dtype=torch.bfloat16)
+    got32 = _run(q, k, v, is_causal=True, block_scale_type="diag", tile=128, output_dtype=torch.float32)
+    want = O.attn_mx(q, k, v, tile=128, causal=True, mode="diag", out_dtype=torch.float32)
+    m = _compare_16bit(got16, got32, want, "C3 all heads")
+    assert m["cos"] > 0.99999, m                                      # well inside the bar on this workload
+    assert torch.isfinite(got16.float()).all()
+    for h in range(32):                                               # and head by head, not only in aggregate
+        _compare(got32[:, h], want[:, h], f"C3 head {h}")
 
 
 def test_full_size_properties():
@@ -131,12 +148,7 @@ def test_step_under_hip_graph_capture_replays_like_eager():
     def step():
         attention_from_operands(prepare_operands(q, k, v, 128, "diag", smooth_k=True), out, True)
 
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        for _ in range(2):                       # first calls set kernel attributes: not inside a capture
-            step()
-    torch.cuda.current_stream().wait_stream(side)
+    # no warm-up call: loading the library set every kernel's attributes (mpsa_init), so a first call can be captured
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
@@ -155,23 +167,31 @@ def test_step_under_hip_graph_capture_replays_like_eager():
         assert torch.equal(replayed, eager), f"replay {r}"
 
 
-def test_long_context_properties():
-    """N = 131072 (B=1, Hq=4, Hkv=1 of the long-context shape: the kernel's work per head is the full one): V = 1
-    gives 1 everywhere, the first causal row returns V[0], and the last query tile (1024 key tiles deep) agrees with
-    the oracle run on that tile alone."""
+def test_c4_long_context_full_shape():
+    """B=1 Hq=32 Hkv=8 N=131072 D=128 causal with the outlier-channel scheme (seed 3), 128x128 tiles, diag: the whole
+    problem runs on the GPU (16384 workgroups of the paired-tile kernel, 1024 key tiles deep).  The oracle checks
+    sampled (head, query tile) pairs: four KV groups, both tiles of a pair (even and odd), the first, middle and last
+    tiles.  Size-independent properties on the full output: V = 1 gives 1, the first causal row returns V[0]."""
     N = 131072
-    g = torch.Generator(device=DEV).manual_seed(3)
-    q = torch.randn(1, 4, N, 128, generator=g, device=DEV).bfloat16()
-    k = torch.randn(1, 1, N, 128, generator=g, device=DEV).bfloat16()
-    v = torch.randn(1, 1, N, 128, generator=g, device=DEV).bfloat16()
-    o1 = mxfp_attn_kernel(q, k, torch.ones_like(v), is_causal=True, block_scale_type="diag", output_dtype=torch.float32)
-    assert (o1 - 1).abs().max().item() < 8e-3
-    del o1
-    o = mxfp_attn_kernel(q, k, v, is_causal=True, block_scale_type="diag", output_dtype=torch.bfloat16)
-    assert torch.equal(o[:, :, 0], v[:, :, 0].expand(1, 4, 128))
-    assert torch.isfinite(o.float()).all()
-    want = O.attn_mx(q[:, :1].cpu(), k.cpu(), v.cpu(), tile=128, causal=True, mode="diag", q_tiles=[N // 128 - 1])
-    _compare(o[:, :1, -128:], want, "last query tile of N=131072")
+    q, k, v = make_qkv(1, 32, 8, N, 128, seed=3, outliers=True)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    o = mxfp_attn_kernel(qd, kd, vd, is_causal=True, block_scale_type="diag", output_dtype=torch.float32)
+    assert torch.isfinite(o).all()
+    assert torch.equal(o[:, :, 0].cpu(), v[:, :, 0].repeat_interleave(4, dim=1).float())
+    samples = {0: [0, 1, 1023], 13: [511, 512], 22: [1022], 31: [2, 1023]}
+    for h, tiles in samples.items():
+        kvh = h // 4
+        want = O.attn_mx(q[:, h:h + 1], k[:, kvh:kvh + 1], v[:, kvh:kvh + 1], tile=128, causal=True, mode="diag", q_tiles=tiles,
+                         out_dtype=torch.float32)
+        got = torch.cat([o[:, h:h + 1, t * 128:(t + 1) * 128] for t in tiles], dim=2)
+        _compare(got, want, f"C4 head {h} tiles {tiles}")
+        for n, t in enumerate(tiles):
+            _compare(got[:, :, n * 128:(n + 1) * 128], want[:, :, n * 128:(n + 1) * 128], f"C4 head {h} tile {t}")
+    o16 = mxfp_attn_kernel(qd, kd, vd, is_causal=True, block_scale_type="diag", output_dtype=torch.bfloat16)
+    assert torch.equal(o16, o.to(torch.bfloat16))                     # the bf16 output is the float32 one, rounded once
+    del o, o16
+    o1 = mxfp_attn_kernel(qd, kd, torch.ones_like(vd), is_causal=True, block_scale_type="diag", output_dtype=torch.bfloat16)
+    assert (o1.float() - 1).abs().max().item() < 8e-3
 
 
 @pytest.mark.parametrize("causal", [False, True])
@@ -367,3 +387,58 @@ def test_error_behaviour():
         mxfp_attn(q, k, v, skip_thresh=0.5, block_scale_type="diag")
     with pytest.raises(AssertionError, match="multiple of key/value heads"):
         mxfp_attn(q[:, :3], k, v)
+
+
+@pytest.mark.parametrize("fmt8", ["mixed", "mixed_e5"])
+@pytest.mark.parametrize("causal,N,D,tile", [(True, 512, 128, 128), (False, 300, 128, 128), (True, 384, 64, 64), (False, 256, 64, 128)])
+def test_mixed_mode_8bit_q_against_4bit_k(fmt8, causal, N, D, tile):
+    """The reference's "mixed" type (ours/mxfp_attn_kernel.py:264-269 with ELEM_PER_BYTE_A = 1, ELEM_PER_BYTE_B = 2):
+    every tile multiplies 8-bit Q codes with 4-bit K codes."""
+    q, k, v = make_qkv(1, 4, 2, N, D, seed=500 + N + D)
+    got = _run(q, k, v, is_causal=causal, block_scale_type=fmt8, tile=tile, output_dtype=torch.float32)
+    f8 = O.FMT_E5M2 if fmt8.endswith("e5") else O.FMT_E4M3
+    want = O.attn_mx(q, k, v, tile=tile, causal=causal, mode="mixed", fmt8=f8, out_dtype=torch.float32)
+    _compare(got, want, f"{fmt8} causal={causal} N={N} D={D} tile={tile}")
+    # the mixed scores differ from both single-precision runs (so the kernel really mixed the operand sets)
+    m4 = _run(q, k, v, is_causal=causal, block_scale_type="mxfp4", tile=tile, output_dtype=torch.float32)
+    assert not torch.equal(got, m4)
+
+
+@pytest.mark.parametrize("bst", ["mxfp4", "mxfp8", "mxfp8e5", "mixed"])
+def test_reference_call_sequence_quantize_package_attend(bst):
+    """The reference wrapper's own sequence (ours/mxfp_attn_kernel.py:36-72): quantize, reshape the scales to the packed
+    layout, initialize_block_scaled_batched_from_tensor, block_scaled_batched_attn."""
+    from ours.mxfp_attn_kernel import initialize_block_scaled_batched_from_tensor, block_scaled_batched_attn
+    from ours.quant_mxint8 import quantize_mx, pre_scale_q
+    from ours.mxfp import MXFP4Tensor
+    B, H, Hkv, M, N, K = 1, 4, 2, 256, 384, 128
+    g = torch.Generator().manual_seed(42)
+    q = torch.randn(B, H, M, K, generator=g).to(torch.float16)
+    k = torch.randn(B, Hkv, N, K, generator=g).to(torch.float16)
+    v = torch.randn(B, Hkv, N, K, generator=g).to(torch.float16)
+    f8 = _lib.FMT_E5M2 if bst == "mxfp8e5" else _lib.FMT_E4M3
+    fq = _lib.FMT_E2M1 if bst == "mxfp4" else f8
+    fk = f8 if bst in ("mxfp8", "mxfp8e5") else _lib.FMT_E2M1
+    def quant_one_code_per_byte(x, pre, fmt):             # what the reference's quantizer returns
+        c, s = quantize_mx(x, pre, fmt)
+        if fmt == _lib.FMT_E2M1:
+            c = MXFP4Tensor(size=(1,)).unpack_packed_tensor(c, 3, (*c.shape[:3], c.shape[3] * 2))
+        return c, s
+
+    a_quant, a_scale = quant_one_code_per_byte(q.to(DEV), pre_scale_q(K), fq)
+    b_quant, b_scale = quant_one_code_per_byte(k.to(DEV), 1.0, fk)
+    # the reference's reshape/permute to [B, H, rows/128, K/128, 32, 4, 4] (ours/mxfp_attn_kernel.py:56-57)
+    a_scale = a_scale.reshape(B, H, M // 128, 4, 32, K // 32 // 4, 4).permute(0, 1, 2, 5, 4, 3, 6).contiguous()
+    b_scale = b_scale.reshape(B, Hkv, N // 128, 4, 32, K // 32 // 4, 4).permute(0, 1, 2, 5, 4, 3, 6).contiguous()
+    a_packed, a_scale, b_packed, b_scale, configs, (reference, _, _) = initialize_block_scaled_batched_from_tensor(
+        a_quant, b_quant, a_scale, b_scale, block_scale_type=bst, compute_reference=False)
+    assert reference is None
+    out = block_scaled_batched_attn(a_packed, a_scale, b_packed, b_scale, v.to(DEV), torch.float16, B, H, M, N, K, configs)
+    assert out.shape == (B, H, M, K) and out.dtype == torch.float16
+    mode = {"mxfp4": "mxfp4", "mxfp8": "mxfp8", "mxfp8e5": "mxfp8", "mixed": "mixed"}[bst]
+    want = O.attn_mx(q, k, v, tile=128, causal=False, mode=mode, fmt8=O.FMT_E5M2 if bst == "mxfp8e5" else O.FMT_E4M3)
+    _compare(out, want, f"reference sequence {bst}")
+    with pytest.raises(NotImplementedError):
+        initialize_block_scaled_batched_from_tensor(a_quant, b_quant, a_scale, b_scale, block_scale_type=bst, compute_reference=True)
+    with pytest.raises(ValueError, match="Unsupported dtype"):
+        block_scaled_batched_attn(a_packed, a_scale, b_packed, b_scale, v.to(DEV), torch.float8_e5m2, B, H, M, N, K, configs)

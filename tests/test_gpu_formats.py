@@ -70,3 +70,20 @@ def test_e8m0_golden():
     assert torch.equal(dec[:255], ref[:255]) and torch.isnan(dec[255])
     r = MXScaleTensor(size=(1000,), device=DEV).random(low=1 / 16, high=16)
     assert r.data.min() >= 123 and r.data.max() <= 131
+
+
+@pytest.mark.parametrize("fmt,dt", [(1, torch.float8_e5m2), (0, torch.float8_e4m3fn)])
+def test_fp8_elementwise_cast_equals_torch(fmt, dt):
+    """mpsa_fp8_encode against torch's own float32 -> FP8 cast on the CPU (a library routine): every float16 value (all
+    65536 bit patterns, NaN and infinities included), a dense sweep around the formats' largest values, subnormals."""
+    from ours.block_scaled_matmul import fp8_cast
+    halves = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.float16).float()
+    big = torch.linspace(400.0, 70000.0, 20001)
+    tiny = torch.linspace(0.0, 2.0 ** -5, 4097)
+    special = torch.tensor([448.0, 464.0, 464.0001, 479.99, 480.0, 57344.0, 61440.0, 61439.9, 65536.0, float("inf"), float("nan"), -0.0])
+    x = torch.cat([halves, big, -big, tiny, -tiny, special, -special])
+    got = fp8_cast(x.to(DEV), fmt).cpu()
+    want = x.to(dt).view(torch.uint8)
+    nan = torch.isnan(want.view(dt).float())
+    assert torch.equal(got[~nan], want[~nan])
+    assert torch.isnan(got.view(dt).float()[nan]).all()          # NaN stays NaN (any payload)

@@ -17,7 +17,7 @@ import torch
 import oracle as O
 from conftest import make_qkv
 from ours import _lib
-from ours.block_scaled_matmul import block_scaled_matmul, initialize_block_scaled_from_tensor, make_configs
+from ours.block_scaled_matmul import block_scaled_matmul, quantize_block_scaled_from_tensor, make_configs
 from ours.mxfp import MXFP4Tensor, MXScaleTensor
 
 pytestmark = pytest.mark.gpu
@@ -45,7 +45,7 @@ def _operands(M, N, K, bst, seed):
     g = torch.Generator().manual_seed(seed)
     a = torch.randn(M, K, generator=g).bfloat16()
     b = torch.randn(N, K, generator=g).bfloat16()
-    return a, b, initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst)
+    return a, b, quantize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst)
 
 
 @pytest.mark.parametrize("bst", ["mxfp4", "mxfp8", "mxfp8e5"])
@@ -93,7 +93,7 @@ def test_identity_like_operand_selects_rows():
     b = torch.zeros(N, K)
     cols = torch.randint(0, K, (N,), generator=g)
     b[torch.arange(N), cols] = 4.0
-    ac, asc, bc, bsc, cfg = initialize_block_scaled_from_tensor(a.to(DEV), b.bfloat16().to(DEV), "mxfp8")
+    ac, asc, bc, bsc, cfg = quantize_block_scaled_from_tensor(a.to(DEV), b.bfloat16().to(DEV), "mxfp8")
     got = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg).cpu()
     adq = O.dequantize_mx(*O.quantize_mx(a, 1.0, O.FMT_E4M3), O.FMT_E4M3)
     assert torch.equal(got, adq[:, cols] * 4.0)
@@ -124,8 +124,12 @@ def test_errors():
     ac, asc, bc, bsc, cfg = _operands(256, 256, 128, "mxfp4", 0)[2]
     with pytest.raises(ValueError, match="Unsupported dtype"):
         block_scaled_matmul(ac, asc, bc, bsc, torch.int32, 256, 256, 128, cfg)
-    with pytest.raises(_lib.MpsaError, match="multiples of 256"):
-        block_scaled_matmul(ac[:128], asc[:128], bc, bsc, torch.float32, 128, 256, 128, cfg)
+    L = _lib.lib()
+    args = lambda K, packed=False: (_lib.ptr(ac), _lib.ptr(asc), 4, _lib.ptr(bc), _lib.ptr(bsc), 4, 256, 256, K, _lib.ptr(ac), 2, 256, None)
+    assert L.mpsa_gemm_mx(*args(96)) == -3 and b"multiple of 64" in L.mpsa_last_error()
+    assert L.mpsa_gemm_mx_packed(_lib.ptr(ac), _lib.ptr(asc), 4, _lib.ptr(bc), _lib.ptr(bsc), 4, 192, 256, 128, _lib.ptr(ac), 2, 256, None) == -3
+    assert b"packed scales need" in L.mpsa_last_error()
+    assert L.mpsa_gemm_mx(_lib.ptr(ac), _lib.ptr(asc), 9, _lib.ptr(bc), _lib.ptr(bsc), 4, 256, 256, 128, _lib.ptr(ac), 2, 256, None) == -1
 
 
 def test_scale_5d_layout_and_matmul_with_packed_scales():
@@ -140,7 +144,7 @@ def test_scale_5d_layout_and_matmul_with_packed_scales():
     M, N, K = 256, 512, 512
     a = torch.randn(M, K, generator=g).bfloat16()
     b = torch.randn(N, K, generator=g).bfloat16()
-    ac, asc, bc, bsc, cfg = initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), "mxfp4")
+    ac, asc, bc, bsc, cfg = quantize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), "mxfp4")
     c_lin = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg)
     c_pk = block_scaled_matmul(ac, pack_scale_5d(asc), bc, pack_scale_5d(bsc), torch.float32, M, N, K, cfg)
     assert torch.equal(c_lin, c_pk)
@@ -159,7 +163,7 @@ def test_packed_scale_kernel_path_equals_the_row_major_one(bst, M, N, K):
     g = torch.Generator().manual_seed(M + N + K)
     a = (torch.randn(M, K, generator=g) * torch.exp2(torch.randint(-6, 6, (M, 1), generator=g).float())).bfloat16()
     b = (torch.randn(N, K, generator=g) * torch.exp2(torch.randint(-6, 6, (1, K), generator=g).float())).bfloat16()
-    ac, asc, bc, bsc, cfg = initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst)
+    ac, asc, bc, bsc, cfg = quantize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst)
     assert asc.unique().numel() > 4                               # scales that differ: a mixed-up byte would show
     a5, b5 = pack_scale_5d(asc), pack_scale_5d(bsc)
     for dt in (torch.float32, torch.bfloat16, torch.float16, torch.float8_e5m2):
@@ -167,7 +171,7 @@ def test_packed_scale_kernel_path_equals_the_row_major_one(bst, M, N, K):
         c_pk = block_scaled_matmul(ac, a5, bc, b5, dt, M, N, K, cfg)
         assert torch.equal(c_lin.view(torch.uint8) if dt == torch.float8_e5m2 else c_lin,
                            c_pk.view(torch.uint8) if dt == torch.float8_e5m2 else c_pk), f"{bst} {M}x{N}x{K} {dt}"
-    ac2, a52, bc2, b52, _ = initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst, packed_scales=True)
+    ac2, a52, bc2, b52, _ = quantize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst, packed_scales=True)
     assert torch.equal(a52, a5) and torch.equal(b52, b5) and torch.equal(ac2, ac)
 
 
@@ -179,7 +183,7 @@ def test_e5m2_output_dtype():
     a = (torch.randn(M, K, generator=g) * 8).bfloat16()
     b = (torch.randn(N, K, generator=g) * 8).bfloat16()
     a[0] *= 64                                                   # one row large enough to overflow E5M2 (57344)
-    ac, asc, bc, bsc, cfg = initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), "mxfp4")
+    ac, asc, bc, bsc, cfg = quantize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), "mxfp4")
     c32 = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg)
     c8 = block_scaled_matmul(ac, asc, bc, bsc, torch.float8_e5m2, M, N, K, cfg)
     assert c8.dtype == torch.float8_e5m2
@@ -215,3 +219,111 @@ def test_batched_matmul_scores_with_grouped_heads(bst):
     assert ((got.cpu() - want).abs() <= 1e-3 * want.abs() + 3e-5 * mag.float().amax()).all()
     got5 = block_scaled_batched_matmul(qc, pack_scale_5d(qs), kc, pack_scale_5d(ks), torch.float32, B, H, M, N, K, cfg)
     assert torch.equal(got5, got)
+
+
+def _oracle_operand(values, four_bit, f8):
+    """CPU restatement of one packaged operand: the elementwise cast (E2M1 through the oracle's encoder, FP8 through
+    torch's own cast -- a library routine, not the reference) and the bytes the kernel is handed."""
+    x = values.float()
+    if four_bit:
+        return O.pack_fp4(O.encode_e2m1(x)), O.FMT_E2M1
+    dt = torch.float8_e5m2 if f8 == O.FMT_E5M2 else torch.float8_e4m3fn
+    return x.to(dt).view(torch.uint8), f8
+
+
+@pytest.mark.parametrize("bst", ["mxfp8e5", "mxfp8", "mixed_e5", "mixed", "mxfp4"])
+def test_reference_validate_call_sequence(bst):
+    """validate_block_scaled_from_tensor(128, 256, 256) of the reference (ours/block_scaled_matmul.py:409-441, :498,
+    seed 42 from :501): fp16 operands, float scale factors rand + 1e-8 in the packed 5-D layout,
+    initialize_block_scaled_from_tensor with the reference's positional arguments, block_scaled_matmul to fp16.
+    "mxfp8e5" is the reference's own 8-bit format; the result is compared with the oracle's product of the same codes
+    and E8M0 bytes (the reference's assert_close bound, atol = rtol = 1e-3, is checked for the types with a 4-bit
+    operand; the 8-bit x 8-bit bound is the norm-wise one used throughout this file)."""
+    from ours.block_scaled_matmul import initialize_block_scaled_from_tensor
+    M, N, K = 128, 256, 256
+    torch.manual_seed(42)
+    a_tensor = torch.randn((M, K), dtype=torch.float16)
+    b_tensor = torch.randn((N, K), dtype=torch.float16)
+    a_scale_tensor = torch.rand((M // 128, K // 32 // 4, 32, 4, 4)) + 1e-8
+    b_scale_tensor = torch.rand((N // 128, K // 32 // 4, 32, 4, 4)) + 1e-8
+    a_desc, a_scale, b_desc, b_scale, configs, reference = initialize_block_scaled_from_tensor(
+        a_tensor.to(DEV), b_tensor.to(DEV), a_scale_tensor.to(DEV), b_scale_tensor.to(DEV), bst, False)
+    assert reference is None
+    output = block_scaled_matmul(a_desc, a_scale, b_desc, b_scale, torch.float16, M, N, K, configs)
+    assert output.shape == (M, N) and output.dtype == torch.float16
+    f8 = O.FMT_E5M2 if bst.endswith("e5") else O.FMT_E4M3
+    a_codes, fa = _oracle_operand(a_tensor, bst == "mxfp4", f8)
+    b_codes, fb = _oracle_operand(b_tensor, bst in ("mxfp4", "mixed", "mixed_e5"), f8)
+    assert torch.equal(a_desc.cpu().view(torch.uint8), a_codes) and torch.equal(b_desc.cpu().view(torch.uint8), b_codes)
+    sa, sb = O.encode_e8m0(a_scale_tensor), O.encode_e8m0(b_scale_tensor)
+    assert torch.equal(a_scale.cpu(), sa) and torch.equal(b_scale.cpu(), sb)
+    sa_lin, sb_lin = O.scales_from_5d(sa), O.scales_from_5d(sb)
+    want = O.gemm_mx(a_codes, sa_lin, b_codes, sb_lin, fa, fb, acc_dtype=torch.float64)
+    mag = O.dequantize_mx(a_codes, sa_lin, fa, torch.float64).abs() @ O.dequantize_mx(b_codes, sb_lin, fb, torch.float64).abs().T
+    err = (output.cpu().double() - want).abs()
+    if fa == O.FMT_E2M1 or fb == O.FMT_E2M1:
+        # the reference's own bound holds where a 4-bit operand keeps the products short
+        assert (err <= 1e-3 + 1e-3 * want.abs()).all(), err.max()
+    assert (err <= (1e-3 + 2 ** -10) * want.abs() + 3e-5 * mag).all(), (err / mag).max()
+    with pytest.raises(NotImplementedError):
+        initialize_block_scaled_from_tensor(a_tensor.to(DEV), b_tensor.to(DEV), a_scale_tensor.to(DEV), b_scale_tensor.to(DEV), bst, True)
+    with pytest.raises(NotImplementedError, match="nvfp4"):
+        initialize_block_scaled_from_tensor(a_tensor.to(DEV), b_tensor.to(DEV), a_scale_tensor.to(DEV), b_scale_tensor.to(DEV), "nvfp4")
+
+
+@pytest.mark.parametrize("fa,fb", [(O.FMT_E2M1, O.FMT_E2M1), (O.FMT_E4M3, O.FMT_E4M3), (O.FMT_E5M2, O.FMT_E5M2),
+                                   (O.FMT_E4M3, O.FMT_E2M1), (O.FMT_E5M2, O.FMT_E2M1), (O.FMT_E2M1, O.FMT_E4M3),
+                                   (O.FMT_E4M3, O.FMT_E5M2)])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 256), (100, 200, 192), (1, 1, 64), (384, 128, 640), (257, 129, 128)])
+def test_edge_tiles_and_mixed_formats_against_oracle(fa, fb, M, N, K):
+    """Shapes off the 256 x 256 tile (the reference's kernel masks its edge tiles, ours/block_scaled_matmul.py:154-267)
+    and operands of different element formats (ELEM_PER_BYTE_A != ELEM_PER_BYTE_B, :318-324), through the C ABI."""
+    from ours.quant_mxint8 import quantize_mx
+    g = torch.Generator().manual_seed(M * 7 + N * 3 + K + fa + 10 * fb)
+    a = (torch.randn(M, K, generator=g) * torch.exp2(torch.randint(-4, 4, (M, 1), generator=g).float())).bfloat16()
+    b = (torch.randn(N, K, generator=g) * torch.exp2(torch.randint(-4, 4, (1, K), generator=g).float())).bfloat16()
+    ac, asc = (t[0, 0] for t in quantize_mx(a[None, None].to(DEV), 1.0, fa))
+    bc, bsc = (t[0, 0] for t in quantize_mx(b[None, None].to(DEV), 1.0, fb))
+    out = torch.full((M, N + 3), 7.0, dtype=torch.float32, device=DEV)          # ldc > N: the padding must stay
+    _lib.check(_lib.lib().mpsa_gemm_mx(_lib.ptr(ac), _lib.ptr(asc), fa, _lib.ptr(bc), _lib.ptr(bsc), fb, M, N, K,
+                                       _lib.ptr(out), _lib.F32, N + 3, _lib.stream_ptr()))
+    assert (out[:, N:] == 7.0).all()
+    want = O.gemm_mx(ac.cpu(), asc.cpu(), bc.cpu(), bsc.cpu(), fa, fb, acc_dtype=torch.float64)
+    mag = O.dequantize_mx(ac.cpu(), asc.cpu(), fa, torch.float64).abs() @ O.dequantize_mx(bc.cpu(), bsc.cpu(), fb, torch.float64).abs().T
+    err = (out[:, :N].cpu().double() - want).abs()
+    # E2M1 x E2M1 products and their float32 sums are exact.  With an 8-bit operand the matrix core aligns the 64
+    # products of a step to the largest exponent and keeps about 16 bits below it; these operands carry a 2^8 spread
+    # of magnitudes inside every MX block (the column gains of b), so more of the small products' bits fall off than
+    # with the Gaussian operands of the other tests: measured err / sum|a||b| up to 5.5e-5 (E5M2 x E5M2).
+    exact = fa == O.FMT_E2M1 and fb == O.FMT_E2M1
+    bound = 1e-7 * mag if exact else 1e-3 * want.abs() + 1e-4 * mag
+    assert (err <= bound).all(), f"worst err/mag {(err / mag.clamp_min(1e-30)).max().item():.3e}"
+
+
+@pytest.mark.parametrize("bst", ["mxfp4", "mxfp8"])
+def test_general_kernel_equals_the_staged_kernel_on_its_shapes(bst):
+    """A 512 x 256 product computed whole (LDS-staged 256 x 256 kernel) and as two row slabs of 384 and 128 rows (the
+    general kernel: 384 is not a multiple of 256): same K order, same matrix instruction, same bits."""
+    M, N, K = 512, 256, 1024
+    a, b, (ac, asc, bc, bsc, cfg) = _operands(M, N, K, bst, seed=77)
+    whole = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg)
+    top = block_scaled_matmul(ac[:384].contiguous(), asc[:384].contiguous(), bc, bsc, torch.float32, 384, N, K, cfg)
+    bottom = block_scaled_matmul(ac[384:].contiguous(), asc[384:].contiguous(), bc, bsc, torch.float32, 128, N, K, cfg)
+    assert torch.equal(whole, torch.cat([top, bottom]))
+
+
+def test_batched_mixed_formats_with_grouped_heads():
+    """The batched entry point with 8-bit A against 4-bit B (the reference's "mixed" Q.K^T) and grouped heads."""
+    from ours.batched_block_scaled_matmul import block_scaled_batched_matmul
+    from ours.quant_mxint8 import quantize_mx
+    B, H, Hkv, M, N, K = 2, 4, 2, 128, 384, 128
+    q, k, _ = make_qkv(B, H, Hkv, 384, K, seed=15)
+    q = q[:, :, :M].contiguous()
+    qc, qs = quantize_mx(q.to(DEV), O.q_pre_scale(K), O.FMT_E4M3)
+    kc, ks = quantize_mx(k.to(DEV), 1.0, O.FMT_E2M1)
+    got = block_scaled_batched_matmul(qc, qs, kc, ks, torch.float32, B, H, M, N, K, make_configs("mixed"))
+    want = O.gemm_mx(qc.cpu(), qs.cpu(), kc.cpu().repeat_interleave(2, dim=1), ks.cpu().repeat_interleave(2, dim=1),
+                     O.FMT_E4M3, O.FMT_E2M1, acc_dtype=torch.float64)
+    mag = O.dequantize_mx(qc.cpu(), qs.cpu(), O.FMT_E4M3, torch.float64).abs() @ \
+        O.dequantize_mx(kc.cpu().repeat_interleave(2, dim=1), ks.cpu().repeat_interleave(2, dim=1), O.FMT_E2M1, torch.float64).abs().transpose(-1, -2)
+    assert ((got.cpu().double() - want).abs() <= 1e-3 * want.abs() + 3e-5 * mag).all()

@@ -242,3 +242,42 @@ def test_routed_dit_shape_thresholds_off_equals_mxfp4():
     cos = torch.nn.functional.cosine_similarity(out.float().flatten(), ref8.float().flatten(), dim=0).item()
     cos4 = torch.nn.functional.cosine_similarity(want.float().flatten(), ref8.float().flatten(), dim=0).item()
     assert cos >= cos4 - 1e-4, (cos, cos4)                 # 8-bit tiles do not make it worse than all-4-bit
+
+
+def test_c5_video_dit_all_heads_diag_and_routed():
+    """B=1 H=40 N=32760 (21 frames x 1560 tokens, a ragged last tile) D=128, bidirectional, q/k/v ~ N(0, 0.5) seed 4
+    plus per-frame offsets: all 40 heads on the GPU in the diag mode and in the routed mode (route_thresh 0.9).  The
+    oracle checks sampled (head, query tile) pairs -- first, middle and the ragged last tile -- and, for the routed
+    run, with its OWN class map computed from its own scale bytes (which the GPU's map must equal bit for bit)."""
+    N, H = 32760, 40
+    q, k, v = make_qkv(1, H, H, N, 128, seed=4, sigma=0.5)
+    q, k = _frames(q, k, 21, seed=5, amp=0.5)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    samples = {0: [0, 255], 7: [100], 19: [254, 37], 39: [255, 128]}
+    rows = lambda tiles: torch.cat([torch.arange(t * 128, min((t + 1) * 128, N)) for t in tiles])
+
+    got = mxfp_attn_kernel(qd, kd, vd, is_causal=False, block_scale_type="diag", tile=128, output_dtype=torch.float32)
+    assert torch.isfinite(got).all()
+    for h, tiles in samples.items():
+        want = O.attn_mx(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], tile=128, causal=False, mode="diag", q_tiles=tiles,
+                         out_dtype=torch.float32)
+        _compare(got[:, h:h + 1, rows(tiles).to(DEV)], want, f"C5 diag head {h} tiles {tiles}")
+    del got
+
+    ops = prepare_operands(qd, kd, vd, 128, "routed")
+    cls, order, counts = route_tiles(ops, False, 0.9, None)
+    share8 = float((cls == 2).float().mean())
+    assert 0.02 < share8 < 0.98, share8
+    out = torch.empty((1, H, N, 128), dtype=torch.float32, device=DEV)
+    attention_from_operands(ops, out, False, route=(cls, order, counts))
+    assert torch.isfinite(out).all()
+    pre = O.q_pre_scale(128)
+    for h, tiles in samples.items():
+        _, qs4 = O.quantize_mx(q[:, h:h + 1], pre, O.FMT_E2M1)
+        _, ks4 = O.quantize_mx(k[:, h:h + 1], 1.0, O.FMT_E2M1)
+        pad = lambda t: torch.nn.functional.pad(t, (0, 0, 0, 256 * 128 - N)).numpy()
+        own = O.route_tiles(pad(qs4), pad(ks4), 128, False, 0.9, None)
+        assert np.array_equal(cls[:, h:h + 1].cpu().numpy(), own), f"class map of head {h}"
+        want = O.attn_mx(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], tile=128, causal=False, mode="routed", route=own, q_tiles=tiles,
+                         out_dtype=torch.float32)
+        _compare(out[:, h:h + 1, rows(tiles).to(DEV)], want, f"C5 routed head {h} tiles {tiles}")

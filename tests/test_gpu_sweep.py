@@ -10,7 +10,7 @@ import torch
 
 import oracle as O
 from conftest import make_qkv
-from ours.block_scaled_matmul import block_scaled_matmul, initialize_block_scaled_from_tensor
+from ours.block_scaled_matmul import block_scaled_matmul, quantize_block_scaled_from_tensor
 from ours.mxfp_attn_kernel import prepare_operands, route_tiles, attention_from_operands, mxfp_attn_kernel
 from ours.quant_mxint8 import quantize_mx, quantize_mx_dual
 
@@ -117,7 +117,7 @@ def test_matmul_sweep():
         scale_a = torch.exp2(torch.randint(-4, 4, (M, K // 32), generator=g).float()).repeat_interleave(32, 1)
         a = (torch.randn(M, K, generator=g) * scale_a).bfloat16()
         b = torch.randn(N, K, generator=g).bfloat16()
-        ac, asc, bc, bsc, cfg = initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst)
+        ac, asc, bc, bsc, cfg = quantize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), bst)
         got = block_scaled_matmul(ac, asc, bc, bsc, dt, M, N, K, cfg).cpu()
         da = O.dequantize_mx(ac.cpu(), asc.cpu(), fmt, torch.float64)
         db = O.dequantize_mx(bc.cpu(), bsc.cpu(), fmt, torch.float64)

@@ -47,7 +47,7 @@ def test_gemm_fp8_against_float64_loop():
     assert (got - exact).abs().max() < 0.08 * exact.abs().max() + 0.5
 
 
-@pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "diag"])
+@pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "diag", "mixed"])
 @pytest.mark.parametrize("causal", [True, False])
 def test_attention_tile_loop_equals_dense_float64(mode, causal):
     q, k, v = make_qkv(1, 4, 2, 200, 64, seed=21)          # N not a multiple of the tile, GQA 2:1
@@ -155,3 +155,21 @@ def test_scale_5d_layout_index_formula_and_round_trip():
     for (bt, cm, ck, r32, r4, c4) in [(0, 0, 0, 0, 0, 0), (1, 1, 1, 31, 3, 3), (0, 1, 0, 7, 2, 1), (1, 0, 1, 30, 1, 2)]:
         assert pk[bt, cm, ck, r32, r4, c4] == lin[bt, cm * 128 + r4 * 32 + r32, ck * 4 + c4]
     assert torch.equal(O.scales_from_5d(pk), lin)
+
+
+def test_mixed_mode_is_8bit_q_times_4bit_k():
+    """The "mixed" scores are exactly dq8(Q) dq4(K)^T: with a single key (softmax weight 1) nothing else shows, so the
+    check goes through a two-key softmax whose weights follow from the score difference alone."""
+    torch.manual_seed(5)
+    q = torch.randn(1, 1, 1, 64).bfloat16()
+    k = torch.randn(1, 1, 2, 64).bfloat16()
+    v = torch.tensor([[[[1.0] * 64, [0.0] * 64]]]).bfloat16()
+    pre = O.q_pre_scale(64)
+    q8 = O.dequantize_mx(*O.quantize_mx(q, pre, O.FMT_E4M3), O.FMT_E4M3).double()
+    k4 = O.dequantize_mx(*O.quantize_mx(k, 1.0, O.FMT_E2M1), O.FMT_E2M1).double()
+    s = (q8[0, 0] @ k4[0, 0].T)[0]
+    want = 1.0 / (1.0 + 2.0 ** float(s[1] - s[0]))
+    got = O.attn_mx(q, k, v, tile=64, causal=False, mode="mixed", out_dtype=torch.float32)
+    assert abs(got[0, 0, 0, 0].item() - want) < 4e-3            # P is rounded to bf16
+    other = O.attn_mx(q, k, v, tile=64, causal=False, mode="mxfp4", out_dtype=torch.float32)
+    assert got[0, 0, 0, 0].item() != other[0, 0, 0, 0].item()
