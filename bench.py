@@ -153,22 +153,25 @@ def cpu_baseline(q, k, v, tile, D, causal=True):
 
 
 def secondary_c4(device):
-    """The long-context configuration (N = 131072) next to the headline line: fused attention kernel, whole step, and
-    the operand preparation on 2.9 GB of traffic -- far beyond the 256 MB last-level cache, i.e. the quantizer's
-    out-of-cache bandwidth."""
+    """The long-context configuration (N = 131072) next to the headline line: fused attention kernel (Q quantized in
+    the kernel), whole step, and the full operand preparation (Q, K, V) on 2.9 GB of traffic -- far beyond the 256 MB
+    last-level cache, i.e. the quantizer's out-of-cache bandwidth."""
     from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands
     B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS["c4"]
     q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device)
     out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
-    ops = prepare_operands(q, k, v, tile, "diag")
+    ops = prepare_operands(q, k, v, tile, "diag", fuse_q=True)
     attention_from_operands(ops, out, True)
     torch.cuda.synchronize()
     iters = 10
     attn_ms = time_events(lambda: attention_from_operands(ops, out, True), iters)
-    prep_ms = time_events(lambda: prepare_operands(q, k, v, tile, "diag", reuse=ops), iters)
+    # the operand preparation with Q included: 2.9 GB of traffic, the quantizer's out-of-cache figure
+    full = prepare_operands(q, k, v, tile, "diag")
+    prep_ms = time_events(lambda: prepare_operands(q, k, v, tile, "diag", reuse=full), iters)
+    del full
 
     def step():
-        attention_from_operands(prepare_operands(q, k, v, tile, "diag", reuse=ops), out, True)
+        attention_from_operands(prepare_operands(q, k, v, tile, "diag", reuse=ops, fuse_q=True), out, True)
 
     step()
     wait_for_device()
@@ -243,7 +246,9 @@ def run_only(args, device):
         causal = args.workload not in NON_CAUSAL
         q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21)
         out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
-        ops = prepare_operands(q, k, v, tile, args.mode)
+        from ours.mxfp_attn_kernel import q_fusable
+        fuse = args.mode != "routed" and not args.no_fuse_q and q_fusable(q, k, tile, args.mode, causal)
+        ops = prepare_operands(q, k, v, tile, args.mode, fuse_q=fuse)
         route = route_tiles(ops, causal, args.route_thresh, args.skip_thresh) if args.mode == "routed" else None
         fn = lambda: attention_from_operands(ops, out, causal, route=route)
         info = {"kernel": "attention", "workload": desc, "mode": args.mode}
@@ -282,8 +287,10 @@ def main():
                          "(tile router on the scale bytes, thresholds below)")
     ap.add_argument("--route-thresh", type=float, default=0.9, help="routed: 8-bit at or above this share of the row's largest tile statistic")
     ap.add_argument("--skip-thresh", type=float, default=None, help="routed: skipped below this share")
+    ap.add_argument("--spinup-ms", type=float, default=80.0, help="untimed device spin-up (steps run for this long) before the warm-up steps")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--no-fuse-q", action="store_true", help="with --only attn: hand the kernel quantized Q operands")
     ap.add_argument("--no-c4", action="store_true", help="leave the long-context figures out of `secondary`")
     ap.add_argument("--eager", action="store_true", help="time plain launches instead of replaying the step as a HIP graph")
     ap.add_argument("--linear-scales", action="store_true",
@@ -307,7 +314,7 @@ def main():
         print("bench.py needs a HIP device", file=sys.stderr)
         sys.exit(1)
 
-    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, route_tiles
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, route_tiles, q_fusable
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
@@ -327,10 +334,12 @@ def main():
     if not args.no_secondary:
         second = secondary(device, quick=args.steps < 10)
 
-    state = {"ops": prepare_operands(q, k, v, tile, args.mode)}
+    # shapes of the paired-tile kernel: Q stays unquantized and the attention kernel quantizes it in registers
+    fuse_q = not routed and q_fusable(q, k, tile, args.mode, causal)
+    state = {"ops": prepare_operands(q, k, v, tile, args.mode, fuse_q=fuse_q)}
 
     def step():
-        ops = prepare_operands(q, k, v, tile, args.mode, reuse=state["ops"])
+        ops = prepare_operands(q, k, v, tile, args.mode, reuse=state["ops"], fuse_q=fuse_q)
         route = route_tiles(ops, causal, args.route_thresh, args.skip_thresh) if routed else None
         attention_from_operands(ops, out, causal, route=route)
 
@@ -350,6 +359,14 @@ def main():
             print(f"bench: graph capture failed ({e}); timing eager launches", file=sys.stderr)
             run_step, launch = step, "eager"
 
+    # Device spin-up, untimed and before the warm-up steps: a GPU that has idled runs its first milliseconds at a low
+    # clock, and `--warmup 5` steps of 0.4 ms do not bring it up (measured: 20 timed steps read 0.42 ms/step without
+    # this and 0.37 with it, the same as 500 timed steps).
+    t_spin = time.perf_counter()
+    while (time.perf_counter() - t_spin) * 1e3 < args.spinup_ms:
+        for _ in range(10):
+            run_step()
+        wait_for_device()
     for _ in range(args.warmup):
         run_step()
     wait_for_device()
@@ -363,13 +380,13 @@ def main():
     tflops = flops / (ms_per_step * 1e-3) / 1e12
 
     # dominant kernel alone: the fused attention kernel on prepared operands
-    ops = prepare_operands(q, k, v, tile, args.mode)
+    ops = prepare_operands(q, k, v, tile, args.mode, fuse_q=fuse_q)
     route = route_tiles(ops, causal, args.route_thresh, args.skip_thresh) if routed else None
     attention_from_operands(ops, out, causal, route=route)
     torch.cuda.synchronize()
     k_iters = max(5, args.steps)
     attn_ms = time_events(lambda: attention_from_operands(ops, out, causal, route=route), k_iters)
-    prep_ms = time_events(lambda: prepare_operands(q, k, v, tile, args.mode, reuse=ops), k_iters)
+    prep_ms = time_events(lambda: prepare_operands(q, k, v, tile, args.mode, reuse=ops, fuse_q=fuse_q), k_iters)
     achieved = flops / (attn_ms * 1e-3) / 1e12
     nt = (N + tile - 1) // tile
     comp = composite_peak_tflops(nt, causal)
@@ -397,8 +414,9 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "mxfp4/mxfp8 scores (E2M1/E4M3 + E8M0), bf16 P.V, f32 accumulate", "data": "synthetic",
         "config": {"workload": desc, "B": B, "Hq": Hq, "Hkv": Hkv, "N": N, "D": D, "tile": tile, "mode": args.mode,
-                   "step": "quantize Q,K (dual) + V repack + " + ("tile router + " if routed else "") + "fused attention",
-                   "launch": launch},
+                   "step": ("quantize K (dual) + V repack + fused attention with Q quantized in the kernel" if fuse_q else
+                            "quantize Q,K (dual) + V repack + " + ("tile router + " if routed else "") + "fused attention"),
+                   "launch": launch, "spinup_ms": args.spinup_ms},
         "frac_mxfp4_peak": round(tflops / PEAK_FP4_TFLOPS, 5),
         "roofline": roofline,
     }

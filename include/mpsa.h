@@ -225,7 +225,8 @@ int mpsa_v_tiles(const void* v, int v_dtype, int64_t B, int64_t H, int64_t N, in
  * mpsa_quantize_mx(_dual) on q and k (emax 3 for E2M1, 7 for the 8-bit format) and mpsa_v_tiles on v, rows padded to
  * ceil(Nq/tile)*tile and ceil(Nk/tile)*tile.  Replaces the prologue of the reference's wrapper, ours/mxfp_attn_kernel.py:27-57.
  *
- *   q [B,Hq,Nq,D], k and v [B,Hkv,Nk,D] of dtype (MPSA_BF16 | MPSA_F16), element strides as for mpsa_quantize_mx
+ *   q [B,Hq,Nq,D], k and v [B,Hkv,Nk,D] of dtype (MPSA_BF16 | MPSA_F16), element strides as for mpsa_quantize_mx;
+ *              q == NULL leaves Q out (its outputs are not touched): for mpsa_attn_fwd_q16, which quantizes Q itself
  *   mode       MPSA_MODE_MXFP4: only the 4-bit outputs are written (8-bit pointers may be null),
  *              MPSA_MODE_MXFP8: only the 8-bit ones, MPSA_MODE_DIAG / MPSA_MODE_ROUTED / MPSA_MODE_MIXED: both
  *   k_sub      NULL or [B,Hkv,D] (smooth-K mean from mpsa_seq_mean)
@@ -263,6 +264,26 @@ int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, cons
                   const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
                   int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t nk, int64_t D, int tile, int causal, int mode,
                   mpsa_stream_t stream);
+
+/*
+ * Fused attention forward that takes Q UNQUANTIZED and MX-quantizes it inside the kernel, in registers: the quantizer
+ * call for Q of the reference's wrapper (quant_mxfp4 / quant_mxfp8e5 on q, ours/mxfp_attn_kernel.py:43-50,
+ * ours/quant_mxint8.py:479-494) and the attention launch (ours/mxfp_attn_kernel.py:66-70) in one; Q's codes and scales
+ * never travel through HBM (at the B1 Hq32 N8192 shape that is 52 MB written and read back).  Same bits as
+ * mpsa_attn_prepare + mpsa_attn_fwd.  Built for the paired-tile kernel's shapes only: causal, D = 128, tile = 128, n a
+ * multiple of 256, mode MPSA_MODE_DIAG or MPSA_MODE_MXFP4 -- mpsa_attn_fwd_q16_supported() says whether a shape
+ * qualifies (1) or not (0); other shapes return MPSA_EUNSUPPORTED and go through mpsa_attn_prepare + mpsa_attn_fwd.
+ *   q            [B,Hq,n,D] of q_dtype == pv_dtype (MPSA_BF16 | MPSA_F16), element strides q_strides[4], last dim
+ *                contiguous, rows 16-byte aligned
+ *   pre_scale_q  float32 factor folded in before quantizing (sm_scale * log2(e))
+ *   k4 .. v_tiles, o   as for mpsa_attn_fwd; mpsa_attn_prepare with q == NULL prepares just these (K and V)
+ */
+int mpsa_attn_fwd_q16(const void* q, const int64_t q_strides[4], int q_dtype, float pre_scale_q,
+                      const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
+                      const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
+                      int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                      mpsa_stream_t stream);
+int mpsa_attn_fwd_q16_supported(int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode);
 
 /*
  * Fused attention forward with the reference's tile-skipping rule (the skip_thresh argument of mxfp_attn /

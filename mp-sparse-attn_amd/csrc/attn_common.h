@@ -16,6 +16,11 @@ struct AttnArgs {
     int32_t* skipped;          // optional [B,Hq,nt] count of skipped key tiles per query tile
     const int32_t* order;      // routed runs only: [B,Hq,ntq,nt] visiting lists and [B,Hq,ntq,4] run lengths
     const int32_t* counts;
+    // paired-tile kernel with the Q quantizer fused in: unquantized Q (16-bit, element strides, last dim contiguous)
+    // and the factor folded in before quantizing; q4 / qs4 / q8 / qs8 are unused then
+    const void* q_raw;
+    int64_t q_sb, q_sh, q_sn;
+    float q_pre;
 };
 
 template <int PVT> struct PV;
@@ -113,4 +118,4 @@ int attn_routed_launch(const AttnArgs& a, int pv_dtype, hipStream_t st);
 
 // Paired-tile ("ping-pong") kernel for causal runs with D = 128, tile = 128 and whole tile pairs: attn_fwd_pp.hip
 bool attn_pp_supported(const AttnArgs& a, int pv_dtype);
-int attn_pp_launch(const AttnArgs& a, int pv_dtype, hipStream_t st);
+int attn_pp_launch(const AttnArgs& a, int pv_dtype, hipStream_t st);       // a.q_raw != nullptr: the fused-quantizer variants

@@ -55,7 +55,9 @@ int launch_dt(const AttnArgs& a, int pv_dtype, hipStream_t st) {
 
 }  // namespace
 
-static int attn_entry(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
+struct RawQ { const void* q; const int64_t* strides; int dtype; float pre; };
+
+static int attn_entry(const RawQ* rq, const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
                       const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
                       const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
                       int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal, int mode,
@@ -67,7 +69,14 @@ static int attn_entry(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, 
     if (routed && ((reinterpret_cast<uintptr_t>(order) | reinterpret_cast<uintptr_t>(counts)) & 3)) return mpsa_fail(MPSA_EALIGN, "attn: order and counts must be 4-byte aligned");
     const bool mixed = mode == MPSA_MODE_MIXED;
     const bool need4 = mode != MPSA_MODE_MXFP8, need8 = mode != MPSA_MODE_MXFP4;
-    if (mixed) {
+    if (rq) {
+        if (!rq->q || !rq->strides) return mpsa_fail(MPSA_EINVAL, "attn: null q");
+        if (rq->dtype != pv_dtype) return mpsa_fail(MPSA_EINVAL, "attn: unquantized q must have the P.V dtype (the dtype of v)");
+        if (rq->strides[3] != 1 || !mpsa_aligned16(rq->q) || (rq->strides[0] % 8) || (rq->strides[1] % 8) || (rq->strides[2] % 8))
+            return mpsa_fail(MPSA_EALIGN, "attn: q rows must be contiguous and 16-byte aligned");
+        if (mode != MPSA_MODE_DIAG && mode != MPSA_MODE_MXFP4) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: unquantized q is taken in the diag and mxfp4 modes only");
+        if ((need4 && (!k4 || !ks4)) || (need8 && (!k8 || !ks8))) return mpsa_fail(MPSA_EINVAL, "attn: K operands missing");
+    } else if (mixed) {
         if (!q8 || !qs8 || !k4 || !ks4) return mpsa_fail(MPSA_EINVAL, "attn: the mixed mode needs 8-bit Q and 4-bit K operands");
     } else {
         if (need4 && (!q4 || !qs4 || !k4 || !ks4)) return mpsa_fail(MPSA_EINVAL, "attn: 4-bit operands missing");
@@ -97,7 +106,15 @@ static int attn_entry(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, 
     a.d = (int)D; a.tile = tile;
     a.skip_thresh = skip_thresh; a.skipped = skipped;
     a.order = order; a.counts = counts;
+    a.q_raw = nullptr; a.q_sb = a.q_sh = a.q_sn = 0; a.q_pre = 1.0f;
     hipStream_t st = (hipStream_t)stream;
+    if (rq) {
+        a.q_raw = rq->q; a.q_sb = rq->strides[0]; a.q_sh = rq->strides[1]; a.q_sn = rq->strides[2]; a.q_pre = rq->pre;
+        if (!attn_pp_supported(a, pv_dtype))
+            return mpsa_fail(MPSA_EUNSUPPORTED, "attn: unquantized q needs the paired-tile kernel's shape (causal, D = 128, tile = 128, "
+                                                "sequence a multiple of 256); quantize q with mpsa_attn_prepare and call mpsa_attn_fwd");
+        return attn_pp_launch(a, pv_dtype, st);
+    }
     if (routed) return attn_routed_launch(a, pv_dtype, st);
     if (skip) {
         if (mixed) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: tile skipping is built for the mxfp4 and mxfp8 modes only");
@@ -118,7 +135,7 @@ extern "C" int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_
                              const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
                              int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal, int mode,
                              mpsa_stream_t stream) {
-    return attn_entry(q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
+    return attn_entry(nullptr, q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
                       B, Hq, Hkv, nq, n, D, tile, causal, mode, false, 0.0f, nullptr, nullptr, nullptr, stream);
 }
 
@@ -127,7 +144,7 @@ extern "C" int mpsa_attn_fwd_skip(const uint8_t* q4, const uint8_t* qs4, const u
                                   const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
                                   int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal, int mode,
                                   float skip_thresh, int32_t* skipped, mpsa_stream_t stream) {
-    return attn_entry(q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
+    return attn_entry(nullptr, q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
                       B, Hq, Hkv, nq, n, D, tile, causal, mode, true, skip_thresh, skipped, nullptr, nullptr, stream);
 }
 
@@ -136,6 +153,24 @@ extern "C" int mpsa_attn_fwd_routed(const uint8_t* q4, const uint8_t* qs4, const
                                     const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
                                     int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t n, int64_t D, int tile, int causal,
                                     const int32_t* order, const int32_t* counts, mpsa_stream_t stream) {
-    return attn_entry(q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
+    return attn_entry(nullptr, q4, qs4, q8, qs8, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
                       B, Hq, Hkv, nq, n, D, tile, causal, MPSA_MODE_ROUTED, false, 0.0f, nullptr, order, counts, stream);
+}
+
+extern "C" int mpsa_attn_fwd_q16(const void* q, const int64_t q_strides[4], int q_dtype, float pre_scale_q,
+                                 const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
+                                 const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
+                                 int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode,
+                                 mpsa_stream_t stream) {
+    const RawQ rq = {q, q_strides, q_dtype, pre_scale_q};
+    return attn_entry(&rq, nullptr, nullptr, nullptr, nullptr, k4, ks4, k8, ks8, fmt8, v_tiles, pv_dtype, o, o_dtype, o_strides,
+                      B, Hq, Hkv, n, n, D, tile, causal, mode, false, 0.0f, nullptr, nullptr, nullptr, stream);
+}
+
+extern "C" int mpsa_attn_fwd_q16_supported(int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode) {
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || n <= 0 || Hq % Hkv || B * Hq * (n / 256 + 1) >= (int64_t(1) << 31)) return 0;
+    AttnArgs a = {};
+    a.B = (int)B; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.n = (int)n; a.d = (int)D; a.tile = tile; a.causal = causal ? 1 : 0; a.mode = mode;
+    a.nt = (int)((n + tile - 1) / (tile > 0 ? tile : 1)); a.n_pad = a.nt * tile;
+    return (tile == 64 || tile == 128) && attn_pp_supported(a, MPSA_BF16) ? 1 : 0;
 }

@@ -23,6 +23,7 @@
 // registers is two steps ahead of the P.V tile), V two; the single 8-bit (diagonal) tile of a "diag" run is read
 // straight from global memory.  The running maximum rides in the score MFMA's C operand.
 #include "attn_common.h"
+#include "quantize_kernel.h"
 
 namespace {
 
@@ -38,7 +39,10 @@ constexpr int VI = V_BYTES / 1024 / NWAVES;     // direct-load instructions per 
 constexpr int NV = KB * 2 * NDB;                // P.V matrix instructions per tile (32)
 static_assert(K_BYTES / 1024 == NWAVES, "one K direct-load instruction per wave");
 
-template <int PVT, int FMT8, int MODE>
+// QRAW: Q arrives unquantized (in the P.V dtype) and is MX-quantized here, in registers, with the quantizer's own device
+// functions -- the bits are those mpsa_quantize_mx would have written (ours/quant_mxint8.py:276-351, :164-219 with
+// sm_scale*log2(e) folded in, :479-494), but the codes and scales never travel through HBM.
+template <int PVT, int FMT8, int MODE, bool QRAW>
 __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     typedef PV<PVT> P;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -46,8 +50,9 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, w = tid >> 6;
     const int h = lane >> 5, r = lane & 31;
-    const int role = w >> 2;                     // 0 = X (tile 2I+1), 1 = Y (tile 2I)
-    const int wq = w & 3;
+    const int wu = __builtin_amdgcn_readfirstlane(w);    // the wave index, known to be uniform
+    const int role = wu >> 2;                    // 0 = X (tile 2I+1), 1 = Y (tile 2I); uniform, so the loops below are scalar
+    const int wq = wu & 3;
 
     // ---- which (batch, kv head, query head, query-tile pair) -- XCD-aware, heavy pairs first ----
     const int npairs = a.nt >> 1;
@@ -79,7 +84,83 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     int qsc = 0;
     v4i kf4[KB][SST];
     int ksc[KB];
+    // shared exponent of an MX block from its largest magnitude, as the quantizer takes it (quantize_kernel.h)
+    auto block_exponent = [&](float amax) __attribute__((always_inline)) {
+        const uint32_t ab = mpsa_f2u(amax);
+        const uint32_t ef = ab >> 23;
+        return ef ? (int)ef - 127 : (31 - __builtin_clz(ab | 1u)) - 149;
+    };
+    auto load_q_raw = [&](bool is8) __attribute__((always_inline)) {
+#pragma clang fp contract(off)        // the quantizer's arithmetic, operation by operation
+        // this lane's query row, unquantized; lane half h owns MX blocks h and 2+h of the row's four in the 4-bit
+        // layout, and one half (16 elements) of every block in the 8-bit layout
+        const char* row = static_cast<const char*>(a.q_raw) +
+                          2 * ((int64_t)b * a.q_sb + (int64_t)hq * a.q_sh + ((int64_t)i * TILE + q_local) * a.q_sn);
+        uint32_t sbytes = 0;
+        if (!is8) {
+#pragma unroll
+            for (int s = 0; s < SST; ++s) {
+                float x[4][8];
+                float amax = 0.0f;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    load8<PVT>(row + 2 * (32 * (2 * s + h) + 8 * c), x[c]);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        x[c][e] = x[c][e] * a.q_pre;
+                        amax = __builtin_fmaxf(amax, __builtin_fabsf(x[c][e]));
+                    }
+                }
+                const bool zero = mpsa_f2u(amax) == 0u;
+                const int se = block_exponent(amax) - 3;                       // emax of E2M1: ours/quant_mxint8.py:303
+                int w[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) w[c] = zero ? 0 : (int)e2m1_pack8<true>(x[c], se, false);
+                qf[s] = (v8i){w[0], w[1], w[2], w[3], 0, 0, 0, 0};
+                sbytes |= (uint32_t)(zero ? 0 : min(max(se + 127, 0), 254)) << (16 * s);
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < SST; ++s) {
+                int w[8];
+#pragma unroll
+                for (int blk = 0; blk < 2; ++blk) {                             // MX block 2s + blk: this lane's 16 of its 32 elements
+                    float x[2][8];
+                    float amax = 0.0f;
+#pragma unroll
+                    for (int c = 0; c < 2; ++c) {
+                        load8<PVT>(row + 2 * (64 * s + 32 * blk + 16 * h + 8 * c), x[c]);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            x[c][e] = x[c][e] * a.q_pre;
+                            amax = __builtin_fmaxf(amax, __builtin_fabsf(x[c][e]));
+                        }
+                    }
+                    amax = max_lane_pair(amax);                                // the other half of the block sits in lane ^ 32
+                    const bool zero = mpsa_f2u(amax) == 0u;
+                    const int se = block_exponent(amax) - 7;                   // emax of the 8-bit formats: ours/quant_mxint8.py:191
+                    const float lim = (FMT8 == MPSA_FMT_E4M3) ? 448.0f : 57344.0f;
+#pragma unroll
+                    for (int c = 0; c < 2; ++c) {
+                        float y[8];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) y[e] = __builtin_fminf(__builtin_fmaxf(ldexpf(x[c][e], -se), -lim), lim);
+                        w[4 * blk + 2 * c] = zero ? 0 : (int)fp8_pack4<FMT8, false>(y[0], y[1], y[2], y[3]);
+                        w[4 * blk + 2 * c + 1] = zero ? 0 : (int)fp8_pack4<FMT8, false>(y[4], y[5], y[6], y[7]);
+                    }
+                    // lane half h hands the matrix core the scale byte of block 2s + h
+                    if (blk == h) sbytes |= (uint32_t)(zero ? 0 : min(max(se + 127, 0), 254)) << (16 * s);
+                }
+                qf[s] = (v8i){w[0], w[1], w[2], w[3], w[4], w[5], w[6], w[7]};
+            }
+        }
+        qsc = (int)sbytes;
+    };
     auto load_q = [&](bool is8) __attribute__((always_inline)) {
+        if constexpr (QRAW) {
+            load_q_raw(is8);
+            return;
+        }
         if (is8) {
 #pragma unroll
             for (int s = 0; s < SST; ++s) {
@@ -117,7 +198,6 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     };
 
     // ---- staging: every wave issues its share of each tile ----
-    const int wu = __builtin_amdgcn_readfirstlane(w);    // the wave index, known to be uniform
     uint32_t koff;                                        // this lane's byte offset into a 4-bit K tile (swizzled rows)
     {
         const int p = w * 64 + lane;
@@ -246,7 +326,8 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                     const float p1 = __builtin_amdgcn_exp2f(st[kb][8 * c + e + 1]);
                     const typename P::v2 pp = P::pack(p0, p1);
                     pk[kb][c][e >> 1] = __builtin_bit_cast(int, pp);
-                    if (e & 2) ps1 = P::add2(pp, ps1); else ps0 = P::add2(pp, ps0);
+                    ps0 += p0;
+                    ps1 += p1;
                 }
         l_run += ps0 + ps1;
         __builtin_amdgcn_s_setprio(2);
@@ -266,58 +347,29 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         }
     };
 
-    // P.V(t) with the softmax of tile t+1 (whose scores are in st) in the gaps between its matrix instructions: after the
-    // four instructions that consume one 16-key group of P(t), that group's registers take the new P(t+1).
-    // The exponentials are taken optimistically, without looking for the tile's maximum first: the running maximum
-    // only has to move when a score exceeds it by more than REBASE, and then the row sum shows it (it exceeds
+    // One pair of exponentials of the coming tile: P = exp2(S - m), rounded to 16 bits for P.V; the row sum adds the
+    // float32 values, as the reference does (ours/mxfp_attn_kernel.py:324-327), with plain additions (the dot-product
+    // instructions share the matrix pipe and stall the P.V stream).
+    auto ex = [&](int g, int j, float& ps0, float& ps1) __attribute__((always_inline)) {
+        const int kb = g >> 1, c = g & 1;
+        const float p0 = __builtin_amdgcn_exp2f(st[kb][8 * c + 2 * j]);
+        const float p1 = __builtin_amdgcn_exp2f(st[kb][8 * c + 2 * j + 1]);
+        const typename P::v2 pp = P::pack(p0, p1);
+        int word = __builtin_bit_cast(int, pp);
+        // pin the conversion here, between the matrix instructions: the redo path overwrites pk, so the compiler
+        // would otherwise sink all 32 conversions behind the check, where nothing overlaps them
+        asm volatile("" : "+v"(word));
+        pk[kb][c][j] = word;
+        ps0 += p0;
+        ps1 += p1;
+    };
+    // The exponentials of tile t+1 were taken optimistically, without looking for the tile's maximum first: the running
+    // maximum only has to move when a score exceeds it by more than REBASE, and then the row sum shows it (it exceeds
     // 2^REBASE or is not finite).  In that rare case the tile is done again the careful way, from its K fragments,
-    // which are still in LDS.
-    auto pv_exp = [&](int t) __attribute__((always_inline)) {
-        constexpr int PRE = 8;
-        const uint8_t* vl = vbuf0 + (t & 1) * V_BYTES + lane * 16;
-        typename P::vec vf[PRE];
-#pragma unroll
-        for (int x = 0; x < PRE; ++x) vf[x] = *reinterpret_cast<const typename P::vec*>(vl + x * 1024);
-        auto mm = [&](int idx) __attribute__((always_inline)) {
-            const int d = idx % NDB, kc = idx / NDB;
-            const typename P::vec cur = vf[idx % PRE];
-            if (idx + PRE < NV) vf[idx % PRE] = *reinterpret_cast<const typename P::vec*>(vl + (idx + PRE) * 1024);
-            acc[d] = P::mfma(cur, __builtin_bit_cast(typename P::vec, pk[kc >> 1][kc & 1]), acc[d]);
-        };
-        float ps0 = 0.0f, ps1 = 0.0f;
-        auto ex = [&](int g, int j) __attribute__((always_inline)) {
-            const int kb = g >> 1, c = g & 1;
-            const float p0 = __builtin_amdgcn_exp2f(st[kb][8 * c + 2 * j]);
-            const float p1 = __builtin_amdgcn_exp2f(st[kb][8 * c + 2 * j + 1]);
-            const typename P::v2 pp = P::pack(p0, p1);
-            pk[kb][c][j] = __builtin_bit_cast(int, pp);
-            if (j & 1) ps1 = P::add2(pp, ps1); else ps0 = P::add2(pp, ps0);
-        };
-        const uint8_t* kl = kbuf0 + ((t + 2) % NKBUF) * K_BYTES;
-        auto kfrag = [&](int kb, int s) __attribute__((always_inline)) {
-            const int krow = 32 * kb + r;
-            const int f = (krow >> SH4) & (CPR4 - 1);
-            kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * ROW4 + (((2 * s + h) ^ f) * 16));
-        };
-#pragma unroll
-        for (int kc = 0; kc < 2 * KB; ++kc)
-#pragma unroll
-            for (int d = 0; d < NDB; ++d) {
-                mm(kc * NDB + d);
-                if (kc > 0) ex(kc - 1, d);
-                if (kc >= KB && d < SST) kfrag(kc - KB, d);   // K fragments of tile t+2 (the score MFMAs are long gone)
-                if (kc > 0) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-                }
-            }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) ex(2 * KB - 1, j);
+    // which are still in LDS: scores again, maximum, rebase (P.V(t) is through, the accumulators can be rescaled now).
+    auto finish_tile = [&](int t, float ps0, float ps1) __attribute__((always_inline)) {
         float tot = ps0 + ps1;
         if (__any(!(tot < P::OPTIMISTIC_LIMIT))) {
-            // the careful way: scores again, maximum, rebase (P.V(t) is through, the accumulators can be rescaled now)
             prep_plain(t + 1);
             s_plain();
             float mx = st[0][0];
@@ -343,12 +395,52 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) st[g >> 1][8 * (g & 1) + e] -= delta;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) ex(g, j);
+                for (int j = 0; j < 4; ++j) ex(g, j, ps0, ps1);
             }
             tot = ps0 + ps1;
             prep_plain(t + 2);                             // back to the operands of the next step
         }
         l_run += tot;
+    };
+
+    // P.V(t) with the softmax of tile t+1 (whose scores are in st) in the gaps between its matrix instructions: after the
+    // four instructions that consume one 16-key group of P(t), that group's registers take the new P(t+1).
+    auto pv_exp = [&](int t) __attribute__((always_inline)) {
+        constexpr int PRE = 8;
+        const uint8_t* vl = vbuf0 + (t & 1) * V_BYTES + lane * 16;
+        typename P::vec vf[PRE];
+#pragma unroll
+        for (int x = 0; x < PRE; ++x) vf[x] = *reinterpret_cast<const typename P::vec*>(vl + x * 1024);
+        auto mm = [&](int idx) __attribute__((always_inline)) {
+            const int d = idx % NDB, kc = idx / NDB;
+            const typename P::vec cur = vf[idx % PRE];
+            if (idx + PRE < NV) vf[idx % PRE] = *reinterpret_cast<const typename P::vec*>(vl + (idx + PRE) * 1024);
+            acc[d] = P::mfma(cur, __builtin_bit_cast(typename P::vec, pk[kc >> 1][kc & 1]), acc[d]);
+        };
+        float ps0 = 0.0f, ps1 = 0.0f;
+        const uint8_t* kl = kbuf0 + ((t + 2) % NKBUF) * K_BYTES;
+        auto kfrag = [&](int kb, int s) __attribute__((always_inline)) {
+            const int krow = 32 * kb + r;
+            const int f = (krow >> SH4) & (CPR4 - 1);
+            kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * ROW4 + (((2 * s + h) ^ f) * 16));
+        };
+#pragma unroll
+        for (int kc = 0; kc < 2 * KB; ++kc)
+#pragma unroll
+            for (int d = 0; d < NDB; ++d) {
+                mm(kc * NDB + d);
+                if (kc > 0) ex(kc - 1, d, ps0, ps1);
+                if (kc >= KB && d < SST) kfrag(kc - KB, d);   // K fragments of tile t+2 (the score MFMAs are long gone)
+                if (kc > 0) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                }
+            }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ex(2 * KB - 1, j, ps0, ps1);
+        finish_tile(t, ps0, ps1);
     };
 
     // ---- prologue (all waves): V(0), K(0..2) on their way; Q into registers ----
@@ -451,27 +543,27 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         }
 }
 
-template <int PVT, int FMT8, int MODE>
+template <int PVT, int FMT8, int MODE, bool QRAW>
 struct PpLds {
-    static inline const bool registered = mpsa_register_lds_kernel(reinterpret_cast<const void*>(attn_pp_kernel<PVT, FMT8, MODE>), SMEM);
+    static inline const bool registered = mpsa_register_lds_kernel(reinterpret_cast<const void*>(attn_pp_kernel<PVT, FMT8, MODE, QRAW>), SMEM);
 };
 
-template <int PVT, int FMT8, int MODE>
+template <int PVT, int FMT8, int MODE, bool QRAW>
 int launch_pp(const AttnArgs& a, hipStream_t st) {
-    if (!PpLds<PVT, FMT8, MODE>::registered) return mpsa_fail(MPSA_ELAUNCH, "attn: kernel not registered");
+    if (!PpLds<PVT, FMT8, MODE, QRAW>::registered) return mpsa_fail(MPSA_ELAUNCH, "attn: kernel not registered");
     const int rc = mpsa_ensure_init();
     if (rc != MPSA_OK) return rc;
     dim3 grid((unsigned)(a.B * a.Hq * (a.nt / 2)));
-    hipLaunchKernelGGL((attn_pp_kernel<PVT, FMT8, MODE>), grid, dim3(512), SMEM, st, a);
+    hipLaunchKernelGGL((attn_pp_kernel<PVT, FMT8, MODE, QRAW>), grid, dim3(512), SMEM, st, a);
     MPSA_CHECK_LAUNCH("attn(pp)");
     return MPSA_OK;
 }
 
-template <int PVT>
+template <int PVT, bool QRAW>
 int launch_pp_mode(const AttnArgs& a, hipStream_t st) {
-    if (a.mode == MPSA_MODE_MXFP4) return launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP4>(a, st);
-    return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_DIAG>(a, st)
-                                   : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_DIAG>(a, st);
+    if (a.mode == MPSA_MODE_MXFP4) return launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP4, QRAW>(a, st);
+    return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_DIAG, QRAW>(a, st)
+                                   : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_DIAG, QRAW>(a, st);
 }
 
 }  // namespace
@@ -489,6 +581,10 @@ bool attn_pp_supported(const AttnArgs& a, int pv_dtype) {
 }
 
 int attn_pp_launch(const AttnArgs& a, int pv_dtype, hipStream_t st) {
-    if (pv_dtype == MPSA_BF16) return launch_pp_mode<MPSA_BF16>(a, st);
-    return launch_pp_mode<MPSA_F16>(a, st);
+    if (a.q_raw) {
+        if (pv_dtype == MPSA_BF16) return launch_pp_mode<MPSA_BF16, true>(a, st);
+        return launch_pp_mode<MPSA_F16, true>(a, st);
+    }
+    if (pv_dtype == MPSA_BF16) return launch_pp_mode<MPSA_BF16, false>(a, st);
+    return launch_pp_mode<MPSA_F16, false>(a, st);
 }

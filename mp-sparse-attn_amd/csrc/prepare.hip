@@ -79,7 +79,7 @@ extern "C" int mpsa_attn_prepare(const void* q, const int64_t q_strides[4], cons
     const bool do4 = mode != MPSA_MODE_MXFP8, do8 = mode != MPSA_MODE_MXFP4;
     const int64_t nq_pad = (Nq + tile - 1) / tile * tile, nk_pad = (Nk + tile - 1) / tile * tile;
     constexpr int EMAX4 = 3, EMAX8 = 7;            // ours/quant_mxint8.py:303, :191
-    if (mpsa_quantize_sw_encoders()) {
+    if (mpsa_quantize_sw_encoders() && q) {
         // the cross-checking encoders exist only as stand-alone kernels
         int rc = do4 && do8 ? mpsa_quantize_mx_dual(q, dtype, B, Hq, Nq, D, q_strides, nullptr, pre_scale_q, EMAX4, fmt8, EMAX8, q4, qs4, q8, qs8, nq_pad, stream)
                             : mpsa_quantize_mx(q, dtype, B, Hq, Nq, D, q_strides, nullptr, pre_scale_q, do4 ? MPSA_FMT_E2M1 : fmt8, do4 ? EMAX4 : EMAX8, do4 ? q4 : q8, do4 ? qs4 : qs8, nq_pad, stream);
@@ -91,8 +91,13 @@ extern "C" int mpsa_attn_prepare(const void* q, const int64_t q_strides[4], cons
     }
     PrepArgs p;
     unsigned bq = 0, bk = 0, bv = 0;
-    int rc = mpsa_quantize_setup(q, dtype, B, Hq, Nq, D, q_strides, nullptr, pre_scale_q, do4, EMAX4, do8, fmt8, EMAX8, q4, qs4, q8, qs8, nq_pad, &p.q, &bq);
-    if (rc != MPSA_OK) return rc;
+    int rc = MPSA_OK;
+    if (q) {
+        rc = mpsa_quantize_setup(q, dtype, B, Hq, Nq, D, q_strides, nullptr, pre_scale_q, do4, EMAX4, do8, fmt8, EMAX8, q4, qs4, q8, qs8, nq_pad, &p.q, &bq);
+        if (rc != MPSA_OK) return rc;
+    } else {
+        p.q = QuantArgs{};                       // no Q job: the attention kernel quantizes Q itself (mpsa_attn_fwd_q16)
+    }
     rc = mpsa_quantize_setup(k, dtype, B, Hkv, Nk, D, k_strides, k_sub, 1.0f, do4, EMAX4, do8, fmt8, EMAX8, k4, ks4, k8, ks8, nk_pad, &p.k, &bk);
     if (rc != MPSA_OK) return rc;
     rc = mpsa_v_tiles_setup(v, dtype, B, Hkv, Nk, D, v_strides, tile, v_tiles, &p.v, &bv);

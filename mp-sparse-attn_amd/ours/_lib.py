@@ -48,6 +48,9 @@ SIGNATURES = {
                                  _f32, _vp] + [_vp] * 9 + [_vp]),
     "mpsa_attn_fwd": (_int, [_vp] * 8 + [_int, _vp, _int, _vp, _int, _p64,
                              _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
+    "mpsa_attn_fwd_q16": (_int, [_vp, _p64, _int, _f32] + [_vp] * 4 + [_int, _vp, _int, _vp, _int, _p64,
+                                 _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
+    "mpsa_attn_fwd_q16_supported": (_int, [_i64, _i64, _i64, _i64, _i64, _int, _int, _int]),
     "mpsa_attn_fwd_skip": (_int, [_vp] * 8 + [_int, _vp, _int, _vp, _int, _p64,
                                   _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _vp, _vp]),
     "mpsa_route_workspace": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),

@@ -17,11 +17,23 @@ _MODES = {"mxfp4": _lib.MODE_MXFP4, "mxfp8": _lib.MODE_MXFP8, "mxfp8e5": _lib.MO
           "mixed": _lib.MODE_MIXED, "mixed_e5": _lib.MODE_MIXED}
 
 
-def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False, reuse=None):
+def q_fusable(q, k, tile, block_scale_type, is_causal):
+    """True when the attention kernel can take this Q unquantized and quantize it itself (``mpsa_attn_fwd_q16``: the
+    paired-tile kernel's shapes -- causal, D = 128, tile = 128, whole pairs of tiles, diag / mxfp4 types)."""
+    mode = _MODES.get(block_scale_type)
+    if mode not in (_lib.MODE_DIAG, _lib.MODE_MXFP4) or q.shape[2] != k.shape[2]:
+        return False
+    B, Hq, N, D = q.shape
+    return bool(_lib.lib().mpsa_attn_fwd_q16_supported(B, Hq, k.shape[1], N, D, tile, 1 if is_causal else 0, mode))
+
+
+def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False, reuse=None, fuse_q=False):
     """Quantize Q/K (K minus its mean over the sequence if ``smooth_k``) and repack V for one attention call.
     q ``[B,Hq,Nq,D]``, k/v ``[B,Hkv,Nk,D]`` of one 16-bit dtype.  Returns a dict of device tensors (rows padded to
     whole tiles) the launcher consumes.  ``reuse``: the dict a previous call returned for the same shapes, dtype, tile
-    and type -- its buffers are written again instead of allocating new ones (a serving loop's steady state)."""
+    and type -- its buffers are written again instead of allocating new ones (a serving loop's steady state).
+    ``fuse_q`` (only where :func:`q_fusable` says so): Q is left unquantized for ``mpsa_attn_fwd_q16``; only K and V are
+    prepared."""
     if block_scale_type not in _MODES:
         raise ValueError(f"Invalid block scale type: {block_scale_type}")
     mode = _MODES[block_scale_type]
@@ -32,7 +44,7 @@ def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False
     n_pad = nt * tile
     nq_pad = (Nq + tile - 1) // tile * tile
     pre = pre_scale_q(D, scale)
-    key = (mode, fmt8, tile, tuple(q.shape), tuple(k.shape), q.dtype, v.dtype, q.device)
+    key = (mode, fmt8, tile, tuple(q.shape), tuple(k.shape), q.dtype, v.dtype, q.device, bool(fuse_q))
     # smooth-K (ours/mxfp_attn_kernel.py:33-34): the mean over the sequence is subtracted inside the K quantizer
     kmean = seq_mean(k) if smooth_k else None
     q, k = _check_input(q), _check_input(k)
@@ -46,21 +58,24 @@ def prepare_operands(q, k, v, tile, block_scale_type, scale=None, smooth_k=False
         need4, need8 = mode != _lib.MODE_MXFP8, mode != _lib.MODE_MXFP4
         u8 = lambda *shape: torch.empty(shape, dtype=torch.uint8, device=dev)
         if need4:
-            ops["q4"], ops["qs4"] = u8(B, Hq, nq_pad, D // 2), u8(B, Hq, nq_pad, D // 32)
+            if not fuse_q:
+                ops["q4"], ops["qs4"] = u8(B, Hq, nq_pad, D // 2), u8(B, Hq, nq_pad, D // 32)
             ops["k4"], ops["ks4"] = u8(B, Hkv, n_pad, D // 2), u8(B, Hkv, n_pad, D // 32)
         if need8:
-            ops["q8"], ops["qs8"] = u8(B, Hq, nq_pad, D), u8(B, Hq, nq_pad, D // 32)
+            if not fuse_q:
+                ops["q8"], ops["qs8"] = u8(B, Hq, nq_pad, D), u8(B, Hq, nq_pad, D // 32)
             ops["k8"], ops["ks8"] = u8(B, Hkv, n_pad, D), u8(B, Hkv, n_pad, D // 32)
         v_tiles = torch.empty((B, Hkv, nt, tile * D), dtype=v.dtype, device=v.device)
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().mpsa_attn_prepare(
-            _lib.ptr(q), _lib.strides4(q), _lib.ptr(k), _lib.strides4(k), _lib.ptr(v), _lib.strides4(v),
+            _lib.ptr(None if fuse_q else q), _lib.strides4(q), _lib.ptr(k), _lib.strides4(k), _lib.ptr(v), _lib.strides4(v),
             _lib.dtype_id(q.dtype), B, Hq, Hkv, Nq, N, D, tile, mode, fmt8, pre, _lib.ptr(kmean),
             _lib.ptr(ops["q4"]), _lib.ptr(ops["qs4"]), _lib.ptr(ops["q8"]), _lib.ptr(ops["qs8"]),
             _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]), _lib.ptr(ops["ks8"]),
             _lib.ptr(v_tiles), _lib.stream_ptr(dev)))
     ops["v_tiles"] = v_tiles
     ops["shape"] = (B, Hq, Hkv, Nq, N, D)
+    ops["q_raw"], ops["pre"] = (q, pre) if fuse_q else (None, pre)
     return ops
 
 
@@ -104,6 +119,17 @@ def attention_from_operands(ops, out, is_causal, skip_thresh=None, skipped=None,
                 _lib.ptr(ops["v_tiles"]), _lib.dtype_id(ops["v_tiles"].dtype), _lib.ptr(out), _lib.dtype_id(out.dtype),
                 _lib.strides4(out), B, Hq, Hkv, Nq, N, D, ops["tile"], 1 if is_causal else 0,
                 _lib.ptr(order), _lib.ptr(counts), _lib.stream_ptr(dev)))
+        return out
+    if ops.get("q_raw") is not None:
+        if skip_thresh is not None:
+            raise ValueError("tile skipping needs quantized Q operands (prepare_operands without fuse_q)")
+        q = ops["q_raw"]
+        with torch.cuda.device(dev):
+            _lib.check(_lib.lib().mpsa_attn_fwd_q16(
+                _lib.ptr(q), _lib.strides4(q), _lib.dtype_id(q.dtype), ops["pre"],
+                _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]), _lib.ptr(ops["ks8"]), ops["fmt8"],
+                _lib.ptr(ops["v_tiles"]), _lib.dtype_id(ops["v_tiles"].dtype), _lib.ptr(out), _lib.dtype_id(out.dtype),
+                _lib.strides4(out), B, Hq, Hkv, N, D, ops["tile"], 1 if is_causal else 0, ops["mode"], _lib.stream_ptr(dev)))
         return out
     if skip_thresh is not None:
         with torch.cuda.device(dev):
@@ -266,7 +292,9 @@ def mxfp_attn_kernel(q, k, v, attn_mask=None, dropout_p=0.0,
         raise ValueError(f"Unsupported dtype: {output_dtype}")       # ours/mxfp_attn_kernel.py:389
     if v.stride(-1) != 1:
         v = v.contiguous()
-    ops = prepare_operands(q, k, v, tile, block_scale_type, scale, smooth_k=smooth_k)
+    # shapes of the paired-tile kernel: Q stays unquantized in HBM and the attention kernel quantizes it in registers
+    fuse_q = skip_thresh is None and q.stride(-1) == 1 and q.dtype == v.dtype and q_fusable(q, k, tile, block_scale_type, is_causal)
+    ops = prepare_operands(q, k, v, tile, block_scale_type, scale, smooth_k=smooth_k, fuse_q=fuse_q)
     nt, ntk = (N + tile - 1) // tile, (Nk + tile - 1) // tile       # query tiles, key tiles
     skipped = None
     routed = ops["mode"] == _lib.MODE_ROUTED

@@ -442,3 +442,54 @@ def test_reference_call_sequence_quantize_package_attend(bst):
         initialize_block_scaled_batched_from_tensor(a_quant, b_quant, a_scale, b_scale, block_scale_type=bst, compute_reference=True)
     with pytest.raises(ValueError, match="Unsupported dtype"):
         block_scaled_batched_attn(a_packed, a_scale, b_packed, b_scale, v.to(DEV), torch.float8_e5m2, B, H, M, N, K, configs)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("bst", ["diag", "mxfp4", "diag_e5"])
+@pytest.mark.parametrize("N,scale", [(256, None), (1024, 0.07), (1536, None)])
+def test_q_quantized_inside_the_attention_kernel_gives_the_same_bits(bst, N, scale, dtype):
+    """mpsa_attn_fwd_q16 (Q handed over unquantized, MX-quantized in registers by the paired-tile kernel) against
+    mpsa_attn_prepare + mpsa_attn_fwd on the same inputs: the quantizer's own device functions run in both, so every
+    output bit is equal -- with outlier channels, a non-default scale, grouped heads, and a q that is a strided view."""
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, q_fusable
+    q, k, v = make_qkv(2, 8, 2, N, 128, seed=600 + N, dtype=dtype, outliers=True)
+    q[0, 0, :40] = 0                                              # all-zero MX blocks: scale byte 0, codes +0
+    q[1, 3, 5, 32:64] = 0
+    qd = q.to(DEV).transpose(1, 2).contiguous().transpose(1, 2)   # [B,H,N,D] view of an [B,N,H,D] tensor
+    kd, vd = k.to(DEV), v.to(DEV)
+    assert not qd.is_contiguous() and q_fusable(qd, kd, 128, bst, True)
+    assert not q_fusable(qd, kd, 128, bst, False) and not q_fusable(qd, kd, 64, bst, True) and not q_fusable(qd, kd, 128, "mxfp8", True)
+    a = torch.empty((2, 8, N, 128), dtype=dtype, device=DEV)
+    b = torch.empty_like(a)
+    attention_from_operands(prepare_operands(qd, kd, vd, 128, bst, scale), a, True)
+    fused = prepare_operands(qd, kd, vd, 128, bst, scale, fuse_q=True)
+    assert fused["q4"] is None and fused["q8"] is None
+    attention_from_operands(fused, b, True)
+    assert torch.equal(a, b)
+    # and the public entry point takes the fused route by itself
+    c = mxfp_attn_kernel(qd, kd, vd, is_causal=True, scale=scale, block_scale_type=bst, output_dtype=dtype)
+    assert torch.equal(a, c)
+    want = O.attn_mx(q, k, v, tile=128, causal=True, mode="diag" if bst.startswith("diag") else "mxfp4", scale=scale,
+                     fmt8=O.FMT_E5M2 if bst.endswith("e5") else O.FMT_E4M3, out_dtype=torch.float32)
+    _compare(mxfp_attn_kernel(qd, kd, vd, is_causal=True, scale=scale, block_scale_type=bst, output_dtype=torch.float32), want, f"fused q {bst} N={N}")
+
+
+def test_q16_entry_point_rejects_other_shapes():
+    L = _lib.lib()
+    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 128, 128, 1, _lib.MODE_DIAG) == 1
+    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 128, 128, 0, _lib.MODE_DIAG) == 0      # not causal
+    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192 + 128, 128, 128, 1, _lib.MODE_DIAG) == 0  # an odd number of tiles
+    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 64, 128, 1, _lib.MODE_DIAG) == 0
+    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 128, 128, 1, _lib.MODE_MXFP8) == 0
+    q, k, v = (t.to(DEV) for t in make_qkv(1, 2, 2, 384, 128, seed=9))
+    from ours.mxfp_attn_kernel import prepare_operands
+    ops = prepare_operands(q, k, v, 128, "diag")
+    out = torch.empty((1, 2, 384, 128), dtype=torch.bfloat16, device=DEV)
+    rc = L.mpsa_attn_fwd_q16(_lib.ptr(q), _lib.strides4(q), _lib.BF16, 0.1275, _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]),
+                             _lib.ptr(ops["ks8"]), 0, _lib.ptr(ops["v_tiles"]), _lib.BF16, _lib.ptr(out), _lib.BF16, _lib.strides4(out),
+                             1, 2, 2, 384, 128, 128, 1, _lib.MODE_DIAG, _lib.stream_ptr())
+    assert rc == -3 and b"paired-tile" in L.mpsa_last_error()
+    rc = L.mpsa_attn_fwd_q16(_lib.ptr(q), _lib.strides4(q), _lib.F16, 0.1275, _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]),
+                             _lib.ptr(ops["ks8"]), 0, _lib.ptr(ops["v_tiles"]), _lib.BF16, _lib.ptr(out), _lib.BF16, _lib.strides4(out),
+                             1, 2, 2, 512, 128, 128, 1, _lib.MODE_DIAG, _lib.stream_ptr())
+    assert rc == -1 and b"dtype" in L.mpsa_last_error()
