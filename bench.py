@@ -230,12 +230,36 @@ def secondary(device, quick):
     return out
 
 
+def mfma_stream_rates(device, seconds=0.05):
+    """Sustained rate of a register-resident matrix-instruction stream (two waves per SIMD, every CU): constant
+    operands and operands with random bits, for the bf16, MXFP4 and MXFP8 instructions the path uses."""
+    import ctypes
+    from ours import _lib
+    L = _lib.lib()
+    sink = torch.zeros(4, dtype=torch.float32, device=device)
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    out = {}
+    for name, kind, peak in (("bf16", 0, PEAK_BF16_TFLOPS), ("mxfp4", 1, PEAK_FP4_TFLOPS), ("mxfp8", 2, PEAK_FP8_TFLOPS)):
+        for label, rnd in (("constant", 0), ("random", 1)):
+            flop = ctypes.c_double(0.0)
+            run = lambda n: _lib.check(L.mpsa_bench_mfma_stream(kind, rnd, n, cus, _lib.ptr(sink), ctypes.byref(flop), _lib.stream_ptr(device)))
+            ms = time_events(lambda: run(2000), 2)
+            iters = max(2000, int(2000 * seconds * 1e3 / max(ms, 1e-3)))
+            ms = time_events(lambda: run(iters), 3)
+            tf = flop.value / ms / 1e9
+            out[f"{name}_{label}"] = {"TFLOP/s": round(tf, 1), "frac_peak": round(tf / peak, 4)}
+    return out
+
+
 def run_only(args, device):
     """Launch one kernel repeatedly (for rocprofv3 --pmc / --kernel-trace runs)."""
     from ours import _lib
     from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, route_tiles
     from ours.quant_mxint8 import quantize_mx, quantize_mx_dual
     from ours.block_scaled_matmul import block_scaled_matmul, make_configs, pack_scale_5d
+    if args.only == "mfma":
+        print(json.dumps({"kernel": "matrix-instruction stream", "rates": mfma_stream_rates(device, 0.2)}))
+        return
     if args.only == "copy":
         src = torch.ones(1 << 29, dtype=torch.bfloat16, device=device)          # 1 GiB
         dst = torch.empty_like(src)
@@ -295,7 +319,7 @@ def main():
     ap.add_argument("--eager", action="store_true", help="time plain launches instead of replaying the step as a HIP graph")
     ap.add_argument("--linear-scales", action="store_true",
                     help="with --only gemm4/gemm8: row-major [rows, K/32] scales instead of the reference's packed form")
-    ap.add_argument("--only", default=None, choices=["attn", "copy", "quant", "gemm4", "gemm8"],
+    ap.add_argument("--only", default=None, choices=["attn", "copy", "quant", "gemm4", "gemm8", "mfma"],
                     help="profiling aid: launch just this kernel --steps times and exit (copy = 1 GiB torch copy, "
                          "the calibration kernel for HBM counters)")
     args = ap.parse_args()
@@ -422,6 +446,15 @@ def main():
     }
     if second is not None:
         result["secondary"] = second
+        # what the matrix cores sustain on this chip (its clock is managed by power: operands with random bits run the
+        # same instruction stream several hundred MHz lower than constants do), and the composite bound at those rates
+        rates = mfma_stream_rates(device)
+        second["mfma_stream"] = rates
+        diag = 2.0 / (nt + 1) if causal else 1.0 / nt
+        sustained = 1.0 / (0.5 * ((1 - diag) / rates["mxfp4_random"]["TFLOP/s"] + diag / rates["mxfp8_random"]["TFLOP/s"]) +
+                           0.5 / rates["bf16_random"]["TFLOP/s"])
+        roofline["sustained_composite"] = round(sustained, 1)
+        roofline["frac_sustained_composite"] = round(achieved / sustained, 5)
         if args.workload == "c3" and args.mode == "diag" and not args.no_c4:
             del ops, route
             state.clear()

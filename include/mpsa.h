@@ -342,6 +342,16 @@ int mpsa_attn_fwd_routed(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q
                          int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t nk, int64_t D, int tile, int causal,
                          const int32_t* order, const int32_t* counts, mpsa_stream_t stream);
 
+/*
+ * Measurement aid (no counterpart in the reference): a register-resident stream of matrix instructions, two waves per
+ * SIMD, `blocks` workgroups, iters x 16 instructions per wave.  kind 0: v_mfma_f32_32x32x16_bf16; 1:
+ * v_mfma_scale_f32_32x32x64_f8f6f4 on E2M1 operands; 2: the same on E4M3 operands.  random_bits != 0 fills the operand
+ * registers with pseudo-random bits instead of one constant: the chip's power management then runs the same stream at
+ * a lower clock, which is the rate a real matmul can at best sustain.  *flop receives the launch's FLOP count; time it
+ * with events on `stream`.  sink: any 4 writable device bytes.
+ */
+int mpsa_bench_mfma_stream(int kind, int random_bits, int iters, int blocks, float* sink, double* flop, mpsa_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libmpsa.so")
 
-SOURCES = ["api.hip", "formats.hip", "quantize.hip", "v_tiles.hip", "prepare.hip", "gemm_mx.hip", "attn_fwd.hip", "attn_fwd_skip.hip", "attn_fwd_routed.hip", "attn_fwd_pp.hip", "route.hip"]
+SOURCES = ["api.hip", "formats.hip", "quantize.hip", "v_tiles.hip", "prepare.hip", "gemm_mx.hip", "attn_fwd.hip", "attn_fwd_skip.hip", "attn_fwd_routed.hip", "attn_fwd_pp.hip", "route.hip", "mfma_stream.hip"]
 
 # packed-fp32 instructions are switched off on purpose (the flag is for the device pass; the host
 # pass warns that it does not know the feature, which is harmless)

@@ -401,7 +401,10 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
                     const float p1 = __builtin_amdgcn_exp2f(st[kb][8 * c + e + 1]);
                     const typename P::v2 pp = P::pack(p0, p1);
                     pk[kb][c][e >> 1] = __builtin_bit_cast(int, pp);
-                    if (e & 2) ps1 = P::add2(pp, ps1); else ps0 = P::add2(pp, ps0);
+                    // float32 additions (ours/mxfp_attn_kernel.py:324-327 sums P before the down-cast); the
+                    // dot-product instructions share the matrix pipe and stall the other waves' matrix work
+                    ps0 += p0;
+                    ps1 += p1;
                 }
         l_run += ps0 + ps1;
         }

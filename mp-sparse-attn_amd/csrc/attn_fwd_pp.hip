@@ -34,6 +34,8 @@ constexpr int CPR4 = ROW4 / 16, SH4 = 2;
 constexpr int K_BYTES = TILE * ROW4, V_BYTES = TILE * D * 2;
 constexpr int NKBUF = 3;                        // K tiles in LDS: one being multiplied, two ahead
 constexpr int SMEM = NKBUF * K_BYTES + 2 * V_BYTES;
+constexpr int Q8_BYTES = 512 * 64;              // fused-quantizer variants: every lane's 8-bit Q fragments (64 bytes), parked until the diagonal tile
+constexpr int SMEM_QRAW = SMEM + Q8_BYTES;
 constexpr int NWAVES = 8;
 constexpr int VI = V_BYTES / 1024 / NWAVES;     // direct-load instructions per wave for one V tile (4)
 constexpr int NV = KB * 2 * NDB;                // P.V matrix instructions per tile (32)
@@ -82,6 +84,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     // ---- operands in registers ----
     v8i qf[SST];
     int qsc = 0;
+    int qsc8 = 0;                                // fused-quantizer variants: scale bytes of the parked 8-bit Q fragments
     v4i kf4[KB][SST];
     int ksc[KB];
     // shared exponent of an MX block from its largest magnitude, as the quantizer takes it (quantize_kernel.h)
@@ -139,12 +142,13 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                     amax = max_lane_pair(amax);                                // the other half of the block sits in lane ^ 32
                     const bool zero = mpsa_f2u(amax) == 0u;
                     const int se = block_exponent(amax) - 7;                   // emax of the 8-bit formats: ours/quant_mxint8.py:191
-                    const float lim = (FMT8 == MPSA_FMT_E4M3) ? 448.0f : 57344.0f;
+                    // (the quantizer clamps to the format's maximum here; with the block maximum scaled into
+                    // [128, 256) that clamp never changes a value, so it is left out)
 #pragma unroll
                     for (int c = 0; c < 2; ++c) {
                         float y[8];
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) y[e] = __builtin_fminf(__builtin_fmaxf(ldexpf(x[c][e], -se), -lim), lim);
+                        for (int e = 0; e < 8; ++e) y[e] = ldexpf(x[c][e], -se);
                         w[4 * blk + 2 * c] = zero ? 0 : (int)fp8_pack4<FMT8, false>(y[0], y[1], y[2], y[3]);
                         w[4 * blk + 2 * c + 1] = zero ? 0 : (int)fp8_pack4<FMT8, false>(y[4], y[5], y[6], y[7]);
                     }
@@ -250,7 +254,18 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     auto prep_special = [&](int t) __attribute__((always_inline)) {      // this wave's diagonal tile
         if constexpr (MODE == MPSA_MODE_DIAG) {
             load_kscales(t, true);
-            load_q(true);
+            if constexpr (QRAW) {
+                const uint8_t* park = smem + SMEM + tid * 16;
+#pragma unroll
+                for (int s = 0; s < SST; ++s) {
+                    const v4i x0 = *reinterpret_cast<const v4i*>(park + (2 * s) * 8192);
+                    const v4i x1 = *reinterpret_cast<const v4i*>(park + (2 * s + 1) * 8192);
+                    qf[s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+                }
+                qsc = qsc8;
+            } else {
+                load_q(true);
+            }
         } else {
             prep_plain(t);
         }
@@ -448,6 +463,19 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     issue_k4(0);
     issue_k4(1);
     if (nsteps > 2) issue_k4(2);
+    if constexpr (QRAW && MODE == MPSA_MODE_DIAG) {
+        // The diagonal tile's 8-bit Q is quantized now, while the first K/V tiles are on their way, and parked in LDS
+        // (each lane reads back only what it wrote itself): at the diagonal tile the loads and the conversion would
+        // sit on the wave's critical path.
+        load_q(true);
+        qsc8 = qsc;
+        uint8_t* park = smem + SMEM + tid * 16;
+#pragma unroll
+        for (int s = 0; s < SST; ++s) {
+            *reinterpret_cast<v4i*>(park + (2 * s) * 8192) = (v4i){qf[s][0], qf[s][1], qf[s][2], qf[s][3]};
+            *reinterpret_cast<v4i*>(park + (2 * s + 1) * 8192) = (v4i){qf[s][4], qf[s][5], qf[s][6], qf[s][7]};
+        }
+    }
     load_q(false);
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
@@ -545,7 +573,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
 
 template <int PVT, int FMT8, int MODE, bool QRAW>
 struct PpLds {
-    static inline const bool registered = mpsa_register_lds_kernel(reinterpret_cast<const void*>(attn_pp_kernel<PVT, FMT8, MODE, QRAW>), SMEM);
+    static inline const bool registered = mpsa_register_lds_kernel(reinterpret_cast<const void*>(attn_pp_kernel<PVT, FMT8, MODE, QRAW>), QRAW ? SMEM_QRAW : SMEM);
 };
 
 template <int PVT, int FMT8, int MODE, bool QRAW>
@@ -554,7 +582,7 @@ int launch_pp(const AttnArgs& a, hipStream_t st) {
     const int rc = mpsa_ensure_init();
     if (rc != MPSA_OK) return rc;
     dim3 grid((unsigned)(a.B * a.Hq * (a.nt / 2)));
-    hipLaunchKernelGGL((attn_pp_kernel<PVT, FMT8, MODE, QRAW>), grid, dim3(512), SMEM, st, a);
+    hipLaunchKernelGGL((attn_pp_kernel<PVT, FMT8, MODE, QRAW>), grid, dim3(512), QRAW ? SMEM_QRAW : SMEM, st, a);
     MPSA_CHECK_LAUNCH("attn(pp)");
     return MPSA_OK;
 }

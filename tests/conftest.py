@@ -38,3 +38,26 @@ def make_qkv(B, Hq, Hkv, N, D, seed, dtype=torch.bfloat16, sigma=1.0, outliers=F
                 idx = torch.randint(0, D, (n_out,), generator=g)
                 t[:, h, :, idx] *= 20.0
     return q.to(dtype), k.to(dtype), v.to(dtype)
+
+
+COS_MIN, MAXABS_MAX = 0.999, 2e-2
+
+
+def attention_close(got, want, what=""):
+    """The acceptance bar of the attention path: cosine >= 0.999 over the flattened tensors and max-abs error <= 2e-2.
+    The bar is a bar on the arithmetic.  A 16-bit OUTPUT adds its own rounding: two float32 results 1e-3 apart can fall
+    on different sides of a rounding boundary, and for an output of magnitude 4 or more one bf16 step is 2^-5 = 0.031.
+    So each side that is a 16-bit tensor gets half a unit in its last place, at the oracle value's magnitude, on top
+    of the 2e-2; float32 tensors get nothing."""
+    import oracle as O
+    g, w = got.detach().cpu(), want.detach().cpu()
+    m = O.precision_metric(g, w)
+    wd = w.double()
+    allow = torch.full_like(wd, MAXABS_MAX)
+    for t in (g, w):
+        bits = {torch.bfloat16: 8, torch.float16: 11}.get(t.dtype)
+        if bits is not None:
+            allow = allow + torch.exp2(torch.floor(torch.log2(wd.abs().clamp_min(2.0 ** -24))) - bits)
+    err = (g.double() - wd).abs()
+    assert m["cos"] >= COS_MIN and bool((err <= allow).all()), f"{what}: {m}, worst excess {(err - allow).max().item():.4g}"
+    return m

@@ -8,33 +8,25 @@ import pytest
 import torch
 
 import oracle as O
-from conftest import make_qkv
+from conftest import make_qkv, attention_close
 from ours import _lib
 from ours.mxfp_attn import mxfp_attn
 from ours.mxfp_attn_kernel import mxfp_attn_kernel
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
-COS_MIN, MAXABS_MAX = 0.999, 2e-2
 
 
 def _compare(got, want, what=""):
-    m = O.precision_metric(got.cpu(), want)
-    assert m["cos"] >= COS_MIN and m["max_abs"] <= MAXABS_MAX, f"{what}: {m}"
-    return m
+    return attention_close(got, want, what)
 
 
 def _compare_16bit(got16, got32, want32, what=""):
-    """A 16-bit output against the oracle.  The 2e-2 bar is a bar on the arithmetic, checked on the float32 outputs;
-    rounding an output of magnitude 4 or more to bf16 can by itself move it by 2^-5 = 0.031 when the two float32
-    values straddle a rounding boundary, so the 16-bit output is checked as what it is: the kernel's own float32
-    result rounded once (bit for bit), hence within the bar plus half a 16-bit unit of the oracle."""
+    """A 16-bit output against the oracle: the bar on the float32 outputs, and the 16-bit output as what it is -- the
+    kernel's own float32 result rounded once, bit for bit (conftest.attention_close gives that rounding its half unit)."""
     m = _compare(got32, want32, what + " (float32 outputs)")
     assert torch.equal(got16.cpu(), got32.cpu().to(got16.dtype)), f"{what}: the 16-bit output is not the rounded float32 output"
-    w = want32.double()
-    half_ulp = torch.exp2(torch.floor(torch.log2(w.abs().clamp_min(1e-30))) - (8 if got16.dtype == torch.bfloat16 else 11))
-    err = (got16.cpu().double() - w).abs()
-    assert (err <= MAXABS_MAX + half_ulp).all(), f"{what}: 16-bit output off by {(err - half_ulp).max().item():.4f} beyond rounding"
+    _compare(got16, want32, what + " (16-bit output)")
     return m
 
 

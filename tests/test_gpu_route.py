@@ -8,14 +8,13 @@ import pytest
 import torch
 
 import oracle as O
-from conftest import make_qkv
+from conftest import make_qkv, attention_close
 from ours import _lib
 from ours.mxfp_attn import mxfp_attn
 from ours.mxfp_attn_kernel import prepare_operands, route_tiles, attention_from_operands, mxfp_attn_kernel
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
-COS_MIN, MAXABS_MAX = 0.999, 2e-2
 
 
 def _frames(q, k, n_frames, seed, amp):
@@ -101,8 +100,7 @@ def test_route_golden_vectors_on_gpu():
 
 
 def _compare(got, want, what=""):
-    m = O.precision_metric(got.cpu(), want)
-    assert m["cos"] >= COS_MIN and m["max_abs"] <= MAXABS_MAX, f"{what}: {m}"
+    return attention_close(got, want, what)
 
 
 @pytest.mark.parametrize("D,tile", [(128, 128), (64, 64), (128, 64), (64, 128)])

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 import oracle as O
-from conftest import make_qkv
+from conftest import make_qkv, attention_close
 from ours.block_scaled_matmul import block_scaled_matmul, quantize_block_scaled_from_tensor
 from ours.mxfp_attn_kernel import prepare_operands, route_tiles, attention_from_operands, mxfp_attn_kernel
 from ours.quant_mxint8 import quantize_mx, quantize_mx_dual
@@ -61,8 +61,7 @@ def test_attention_sweep(sweep_seed):
                                    tile=p["tile"], output_dtype=p["dt"])
             want = O.attn_mx(q, k, v, tile=p["tile"], causal=p["causal"], mode={"mxfp8e5": "mxfp8"}.get(p["mode"], p["mode"]),
                              fmt8=fmt8)
-        m = O.precision_metric(out.cpu(), want)
-        assert m["cos"] >= 0.999 and m["max_abs"] <= 2e-2, f"{what}: {m}"
+        attention_close(out, want, what)
 
 
 def test_paired_tile_kernel_sweep():
@@ -100,8 +99,7 @@ def test_paired_tile_kernel_sweep():
         want = O.attn_mx(q, k, v, tile=128, causal=True, mode="diag" if mode.startswith("diag") else mode, fmt8=fmt8,
                          out_dtype=torch.float32)
         assert torch.isfinite(got).all(), what
-        m = O.precision_metric(got.cpu(), want)
-        assert m["cos"] >= 0.999 and m["max_abs"] <= 2e-2, f"{what}: {m}"
+        attention_close(got, want, what)
 
 
 def test_matmul_sweep():
