@@ -174,14 +174,15 @@ def initialize_block_scaled_from_tensor(a_tensor, b_tensor, a_scale, b_scale, bl
 def quantize_block_scaled_from_tensor(a_tensor, b_tensor, block_scale_type="mxfp4", packed_scales=False):
     """MX-quantize bf16/fp16 ``A [M,K]`` and ``B [N,K]`` per 32 along K (scales derived from the data, as the attention
     path does) and package them for :func:`block_scaled_matmul`: returns ``(a, a_scale, b, b_scale, configs)``.
-    ``block_scale_type``: ``"mxfp4"``, ``"mxfp8"`` (E4M3), ``"mxfp8e5"`` (E5M2).
-    Scales stay in the linear ``[rows, K/32]`` layout unless ``packed_scales`` asks for the reference's packed one."""
-    if block_scale_type not in ("mxfp4", "mxfp8", "mxfp8e5"):
+    ``block_scale_type``: ``"mxfp4"``, ``"mxfp8"`` (E4M3), ``"mxfp8e5"`` (E5M2), ``"mixed"`` / ``"mixed_e5"`` (8-bit A,
+    4-bit B).  Scales stay in the linear ``[rows, K/32]`` layout unless ``packed_scales`` asks for the reference's
+    packed one."""
+    if block_scale_type not in ("mxfp4", "mxfp8", "mxfp8e5", "mixed", "mixed_e5"):
         raise ValueError(f"Invalid block scale type: {block_scale_type}")
     configs = make_configs(block_scale_type)
-    fmt, _ = _fmts_of(configs)
-    a, sa = quantize_mx(a_tensor[None, None], 1.0, fmt)
-    b, sb = quantize_mx(b_tensor[None, None], 1.0, fmt)
+    fmt_a, fmt_b = _fmts_of(configs)
+    a, sa = quantize_mx(a_tensor[None, None], 1.0, fmt_a)
+    b, sb = quantize_mx(b_tensor[None, None], 1.0, fmt_b)
     if packed_scales:
         return a[0, 0], pack_scale_5d(sa[0, 0]), b[0, 0], pack_scale_5d(sb[0, 0]), configs
     return a[0, 0], sa[0, 0], b[0, 0], sb[0, 0], configs

@@ -17,7 +17,10 @@ Parity status of each restated function:
 * ``encode_e2m1`` -- pinned by an exhaustive brute-force nearest/ties-to-even
   search over every bf16 and fp16 value, and by golden vectors minted from the
   reference's own ``MXFP4Tensor._from_float`` for the near-tie bias
-  (tests/golden/mxfp_vectors.npz).
+  (tests/golden/mxfp_vectors.npz).  One corner is PARITY UNPINNED: the reference
+  applies the 1e-6 bias under a whole-tensor test (``if is_tie.sum() > 1``,
+  ours/mxfp.py:151-158) that only a one-element tensor without an exact tie
+  fails; this restatement applies the bias for every length.
 * ``encode_e4m3`` -- not in the reference (which stores E5M2); pinned by an
   independent closed-form encoder and torch's own float8_e4m3fn cast.
 * ``quantize_mx`` -- composition of the above; pinned by invariants and

@@ -163,7 +163,8 @@ def test_c4_long_context_full_shape():
     """B=1 Hq=32 Hkv=8 N=131072 D=128 causal with the outlier-channel scheme (seed 3), 128x128 tiles, diag: the whole
     problem runs on the GPU (16384 workgroups of the paired-tile kernel, 1024 key tiles deep).  The oracle checks
     sampled (head, query tile) pairs: four KV groups, both tiles of a pair (even and odd), the first, middle and last
-    tiles.  Size-independent properties on the full output: V = 1 gives 1, the first causal row returns V[0]."""
+    tiles, and one query tile of each of the 32 heads.  Size-independent properties on the full output: V = 1 gives 1,
+    the first causal row returns V[0]."""
     N = 131072
     q, k, v = make_qkv(1, 32, 8, N, 128, seed=3, outliers=True)
     qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
@@ -179,6 +180,11 @@ def test_c4_long_context_full_shape():
         _compare(got, want, f"C4 head {h} tiles {tiles}")
         for n, t in enumerate(tiles):
             _compare(got[:, :, n * 128:(n + 1) * 128], want[:, :, n * 128:(n + 1) * 128], f"C4 head {h} tile {t}")
+    for h in range(32):                                               # and one query tile of every head
+        t, kvh = (h * 33 + 5) % 1024, h // 4
+        want = O.attn_mx(q[:, h:h + 1], k[:, kvh:kvh + 1], v[:, kvh:kvh + 1], tile=128, causal=True, mode="diag", q_tiles=[t],
+                         out_dtype=torch.float32)
+        _compare(o[:, h:h + 1, t * 128:(t + 1) * 128], want, f"C4 head {h} tile {t}")
     o16 = mxfp_attn_kernel(qd, kd, vd, is_causal=True, block_scale_type="diag", output_dtype=torch.bfloat16)
     assert torch.equal(o16, o.to(torch.bfloat16))                     # the bf16 output is the float32 one, rounded once
     del o, o16

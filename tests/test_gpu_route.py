@@ -245,7 +245,8 @@ def test_routed_dit_shape_thresholds_off_equals_mxfp4():
 def test_c5_video_dit_all_heads_diag_and_routed():
     """B=1 H=40 N=32760 (21 frames x 1560 tokens, a ragged last tile) D=128, bidirectional, q/k/v ~ N(0, 0.5) seed 4
     plus per-frame offsets: all 40 heads on the GPU in the diag mode and in the routed mode (route_thresh 0.9).  The
-    oracle checks sampled (head, query tile) pairs -- first, middle and the ragged last tile -- and, for the routed
+    oracle checks sampled (head, query tile) pairs -- first, middle and the ragged last tile, and one query tile of each
+    of the 40 heads -- and, for the routed
     run, with its OWN class map computed from its own scale bytes (which the GPU's map must equal bit for bit)."""
     N, H = 32760, 40
     q, k, v = make_qkv(1, H, H, N, 128, seed=4, sigma=0.5)
@@ -260,6 +261,11 @@ def test_c5_video_dit_all_heads_diag_and_routed():
         want = O.attn_mx(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], tile=128, causal=False, mode="diag", q_tiles=tiles,
                          out_dtype=torch.float32)
         _compare(got[:, h:h + 1, rows(tiles).to(DEV)], want, f"C5 diag head {h} tiles {tiles}")
+    every_head = {h: [(h * 19 + 3) % 256] for h in range(H)}         # and one query tile of every head
+    for h, tiles in every_head.items():
+        want = O.attn_mx(q[:, h:h + 1], k[:, h:h + 1], v[:, h:h + 1], tile=128, causal=False, mode="diag", q_tiles=tiles,
+                         out_dtype=torch.float32)
+        _compare(got[:, h:h + 1, rows(tiles).to(DEV)], want, f"C5 diag head {h} tiles {tiles}")
     del got
 
     ops = prepare_operands(qd, kd, vd, 128, "routed")
@@ -270,7 +276,7 @@ def test_c5_video_dit_all_heads_diag_and_routed():
     attention_from_operands(ops, out, False, route=(cls, order, counts))
     assert torch.isfinite(out).all()
     pre = O.q_pre_scale(128)
-    for h, tiles in samples.items():
+    for h, tiles in list(samples.items()) + [(h, t) for h, t in every_head.items() if h not in samples]:
         _, qs4 = O.quantize_mx(q[:, h:h + 1], pre, O.FMT_E2M1)
         _, ks4 = O.quantize_mx(k[:, h:h + 1], 1.0, O.FMT_E2M1)
         pad = lambda t: torch.nn.functional.pad(t, (0, 0, 0, 256 * 128 - N)).numpy()
