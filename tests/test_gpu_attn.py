@@ -278,7 +278,9 @@ def _robust_thresh(q, k, v, **kw):
 
 @pytest.mark.parametrize("mode,causal,N,D,tile", [("mxfp4", False, 1024, 128, 128), ("mxfp4", True, 1024, 128, 128),
                                                   ("mxfp8", False, 1000, 128, 128), ("mxfp4", False, 512, 64, 64),
-                                                  ("mxfp8", True, 640, 64, 128), ("mxfp4", False, 520, 128, 64)])
+                                                  ("mxfp8", True, 640, 64, 128), ("mxfp4", False, 520, 128, 64),
+                                                  ("diag", True, 1024, 128, 128), ("diag", True, 1000, 128, 128),
+                                                  ("diag", True, 448, 64, 64), ("diag_e5", True, 640, 128, 64)])
 def test_tile_skipping_follows_the_reference_rule(mode, causal, N, D, tile):
     """skip_thresh: key tile 0 always kept; tile j kept iff mean-of-row-maxima(j) >= skip_thresh * that of tile 0.  The kernel must skip
     exactly the tiles the oracle skips (counted per query tile) and match its output."""
@@ -291,7 +293,8 @@ def test_tile_skipping_follows_the_reference_rule(mode, causal, N, D, tile):
     q = q + 1.0                                                    # a common direction in q, a per-tile amount of it in k:
     k = k + torch.rand(nt, generator=g).repeat_interleave(tile)[:N].view(1, 1, N, 1) * 0.5     # tile statistics spread out
     q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
-    kw = dict(tile=tile, causal=causal, mode=mode)
+    kw = dict(tile=tile, causal=causal, mode="diag" if mode.startswith("diag") else mode,
+              fmt8=O.FMT_E5M2 if mode.endswith("e5") else O.FMT_E4M3)
     th = _robust_thresh(q, k, v, **kw)
     want, want_sk = O.attn_mx(q, k, v, skip_thresh=th, return_skipped=True, **kw)
     got, sparsity = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=causal, block_scale_type=mode, tile=tile,
@@ -381,8 +384,8 @@ def test_error_behaviour():
         mxfp_attn(q, k, v, block_scale_type="nvfp4")
     with pytest.raises(ValueError, match="Unsupported dtype"):
         mxfp_attn(q, k, v, output_dtype=torch.int8)
-    with pytest.raises(NotImplementedError, match="single-precision"):
-        mxfp_attn(q, k, v, skip_thresh=0.5, block_scale_type="diag")
+    with pytest.raises(NotImplementedError, match="needs is_causal=True"):
+        mxfp_attn(q, k, v, skip_thresh=0.5, block_scale_type="diag", is_causal=False)
     with pytest.raises(AssertionError, match="multiple of key/value heads"):
         mxfp_attn(q[:, :3], k, v)
 
