@@ -15,10 +15,15 @@
 // row-major HBM layout.  K advances 64 bytes of codes per row per stage (128 E2M1 or 64 8-bit elements).
 //
 // Staging.  Codes go HBM/L2 -> LDS with direct-to-LDS loads (no registers, no LDS-write instructions) into a
-// ring of four stages, three of them in flight while one is being multiplied: with one workgroup per CU nothing
-// else hides the memory latency.  The 16-byte chunks of a row are XOR-swizzled with the row index so that the
-// 128-bit operand reads of 16 consecutive rows hit 16 distinct 4-bank groups.  One barrier per stage.  Wave
-// tiles of 128x128 keep LDS reads at 8 operand fragments per 16 matrix instructions.
+// ring of four stages.  The vector memory path moves cache lines: a wave instruction that takes 64 bytes from each
+// of 16 rows uses half of every 128-byte line it touches and runs at half the rate of one that takes 128 bytes
+// from each of 8 rows (measured L2 -> LDS: 17 against 31 TB/s chip-wide).  So whenever the number of stages is
+// even (PAIR) the ring is refilled two stages -- one "unit" of 128 bytes per row -- at a time: the unit's LDS image
+// has a 128-byte row pitch, one workgroup barrier per unit, one unit in flight while the other is multiplied.
+// Runs with an odd number of stages (4-bit codes, K % 256 == 128) keep the stage-by-stage ring, three stages in
+// flight while one is multiplied.  Either way the 16-byte pieces of a row are XOR-swizzled with the row index so
+// that the 128-bit operand reads of 16 consecutive rows hit 16 distinct 4-bank groups, and wave tiles of
+// 128x128 keep LDS reads at 8 operand fragments per 16 matrix instructions.
 //
 // Scale bytes.  A row's scale bytes for one stage are 4 (or 2) bytes in a line of their own, so fetching them
 // stage by stage costs the vector memory path one cache-line access per row per stage - as many accesses as
@@ -96,9 +101,10 @@ __device__ __forceinline__ void load_to_lds(uint32_t lane_off, const uint8_t* wa
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(base), "v"(lane_off), "s"(gb) : "memory", "m0");
 }
 
-template <int FMT, typename OutT, bool WIDE, bool PK>
+template <int FMT, typename OutT, bool WIDE, bool PK, bool PAIR>
 __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     static_assert(!(WIDE && PK), "packed scales use the per-stage scale area");
+    static_assert(NSTAGE == 4, "PAIR: the ring is two units of two stages");
     constexpr bool FP4 = (FMT == MPSA_FMT_E2M1);
     constexpr int STAGE_BYTES = stage_bytes<WIDE>();
     constexpr int GROUP = FP4 ? 4 : 8;                 // stages covered by 16 scale bytes of a row
@@ -145,13 +151,27 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     g.b += zb * g.N * row_bytes;
     g.sb += zb * g.N * srow_bytes;
     // lane offsets inside a tile's operand (the same for A and B) and inside its scale rows; tile bases are scalar
+    // PAIR: a unit = two consecutive stages = 128 code bytes per row, fetched as whole cache lines: an instruction
+    // of a wave covers 8 rows x 128 B (half-used lines move at half the rate through the vector memory path).  The
+    // unit's LDS image has a 128-byte row pitch; row's 16-byte piece c sits at slot c ^ ((row >> 1) & 7), so that
+    // 16 consecutive rows' reads of one piece fall into 16 distinct 4-bank groups.  Instruction x of the unit
+    // (wave * 8 + c2, c2 = 0..7) covers rows 8x .. 8x+7: only the parity of c2 enters the lane's swizzle.
     uint32_t lo[4];
+    if constexpr (PAIR) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const int p = (wave * 4 + c) * 64 + lane;
-        const int row = p >> 2, slot = p & 3;
-        const int cb = slot ^ ((row >> 2) & 3);
-        lo[c] = (uint32_t)row * (uint32_t)row_bytes + cb * 16;
+        for (int e = 0; e < 2; ++e) {
+            const int cb = (lane & 7) ^ (4 * e + ((lane >> 4) & 3));
+            lo[e] = (uint32_t)(lane >> 3) * (uint32_t)row_bytes + cb * 16;
+        }
+        lo[2] = lo[3] = 0;
+    } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int p = (wave * 4 + c) * 64 + lane;
+            const int row = p >> 2, slot = p & 3;
+            const int cb = slot ^ ((row >> 2) & 3);
+            lo[c] = (uint32_t)row * (uint32_t)row_bytes + cb * 16;
+        }
     }
     const uint32_t los = (uint32_t)(wave * 64 + lane) * (uint32_t)srow_bytes;
     const uint8_t* const a_base = g.a + (int64_t)m0 * row_bytes;
@@ -167,6 +187,36 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
                                 (int64_t)(wave & 1) * kchunks * 512;
     // a stage's loads go out in four parts (two code instructions each, the narrow path's scale words with the
     // last) so that they can be spread between the matrix instructions of a step
+    // PAIR: part `part` of unit u's loads (four code instructions: two per operand; the scale bytes with the last).
+    // Unit u lives in ring half u & 1: [A codes 32 KiB][B codes 32 KiB][scale bytes of its two stages]
+    auto unit_base = [&](int u) __attribute__((always_inline)) { return smem + (u & 1) * 2 * STAGE_BYTES; };
+    auto issue_unit_part = [&](int u, int part) __attribute__((always_inline)) {
+        const int NU = KT / 2;
+        const int uc = u < NU ? u : NU - 1;               // past the end: re-load the last unit
+        uint8_t* ub = unit_base(u);
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int c2 = part * 2 + q, x = wave * 8 + c2;
+            const int64_t go = (int64_t)uc * (2 * ROWB) + (int64_t)x * 8 * row_bytes;
+            load_to_lds<16>(lo[q], a_base + go, ub + x * 1024);
+            load_to_lds<16>(lo[q], b_base + go, ub + 2 * OP_BYTES + x * 1024);
+        }
+        if (part != 3) return;
+        uint8_t* sc = ub + 4 * OP_BYTES;
+        if constexpr (PK) {
+            // 4-bit codes: the unit's two stages are two consecutive 512-byte chunks -- one 64-lane load; 8-bit
+            // codes: one chunk covers the unit, the odd stage takes its scale words from the even stage's registers
+            if constexpr (FP4) load_to_lds<16>((uint32_t)lane * 16u, s_pk + (int64_t)uc * 1024, sc + wave * 1024);
+            else if (lane < 32) load_to_lds<16>(pko, s_pk + (int64_t)uc * 512, sc + wave * 1024);
+        } else if constexpr (!WIDE) {
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const int sco = FP4 ? (2 * uc + hh) * 4 : uc * 4;
+                load_to_lds<4>(los, sa_base + sco, sc + hh * 2 * SC_BYTES + wave * 256);
+                load_to_lds<4>(los, sb_base + sco, sc + hh * 2 * SC_BYTES + SC_BYTES + wave * 256);
+            }
+        }
+    };
     auto issue_part = [&](int kt, int part) __attribute__((always_inline)) {
         const int kc = kt < KT ? kt : KT - 1;             // past the end: re-load the last stage (keeps the count uniform)
         uint8_t* st = smem + (kt % NSTAGE) * STAGE_BYTES;
@@ -194,6 +244,10 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
 #pragma unroll
         for (int part = 0; part < 4; ++part) issue_part(kt, part);
     };
+    auto issue_unit = [&](int u) __attribute__((always_inline)) {
+#pragma unroll
+        for (int part = 0; part < 4; ++part) issue_unit_part(u, part);
+    };
     // wide path: the 16 scale bytes per row of group grp (two instructions per wave)
     auto issue_scales = [&](int grp) __attribute__((always_inline)) {
         const int ng = KT / GROUP;
@@ -212,16 +266,26 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
     if constexpr (WIDE) issue_scales(0);
+    if constexpr (PAIR) {
+        issue_unit(0);
+        issue_unit(1);
+    } else {
 #pragma unroll
-    for (int s = 0; s < NSTAGE; ++s) issue_stage(s);
+        for (int s = 0; s < NSTAGE; ++s) issue_stage(s);
+    }
 
-    // LDS offsets of this lane's operand rows (row-major 64-byte rows, swizzled chunks)
+    // LDS offsets of this lane's operand rows (row-major 64-byte rows -- PAIR: 128-byte rows --, swizzled chunks)
     int offa[4], offb[4], swz_a[4], swz_b[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int ra_ = wm * 128 + i * 32 + r, rb_ = wn * 128 + i * 32 + r;
-        offa[i] = ra_ * ROWB; swz_a[i] = (ra_ >> 2) & 3;
-        offb[i] = rb_ * ROWB; swz_b[i] = (rb_ >> 2) & 3;
+        if constexpr (PAIR) {
+            offa[i] = ra_ * 2 * ROWB; swz_a[i] = (ra_ >> 1) & 7;
+            offb[i] = rb_ * 2 * ROWB; swz_b[i] = (rb_ >> 1) & 7;
+        } else {
+            offa[i] = ra_ * ROWB; swz_a[i] = (ra_ >> 2) & 3;
+            offb[i] = rb_ * ROWB; swz_b[i] = (rb_ >> 2) & 3;
+        }
     }
 
     // One matrix-instruction step's operands: 4 + 4 fragments and their scale bytes.  Two sets alternate: while
@@ -242,11 +306,15 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     // reads operands of step s of stage kt out of the ring: part 0 the B fragments and their scale bytes,
     // part 1 the A fragments and theirs.  grp >= 0 (wide path): also this part's scale rows of group grp.
     auto read_part = [&](Frag& f, const Frag& even, int kt, int s, int part, bool fresh, int grp) __attribute__((always_inline)) {
-        const uint8_t* st = smem + (kt % NSTAGE) * STAGE_BYTES;
         const bool isb = part == 0;
-        const uint8_t* lx = isb ? st + OP_BYTES : st;
+        const int hh = kt & 1;                             // PAIR: which stage of its unit
+        const uint8_t* st = PAIR ? unit_base(kt >> 1) : smem + (kt % NSTAGE) * STAGE_BYTES;
+        const uint8_t* lx = PAIR ? (isb ? st + 2 * OP_BYTES : st) : (isb ? st + OP_BYTES : st);
+        const int c0 = PAIR ? 4 * hh : 0;                  // first 16-byte piece of this stage inside the LDS row
         // the row's scale word of this step pair (paths without the per-group read)
         const uint8_t* sc = WIDE ? scg + ((kt / GROUP) & 1) * 2 * SCG_BYTES + 4 * (FP4 ? kt % GROUP : (kt % GROUP) >> 1) + (isb ? SCG_BYTES : 0)
+                          : PAIR ? (PK ? st + 4 * OP_BYTES + hh * 512 + (isb ? 2048 : 0)
+                                       : st + 4 * OP_BYTES + hh * 2 * SC_BYTES + (isb ? SC_BYTES : 0))
                                  : st + 2 * OP_BYTES + (isb ? SC_BYTES : 0);
         constexpr int sstride = WIDE ? 16 : 4;
         const uint8_t* sg = scg + (grp & 1) * 2 * SCG_BYTES + (isb ? SCG_BYTES : 0);
@@ -264,7 +332,7 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
                 if constexpr (PK) {
                     // one conflict-free 128-bit read: the scale words of this lane's row in all four row blocks
                     if (i == 0) {
-                        const v4i wsc = *reinterpret_cast<const v4i*>(sc + (isb ? wn : wm) * 512 + r * 16);
+                        const v4i wsc = *reinterpret_cast<const v4i*>(sc + (isb ? wn : wm) * (PAIR ? 1024 : 512) + r * 16);
 #pragma unroll
                         for (int q = 0; q < 4; ++q) (isb ? f.rb[q] : f.ra[q]) = (uint32_t)wsc[q];
                     }
@@ -275,13 +343,13 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
                 if (isb) f.sb[i] = even.sb[i]; else f.sa[i] = even.sa[i];
             }
             if constexpr (FP4) {
-                const v4i x = *reinterpret_cast<const v4i*>(lx + off + (((2 * s + h) ^ swz) * 16));
+                const v4i x = *reinterpret_cast<const v4i*>(lx + off + (((c0 + 2 * s + h) ^ swz) * 16));
                 fx = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
             } else {
                 // 8-bit operands: registers 0-3 of both lane halves form MX block 0 (scaled by the byte
                 // lane half 0 supplies), registers 4-7 form block 1 (scaled by lane half 1's byte)
-                const v4i x0 = *reinterpret_cast<const v4i*>(lx + off + ((h ^ swz) * 16));
-                const v4i x1 = *reinterpret_cast<const v4i*>(lx + off + (((h + 2) ^ swz) * 16));
+                const v4i x0 = *reinterpret_cast<const v4i*>(lx + off + (((c0 + h) ^ swz) * 16));
+                const v4i x1 = *reinterpret_cast<const v4i*>(lx + off + (((c0 + h + 2) ^ swz) * 16));
                 fx = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
             }
         }
@@ -319,7 +387,8 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             if (refill) {
-                issue_part(lkt, i);
+                if constexpr (PAIR) issue_unit_part(lkt >> 1, i);     // lkt: first stage of the unit to fetch
+                else issue_part(lkt, i);
                 if constexpr (WIDE) {
                     if (i == 3 && fetch_grp >= 0) issue_scales(fetch_grp);
                 }
@@ -343,8 +412,10 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     // stages later, before the next group's first stage is read.  (The wait leaves 16 loads in flight on the
     // wide path although the two stages after a scale fetch amount to 18: waiting for two loads more than
     // needed is harmless and keeps the count a constant.)
+    // PAIR: called once per unit, after its second stage has been read: the only loads in flight are the next
+    // unit's (and possibly a scale group's), all of which must have landed before that unit is read.
     auto publish = [&]() __attribute__((always_inline)) {
-        constexpr int KEEP = WIDE ? 2 * CODE_LOADS : PK ? (FP4 ? 2 * (CODE_LOADS + 1) : 2 * CODE_LOADS + 1) : 2 * (CODE_LOADS + 2);
+        constexpr int KEEP = PAIR ? 0 : WIDE ? 2 * CODE_LOADS : PK ? (FP4 ? 2 * (CODE_LOADS + 1) : 2 * CODE_LOADS + 1) : 2 * (CODE_LOADS + 2);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(wait_imm(KEEP));
         __syncthreads();
@@ -354,7 +425,9 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     Frag f0, f1;
     {
         // stages 1 .. NSTAGE-1 stay in flight (packed 8-bit: only stage 2 of them carries scale loads)
-        constexpr int KEEP = WIDE ? (NSTAGE - 1) * CODE_LOADS : PK ? (FP4 ? (NSTAGE - 1) * (CODE_LOADS + 1) : (NSTAGE - 1) * CODE_LOADS + 1) : (NSTAGE - 1) * (CODE_LOADS + 2);
+        // PAIR: unit 1 stays in flight (16 code loads and its scale loads: none, one, or four)
+        constexpr int KEEP = PAIR ? 2 * CODE_LOADS + (WIDE ? 0 : PK ? 1 : 4)
+                           : WIDE ? (NSTAGE - 1) * CODE_LOADS : PK ? (FP4 ? (NSTAGE - 1) * (CODE_LOADS + 1) : (NSTAGE - 1) * CODE_LOADS + 1) : (NSTAGE - 1) * (CODE_LOADS + 2);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(wait_imm(KEEP));
         __syncthreads();
@@ -363,8 +436,35 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     read_part(f0, f0, 0, 0, 0, true, GREAD ? 0 : -1);
     read_part(f0, f0, 0, 0, 1, true, GREAD ? 0 : -1);
     // wide path without the per-group read: the group whose scale bytes the refill of stage kt also fetches
-    auto fetch_at = [&](int kt) { return (WIDE && kt % GROUP == 0) ? kt / GROUP + 1 : -1; };
-    if constexpr (GREAD) {
+    auto fetch_at = [&](int kt) { return (WIDE && kt % GROUP == (PAIR ? 1 : 0)) ? kt / GROUP + 1 : -1; };
+    if constexpr (PAIR && GREAD) {
+        // as below, with the ring refilled unit by unit: barrier and refill after a unit's second stage only
+        for (int grp = 0; grp < KT / GROUP; ++grp) {
+#pragma unroll
+            for (int u = 0; u < GROUP; ++u) {
+                const int kt = grp * GROUP + u;            // written so that the stage's parity is a constant
+                step(f0, f1, kt, 1, false, 0, false, u, -1, -1);
+                if (u & 1) publish();
+                step(f1, f0, kt + 1, 0, (u & 1) != 0, kt + 3, true, 0, u == 1 ? grp + 1 : -1, u == GROUP - 1 ? grp + 1 : -1);
+            }
+        }
+    } else if constexpr (PAIR && FP4) {
+        for (int u2 = 0; u2 < KT / 2; ++u2) {
+            const int kt = 2 * u2;
+            step(f0, f1, kt, 1, false, 0, false, 0, -1, -1);
+            step(f1, f0, kt + 1, 0, false, 0, true, 0, -1, -1);
+            step(f0, f1, kt + 1, 1, false, 0, false, 0, -1, -1);
+            publish();
+            step(f1, f0, kt + 2, 0, true, kt + 4, true, 0, fetch_at(kt + 1), -1);
+        }
+    } else if constexpr (PAIR) {
+        for (int u2 = 0; u2 < KT / 2; ++u2) {
+            const int kt = 2 * u2;
+            step(f0, f1, kt + 1, 0, false, 0, false, 0, -1, -1);
+            publish();
+            step(f1, f0, kt + 2, 0, true, kt + 4, true, 0, fetch_at(kt + 1), -1);
+        }
+    } else if constexpr (GREAD) {
         // one trip = one scale group (4 stages = four step pairs), unrolled so that the dword a pair takes from the
         // group's scale rows, the refill that fetches the next group's scale bytes and the step that reads them
         // into registers are all fixed at compile time
@@ -544,23 +644,35 @@ bool force_general() {
     return on;
 }
 
-template <int FMT, typename OutT, bool WIDE, bool PK>
+template <int FMT, typename OutT, bool WIDE, bool PK, bool PAIR>
 struct GemmLds {
     static inline const bool registered =
-        mpsa_register_lds_kernel(reinterpret_cast<const void*>(gemm_mx_kernel<FMT, OutT, WIDE, PK>), smem_bytes<WIDE>());
+        mpsa_register_lds_kernel(reinterpret_cast<const void*>(gemm_mx_kernel<FMT, OutT, WIDE, PK, PAIR>), smem_bytes<WIDE>());
 };
 
-template <int FMT, typename OutT, bool WIDE, bool PK>
+template <int FMT, typename OutT, bool WIDE, bool PK, bool PAIR>
 void launch_kernel(const GemmArgs& g, dim3 grid, hipStream_t st) {
-    if (!GemmLds<FMT, OutT, WIDE, PK>::registered) return;
-    hipLaunchKernelGGL((gemm_mx_kernel<FMT, OutT, WIDE, PK>), grid, dim3(256), smem_bytes<WIDE>(), st, g);
+    if (!GemmLds<FMT, OutT, WIDE, PK, PAIR>::registered) return;
+    hipLaunchKernelGGL((gemm_mx_kernel<FMT, OutT, WIDE, PK, PAIR>), grid, dim3(256), smem_bytes<WIDE>(), st, g);
+}
+
+template <int FMT, typename OutT, bool PAIR>
+void launch_scales(const GemmArgs& g, dim3 grid, hipStream_t st) {
+    if (g.packed)            launch_kernel<FMT, OutT, false, true, PAIR>(g, grid, st);
+    else if (g.K % 512 == 0) launch_kernel<FMT, OutT, true, false, PAIR>(g, grid, st);
+    else                     launch_kernel<FMT, OutT, false, false, PAIR>(g, grid, st);
 }
 
 template <int FMT, typename OutT>
 void launch_one(const GemmArgs& g, dim3 grid, hipStream_t st) {
-    if (g.packed)            launch_kernel<FMT, OutT, false, true>(g, grid, st);
-    else if (g.K % 512 == 0) launch_kernel<FMT, OutT, true, false>(g, grid, st);
-    else                     launch_kernel<FMT, OutT, false, false>(g, grid, st);
+    // whole cache lines per row (two stages at a time) need an even number of stages: always so with 8-bit codes
+    // (K % 128 == 0), with 4-bit codes when K % 256 == 0
+    if constexpr (FMT != MPSA_FMT_E2M1) {
+        launch_scales<FMT, OutT, true>(g, grid, st);
+    } else {
+        if (g.K % 256 == 0) launch_scales<FMT, OutT, true>(g, grid, st);
+        else                launch_scales<FMT, OutT, false>(g, grid, st);
+    }
 }
 
 template <int FMT>
