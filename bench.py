@@ -269,6 +269,8 @@ def run_only(args, device):
         B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
         causal = args.workload not in NON_CAUSAL
         q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21)
+        if args.gemm_operands != "random":     # every element the same: the clock the kernel gets without the operands' bit toggling
+            q, k, v = (torch.full_like(t, 1.0 if args.gemm_operands == "ones" else 0.0) for t in (q, k, v))
         out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
         from ours.mxfp_attn_kernel import q_fusable
         fuse = args.mode != "routed" and not args.no_fuse_q and q_fusable(q, k, tile, args.mode, causal)
@@ -325,7 +327,7 @@ def main():
     ap.add_argument("--no-c4", action="store_true", help="leave the long-context figures out of `secondary`")
     ap.add_argument("--eager", action="store_true", help="time plain launches instead of replaying the step as a HIP graph")
     ap.add_argument("--gemm-operands", default="random", choices=["random", "ones", "zeros"],
-                    help="--only gemm4|gemm8: N(0,1) operands (default) or constant ones (the clock then stays up)")
+                    help="--only gemm4|gemm8|attn: the workload's random operands (default) or constant ones (the clock then stays up)")
     ap.add_argument("--linear-scales", action="store_true",
                     help="with --only gemm4/gemm8: row-major [rows, K/32] scales instead of the reference's packed form")
     ap.add_argument("--only", default=None, choices=["attn", "copy", "quant", "gemm4", "gemm8", "mfma"],
