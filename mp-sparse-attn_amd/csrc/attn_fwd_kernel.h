@@ -76,6 +76,8 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
     uint8_t* const vbuf0 = smem + 2 * G::K_BYTES;
     float* const stat_lds = reinterpret_cast<float*>(smem + G::SMEM);     // SKIP: [2][NW] partial statistics
     float sink_stat = 0.0f;
+    bool sink_preset = false;   // SKIP, non-causal diag run, query tile 0: the sink's statistic was taken ahead of the walk
+    bool started = false;       // SKIP: a kept tile has set the running maximum
     int n_skipped = 0;
     // Visiting order.  The order of key tiles does not matter to the softmax, so the tiles that need special
     // treatment go LAST: first every plain tile (main precision, no mask) in one tight loop, then the tile that
@@ -285,6 +287,46 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
         }
     }
 
+    // SKIP in a non-causal diag run: the rule's reference tile, key tile 0, is query tile 0's diagonal tile, which
+    // the walk visits last.  That one workgroup takes the tile's statistic (8-bit scores, no softmax, no P.V) first.
+    if constexpr (SKIP && MODE == MPSA_MODE_DIAG) {
+        if (!a.causal && i == 0 && nsteps > 1) {
+            load_kscales(0, true);
+            load_q(true);
+            float mx = -__builtin_inff();
+#pragma unroll
+            for (int kb = 0; kb < G::KB; ++kb) {
+                const uint8_t* src = a.k8 + (khead_row + 32 * kb + r) * G::ROW8 + h * 16;
+                v16f sk;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) sk[e] = 0.0f;
+#pragma unroll
+                for (int s = 0; s < G::SST; ++s) {
+                    const v4i x0 = *reinterpret_cast<const v4i*>(src + s * 64);
+                    const v4i x1 = *reinterpret_cast<const v4i*>(src + s * 64 + 32);
+                    const v8i kd = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+                    sk = score_mfma8<FMT8>(kd, qf[s], sk, s, ksc[kb], qsc);
+                }
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, sk[e]);     // more than one key tile: tile 0 is full
+            }
+            mx = max_lane_pair(mx);
+            float sv = (q_local < a.nq) ? mx : 0.0f;
+#pragma unroll
+            for (int o = 1; o < 32; o <<= 1) sv += __shfl_xor(sv, o);
+            float* sl = stat_lds + G::NW;                  // the slot of odd steps: step 1 writes it after step 0's barrier
+            if (lane == 0) sl[w] = sv;
+            __syncthreads();
+            float tot = 0.0f;
+#pragma unroll
+            for (int x = 0; x < G::NW; ++x) tot += sl[x];
+            sink_stat = tot / (float)min(TILE, a.nq);
+            sink_preset = true;
+            load_kscales(tile_rel(0, R0{}), false);        // back to the operands of step 0
+            load_q(false);
+        }
+    }
+
     // One step = one key tile.  IS8 / MASKED are compile-time so the common step (4-bit, unmasked) carries no
     // branches or mask arithmetic.
     //   PREP: also pull the next step's K operand (same precision as the run's plain tiles) into registers.
@@ -366,16 +408,19 @@ __global__ __launch_bounds__(TILE * 2, 2) void attn_fwd_kernel(AttnArgs a) {
             const float stat = tot / (float)min(TILE, a.nq - i * TILE);
             // the diagonal tile of a causal run is exempt like the sink: the reference walks it in a stage of its
             // own, whose first tile is always kept (ours/online_routing.py:68-77, :87-112)
-            if (t == 0) sink_stat = stat;
-            else keep = (a.causal && j == i) || stat >= sink_stat * a.skip_thresh;
+            if (t == 0 && !sink_preset) sink_stat = stat;
+            else keep = j == 0 || (a.causal && j == i) || stat >= sink_stat * a.skip_thresh;
             if (!keep) ++n_skipped;
         }
+        // the first tile that counts sets the running maximum (with a sink taken ahead, step 0 may be skipped)
+        const bool first = SKIP ? !started : (t == 0);
         v4i pk[G::KB][2];                               // 8 packed 16-bit values = one P^T operand
         if (keep) {
-        if (t == 0 || __any(mx > REBASE)) {
+        if constexpr (SKIP) started = true;
+        if (first || __any(mx > REBASE)) {
             // move the reference maximum up to this tile's maximum (first tile: set it)
-            const float delta = (t == 0) ? mx : __builtin_fmaxf(mx, 0.0f);
-            const float alpha = (t == 0) ? 1.0f : __builtin_amdgcn_exp2f(-delta);
+            const float delta = first ? mx : __builtin_fmaxf(mx, 0.0f);
+            const float alpha = first ? 1.0f : __builtin_amdgcn_exp2f(-delta);
             m_run += delta;
 #pragma unroll
             for (int e = 0; e < 16; ++e) negm[e] = -m_run;

@@ -1,7 +1,7 @@
 // Tile-skipping variants of the general fused attention kernel (see attn_fwd_kernel.h for the rule, which is the
-// reference's, ours/mxfp_attn_kernel.py:272-297).  Single-precision modes, and the diag mode of a causal run: there
-// the first step of every query tile is key tile 0 (for query tile 0 it is the diagonal tile itself), as the rule
-// needs; a non-causal diag run visits tile 0 last for query tile 0 and is rejected.
+// reference's, ours/mxfp_attn_kernel.py:272-297).  Single-precision modes and the diag mode.  The rule's reference
+// tile is key tile 0; every walk starts there except query tile 0 of a non-causal diag run, whose diagonal tile
+// (= key tile 0) comes last -- that workgroup takes the tile's statistic ahead of its walk.
 #include "attn_fwd_kernel.h"
 
 namespace {
@@ -25,10 +25,8 @@ int launch_dt(const AttnArgs& a, int pv_dtype, hipStream_t st) {
 }  // namespace
 
 int attn_skip_launch(const AttnArgs& a, int pv_dtype, hipStream_t st) {
-    if (a.mode == MPSA_MODE_DIAG && !a.causal)
-        return mpsa_fail(MPSA_EUNSUPPORTED, "attn: tile skipping in the diag mode needs a causal run (the rule's reference tile is the first key tile, which a non-causal diag run visits last for query tile 0)");
     if (a.mode != MPSA_MODE_MXFP4 && a.mode != MPSA_MODE_MXFP8 && a.mode != MPSA_MODE_DIAG)
-        return mpsa_fail(MPSA_EUNSUPPORTED, "attn: tile skipping needs mode mxfp4, mxfp8 or (causal) diag");
+        return mpsa_fail(MPSA_EUNSUPPORTED, "attn: tile skipping needs mode mxfp4, mxfp8 or diag");
     if (a.d == 128 && a.tile == 128) return launch_dt<128, 128>(a, pv_dtype, st);
     if (a.d == 64 && a.tile == 64)   return launch_dt<64, 64>(a, pv_dtype, st);
     if (a.d == 128 && a.tile == 64)  return launch_dt<128, 64>(a, pv_dtype, st);

@@ -247,15 +247,10 @@ def _normalise(q, k, v):
     return q.to(lp), k.to(lp), v.to(lp)
 
 
-def _reject_unsupported(attn_mask, dropout_p, attention_sink, block_scale_type, skip_thresh, is_causal):
+def _reject_unsupported(attn_mask, dropout_p, attention_sink):
     if attn_mask is not None or dropout_p != 0.0 or attention_sink:
         raise NotImplementedError("attn_mask, dropout_p and attention_sink are not implemented "
                                   "(the reference accepts and ignores them)")
-    if skip_thresh is not None and not is_causal and _MODES.get(block_scale_type) == _lib.MODE_DIAG:
-        raise NotImplementedError("tile skipping (skip_thresh) with a diag block_scale_type needs is_causal=True: the "
-                                  "rule's reference tile is the first key tile, which a non-causal diag run visits "
-                                  "last for query tile 0 (mxfp4, mxfp8, mxfp8e5 skip either way; \"routed\" skips by "
-                                  "its own statistic)")
 
 
 @torch.compiler.disable
@@ -269,14 +264,14 @@ def mxfp_attn_kernel(q, k, v, attn_mask=None, dropout_p=0.0,
     ``block_scale_type``: ``"mxfp4"``, ``"mxfp8"`` (E4M3), ``"mxfp8e5"`` (E5M2, the reference's 8-bit format),
     ``"diag"`` (tile j == i in MXFP8, the rest in MXFP4) or ``"diag_e5"``.  K/V may have fewer heads than Q
     (grouped-query attention); ``is_causal`` is honoured.  ``skip_thresh`` switches on the reference's tile
-    skipping (ours/mxfp_attn_kernel.py:272-297; the diag types only with ``is_causal``); ``return_sparsity`` adds the share of
+    skipping (ours/mxfp_attn_kernel.py:272-297; fixed-precision and diag types); ``return_sparsity`` adds the share of
     skipped tiles as a second result.
 
     ``block_scale_type="routed"`` (``"routed_e5"``): per-tile precision from the tile router -- a tile whose score
     bound (from the E8M0 bytes of Q and K) reaches ``route_thresh`` times the largest of its query tile runs in
     MXFP8, one below ``skip_thresh`` times it is skipped, the rest runs in MXFP4."""
     _lib.require_device(q, k, v)
-    _reject_unsupported(attn_mask, dropout_p, attention_sink, block_scale_type, skip_thresh, is_causal)
+    _reject_unsupported(attn_mask, dropout_p, attention_sink)
     torch.cuda.set_device(v.device)
     q, k, v = _normalise(q, k, v)
     q, k, v = _as_bhnd(q, tensor_layout), _as_bhnd(k, tensor_layout), _as_bhnd(v, tensor_layout)

@@ -280,7 +280,10 @@ def _robust_thresh(q, k, v, **kw):
                                                   ("mxfp8", False, 1000, 128, 128), ("mxfp4", False, 512, 64, 64),
                                                   ("mxfp8", True, 640, 64, 128), ("mxfp4", False, 520, 128, 64),
                                                   ("diag", True, 1024, 128, 128), ("diag", True, 1000, 128, 128),
-                                                  ("diag", True, 448, 64, 64), ("diag_e5", True, 640, 128, 64)])
+                                                  ("diag", True, 448, 64, 64), ("diag_e5", True, 640, 128, 64),
+                                                  ("diag", False, 1024, 128, 128), ("diag", False, 1000, 128, 128),
+                                                  ("diag_e5", False, 448, 64, 64), ("diag", False, 520, 128, 64),
+                                                  ("diag", False, 256, 128, 128)])
 def test_tile_skipping_follows_the_reference_rule(mode, causal, N, D, tile):
     """skip_thresh: key tile 0 always kept; tile j kept iff mean-of-row-maxima(j) >= skip_thresh * that of tile 0.  The kernel must skip
     exactly the tiles the oracle skips (counted per query tile) and match its output."""
@@ -384,8 +387,6 @@ def test_error_behaviour():
         mxfp_attn(q, k, v, block_scale_type="nvfp4")
     with pytest.raises(ValueError, match="Unsupported dtype"):
         mxfp_attn(q, k, v, output_dtype=torch.int8)
-    with pytest.raises(NotImplementedError, match="needs is_causal=True"):
-        mxfp_attn(q, k, v, skip_thresh=0.5, block_scale_type="diag", is_causal=False)
     with pytest.raises(AssertionError, match="multiple of key/value heads"):
         mxfp_attn(q[:, :3], k, v)
 
