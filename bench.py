@@ -269,8 +269,8 @@ def run_only(args, device):
         B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
         causal = args.workload not in NON_CAUSAL
         q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21)
-        if args.gemm_operands != "random":     # every element the same: the clock the kernel gets without the operands' bit toggling
-            q, k, v = (torch.full_like(t, 1.0 if args.gemm_operands == "ones" else 0.0) for t in (q, k, v))
+        if args.operands != "random":     # every element the same: the clock the kernel gets without the operands' bit toggling
+            q, k, v = (torch.full_like(t, 1.0 if args.operands == "ones" else 0.0) for t in (q, k, v))
         out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
         from ours.mxfp_attn_kernel import q_fusable
         fuse = args.mode != "routed" and not args.no_fuse_q and q_fusable(q, k, tile, args.mode, causal)
@@ -286,11 +286,11 @@ def run_only(args, device):
     else:
         M = N = K = 8192
         g = torch.Generator(device=device).manual_seed(1)
-        if args.gemm_operands == "random":
+        if args.operands == "random":
             a = torch.randn(M, K, generator=g, device=device).to(torch.bfloat16)[None, None]
             b = torch.randn(N, K, generator=g, device=device).to(torch.bfloat16)[None, None]
         else:          # every code and scale byte the same: what the kernel does when power management leaves the clock alone
-            a = torch.full((1, 1, M, K), 1.0 if args.gemm_operands == "ones" else 0.0, dtype=torch.bfloat16, device=device)
+            a = torch.full((1, 1, M, K), 1.0 if args.operands == "ones" else 0.0, dtype=torch.bfloat16, device=device)
             b = a.clone()
         bst, fmt = ("mxfp4", _lib.FMT_E2M1) if args.only == "gemm4" else ("mxfp8", _lib.FMT_E4M3)
         ac, asc = quantize_mx(a, 1.0, fmt)
@@ -299,7 +299,7 @@ def run_only(args, device):
         sa2, sb2 = (asc[0, 0], bsc[0, 0]) if args.linear_scales else (pack_scale_5d(asc[0, 0]), pack_scale_5d(bsc[0, 0]))
         fn = lambda: block_scaled_matmul(ac[0, 0], sa2, bc[0, 0], sb2, torch.bfloat16, M, N, K, cfg)
         info = {"kernel": "gemm " + bst, "flops": 2.0 * M * N * K, "scales": "row-major" if args.linear_scales else "packed",
-                "operands": args.gemm_operands}
+                "operands": args.operands}
     fn()
     torch.cuda.synchronize()
     ms = time_events(fn, args.steps)
@@ -326,7 +326,7 @@ def main():
     ap.add_argument("--no-fuse-q", action="store_true", help="with --only attn: hand the kernel quantized Q operands")
     ap.add_argument("--no-c4", action="store_true", help="leave the long-context figures out of `secondary`")
     ap.add_argument("--eager", action="store_true", help="time plain launches instead of replaying the step as a HIP graph")
-    ap.add_argument("--gemm-operands", default="random", choices=["random", "ones", "zeros"],
+    ap.add_argument("--operands", default="random", choices=["random", "ones", "zeros"],
                     help="--only gemm4|gemm8|attn: the workload's random operands (default) or constant ones (the clock then stays up)")
     ap.add_argument("--linear-scales", action="store_true",
                     help="with --only gemm4/gemm8: row-major [rows, K/32] scales instead of the reference's packed form")
