@@ -69,18 +69,11 @@ template <> __device__ __forceinline__ _Float16 cvt_out<_Float16>(float v) { ret
 struct OutE5M2 { uint8_t b; };
 template <> __device__ __forceinline__ OutE5M2 cvt_out<OutE5M2>(float v) {
     const uint32_t u = mpsa_f2u(v);
-    const uint32_t sign = (u >> 24) & 0x80u;
-    uint32_t a = u & 0x7FFFFFFFu;
-    if (a > 0x7F800000u) return OutE5M2{(uint8_t)(sign | 0x7Fu)};
-    uint32_t code;
-    if (a >= 0x38800000u) {                       // |v| >= 2^-14: normal
-        a += 0xFFFFFu + ((a >> 21) & 1u);
-        code = (a >> 21) - (112u << 2);
-        code = code > 0x7Cu ? 0x7Cu : code;
-    } else {                                      // subnormal, unit 2^-16
-        code = mpsa_f2u(mpsa_u2f(a) + 128.0f) - 0x43000000u;
-    }
-    return OutE5M2{(uint8_t)(sign | code)};
+    const uint32_t a = u & 0x7FFFFFFFu;
+    // 61440 = the largest finite E5M2 value plus half a step: from there on the cast gives infinity (or keeps NaN)
+    if (a >= 0x47700000u) return OutE5M2{(uint8_t)(((u >> 24) & 0x80u) | (a > 0x7F800000u ? 0x7Fu : 0x7Cu))};
+    // below that the conversion instruction rounds to nearest even, subnormals included
+    return OutE5M2{(uint8_t)(__builtin_amdgcn_cvt_pk_bf8_f32(v, v, 0, false) & 0xFF)};
 }
 
 // Direct-to-LDS load written as inline assembly: lane L's BYTES bytes at wave_base + lane_off land at

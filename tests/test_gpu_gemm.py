@@ -190,6 +190,14 @@ def test_e5m2_output_dtype():
     want = c32.cpu().to(torch.float8_e5m2)
     assert torch.equal(c8.cpu().view(torch.uint8), want.view(torch.uint8))
     assert torch.isinf(want.float()).any() and (want.float().abs() < 1).any()
+    # results down in E5M2's subnormal range (below 2^-14) and under its smallest step (2^-16)
+    ac, asc, bc, bsc, cfg = quantize_block_scaled_from_tensor((a * 2.0 ** -14).bfloat16().to(DEV), (b * 2.0 ** -12).bfloat16().to(DEV), "mxfp4")
+    c32 = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg)
+    c8 = block_scaled_matmul(ac, asc, bc, bsc, torch.float8_e5m2, M, N, K, cfg)
+    want = c32.cpu().to(torch.float8_e5m2)
+    assert torch.equal(c8.cpu().view(torch.uint8), want.view(torch.uint8))
+    mag = want.float().abs()
+    assert ((mag > 0) & (mag < 2.0 ** -14)).any() and (mag == 0).any() and (mag >= 2.0 ** -14).any()
 
 
 @pytest.mark.parametrize("bst", ["mxfp4", "mxfp8", "mxfp8e5"])
