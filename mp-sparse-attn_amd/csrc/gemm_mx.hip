@@ -509,21 +509,35 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
 // The reference's kernel tiles 128 x 256 with masked edges (ours/block_scaled_matmul.py:154-267) and takes the two
 // operands' element widths separately (ELEM_PER_BYTE_A / ELEM_PER_BYTE_B, "mixed" = 8-bit A x 4-bit B,
 // ours/block_scaled_matmul.py:318-324).  This kernel covers what the 256 x 256 kernel above does not: a workgroup of
-// four waves owns a 128 x 128 tile, a wave 64 x 64 (2 x 2 accumulators); operand fragments and scale bytes come
-// straight from global memory (L2), one 64-element step ahead of the matrix instructions.  Rows past M or N are
-// read from the last valid row and never stored.  Each operand's registers follow its own format's layout (4-bit:
-// the lane half's registers are MX block h of the step; 8-bit: registers 0-3 of both halves are block 0, 4-7 block 1).
-template <int FMT>
-__device__ __forceinline__ v8i load_frag(const uint8_t* row_ptr, int ks, int h) {
-    if constexpr (FMT == MPSA_FMT_E2M1) {
-        const v4i x = *reinterpret_cast<const v4i*>(row_ptr + ks * 32 + h * 16);
-        return (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
-    } else {
-        const v4i x0 = *reinterpret_cast<const v4i*>(row_ptr + ks * 64 + h * 16);
-        const v4i x1 = *reinterpret_cast<const v4i*>(row_ptr + ks * 64 + h * 16 + 32);
-        return (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+// four waves owns a 128 x 128 tile, a wave 64 x 64 (2 x 2 accumulators), two workgroups share a CU.  K advances
+// 128 elements per stage (two matrix-instruction steps; 64 code bytes per row of a 4-bit operand, 128 of an 8-bit
+// one): the stage's codes travel L2 -> LDS with direct-to-LDS loads into one of two buffers while the other is
+// multiplied, rows XOR-swizzled as in the kernel above; rows past M or N are fetched from the last valid row and
+// never stored.  The four scale bytes a row has per stage come straight from global memory as one word, a stage
+// ahead (byte by byte when K is not a multiple of 128: the last stage is then half a stage).  Each operand's
+// registers follow its own format's layout (4-bit: the lane half's registers are MX block h of the step; 8-bit:
+// registers 0-3 of both halves are block 0, 4-7 block 1).
+template <int FMT> struct EdgeOp {
+    static constexpr bool FP4 = FMT == MPSA_FMT_E2M1;
+    static constexpr int ROW = FP4 ? 64 : 128;           // code bytes per row per stage
+    static constexpr int CPR = ROW / 16;                 // 16-byte pieces per row
+    static constexpr int BYTES = 128 * ROW;              // the operand's codes of one stage
+    static constexpr int IPW = BYTES / 1024 / 4;         // direct-to-LDS instructions per wave and stage
+    __device__ static __forceinline__ int swz(int row) { return FP4 ? (row >> 2) & 3 : (row >> 1) & 7; }
+    // the fragment of matrix-instruction step k (0 / 1) of the stage, LDS row `row` of the operand's stage image
+    __device__ static __forceinline__ v8i frag(const uint8_t* img, int row, int k, int h) {
+        const uint8_t* p = img + row * ROW;
+        const int f = swz(row);
+        if constexpr (FP4) {
+            const v4i x = *reinterpret_cast<const v4i*>(p + (((2 * k + h) ^ f) * 16));
+            return (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+        } else {
+            const v4i x0 = *reinterpret_cast<const v4i*>(p + (((4 * k + h) ^ f) * 16));
+            const v4i x1 = *reinterpret_cast<const v4i*>(p + (((4 * k + h + 2) ^ f) * 16));
+            return (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        }
     }
-}
+};
 
 // scale byte of row `row`, MX block kb: row-major [rows, K/32] or the packed [rows/128, K/128, 32, 4, 4] form
 __device__ __forceinline__ int load_scale(const uint8_t* s, int row, int kb, int kblocks, bool packed) {
@@ -532,32 +546,92 @@ __device__ __forceinline__ int load_scale(const uint8_t* s, int row, int kb, int
     return s[chunk * 512 + (row & 31) * 16 + ((row >> 5) & 3) * 4 + (kb & 3)];
 }
 
+template <int FA, int FB>
+constexpr int general_smem() { return 2 * (EdgeOp<FA>::BYTES + EdgeOp<FB>::BYTES); }
+
 template <int FA, int FB, typename OutT>
-__global__ __launch_bounds__(256) void gemm_mx_general_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256, 2) void gemm_mx_general_kernel(GemmArgs g) {
+    typedef EdgeOp<FA> OA;
+    typedef EdgeOp<FB> OB;
+    constexpr int STAGE = OA::BYTES + OB::BYTES;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     const int h = lane >> 5, r = lane & 31;
-    const int rowb_a = FA == MPSA_FMT_E2M1 ? g.K / 2 : g.K;
-    const int rowb_b = FB == MPSA_FMT_E2M1 ? g.K / 2 : g.K;
+    const int rowb_a = OA::FP4 ? g.K / 2 : g.K;
+    const int rowb_b = OB::FP4 ? g.K / 2 : g.K;
     const int kblocks = g.K / 32;
     const int tiles_n = (g.N + 127) / 128;
-    const int m0 = (blockIdx.x / tiles_n) * 128 + wm * 64;
-    const int n0 = (blockIdx.x % tiles_n) * 128 + wn * 64;
+    const int tm0 = (blockIdx.x / tiles_n) * 128, tn0 = (blockIdx.x % tiles_n) * 128;   // the workgroup's tile
+    const int m0 = tm0 + wm * 64, n0 = tn0 + wn * 64;                                   // the wave's
     const int bz = blockIdx.y;
     const int bb = bz / g.heads_a, ha = bz - bb * g.heads_a;
     const int64_t zb = (int64_t)bb * g.heads_b + ha / (g.heads_a / g.heads_b);
-    // scale rows per matrix: the packed form pads nothing (rows % 128 == 0 is required for it)
     const uint8_t* a = g.a + (int64_t)bz * g.M * rowb_a;
     const uint8_t* b = g.b + zb * g.N * rowb_b;
     const uint8_t* sa = g.sa + (int64_t)bz * g.M * kblocks;
     const uint8_t* sb = g.sb + zb * g.N * kblocks;
+    const int steps = g.K / 64;                          // matrix-instruction steps
+    const int nstages = (steps + 1) / 2;                 // the last stage is half a stage when `steps` is odd
+    const bool words = (g.K % 128) == 0;                 // a row's four scale bytes of a stage are one aligned word
+
+    // ---- staging: lane offsets of this wave's pieces (rows past the matrix clamp to its last row) ----
+    uint32_t loa[OA::IPW], lob[OB::IPW];
+    bool firsta[OA::IPW], firstb[OB::IPW];               // the piece lies in the stage's first half (first step)
+#pragma unroll
+    for (int c = 0; c < OA::IPW; ++c) {
+        const int p = (wave * OA::IPW + c) * 64 + lane;
+        const int row = p / OA::CPR, cb = (p % OA::CPR) ^ OA::swz(row);
+        loa[c] = (uint32_t)min(tm0 + row, g.M - 1) * (uint32_t)rowb_a + cb * 16;
+        firsta[c] = cb < OA::CPR / 2;
+    }
+#pragma unroll
+    for (int c = 0; c < OB::IPW; ++c) {
+        const int p = (wave * OB::IPW + c) * 64 + lane;
+        const int row = p / OB::CPR, cb = (p % OB::CPR) ^ OB::swz(row);
+        lob[c] = (uint32_t)min(tn0 + row, g.N - 1) * (uint32_t)rowb_b + cb * 16;
+        firstb[c] = cb < OB::CPR / 2;
+    }
+    auto issue = [&](int s) __attribute__((always_inline)) {
+        uint8_t* st = smem + (s & 1) * STAGE;
+        const bool half = 2 * s + 1 >= steps;            // only the stage's first step exists
+#pragma unroll
+        for (int c = 0; c < OA::IPW; ++c)
+            if (!half || firsta[c]) load_to_lds<16>(loa[c], a + (int64_t)s * OA::ROW, st + (wave * OA::IPW + c) * 1024);
+#pragma unroll
+        for (int c = 0; c < OB::IPW; ++c)
+            if (!half || firstb[c]) load_to_lds<16>(lob[c], b + (int64_t)s * OB::ROW, st + OA::BYTES + (wave * OB::IPW + c) * 1024);
+    };
+
+    // ---- this lane's rows (for the scale bytes) and the scale words of a stage ----
     int ra[2], rb[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         ra[i] = min(m0 + i * 32 + r, g.M - 1);
         rb[i] = min(n0 + i * 32 + r, g.N - 1);
     }
+    auto scale_word = [&](const uint8_t* sc, int row, int s) __attribute__((always_inline)) -> uint32_t {
+        if (words) {
+            const int64_t off = g.packed ? ((int64_t)(row >> 7) * (kblocks >> 2) + s) * 512 + (row & 31) * 16 + ((row >> 5) & 3) * 4
+                                         : (int64_t)row * kblocks + 4 * s;
+            return *reinterpret_cast<const uint32_t*>(sc + off);
+        }
+        uint32_t w = 0;                                  // K % 128 == 64 (row-major scales only): byte by byte
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (4 * s + q < kblocks) w |= (uint32_t)load_scale(sc, row, 4 * s + q, kblocks, false) << (8 * q);
+        return w;
+    };
+    uint32_t wa[2], wb[2], na[2] = {0, 0}, nb[2] = {0, 0};
+    auto fetch_scales = [&](int s, uint32_t (&xa)[2], uint32_t (&xb)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            xa[i] = scale_word(sa, ra[i], s);
+            xb[i] = scale_word(sb, rb[i], s);
+        }
+    };
+
     v16f acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -566,31 +640,41 @@ __global__ __launch_bounds__(256) void gemm_mx_general_kernel(GemmArgs g) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    const int steps = g.K / 64;
-    v8i fa[2], fb[2];
-    int ca[2], cb[2];
-    auto fetch = [&](int ks, v8i (&xa)[2], v8i (&xb)[2], int (&ya)[2], int (&yb)[2]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            xa[i] = load_frag<FA>(a + (int64_t)ra[i] * rowb_a, ks, h);
-            xb[i] = load_frag<FB>(b + (int64_t)rb[i] * rowb_b, ks, h);
-            ya[i] = load_scale(sa, ra[i], 2 * ks + h, kblocks, g.packed != 0);
-            yb[i] = load_scale(sb, rb[i], 2 * ks + h, kblocks, g.packed != 0);
+    issue(0);
+    fetch_scales(0, wa, wb);
+    for (int s = 0; s < nstages; ++s) {
+        // stage s has landed for every wave, and every wave is through with the buffer stage s + 1 goes to
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0070);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        if (s + 1 < nstages) {
+            issue(s + 1);
+            fetch_scales(s + 1, na, nb);
         }
-    };
-    fetch(0, fa, fb, ca, cb);
-    for (int ks = 0; ks < steps; ++ks) {
-        v8i na[2], nb[2];
-        int da[2], db[2];
-        fetch(ks + 1 < steps ? ks + 1 : ks, na, nb, da, db);
+        const uint8_t* ia = smem + (s & 1) * STAGE;
+        const uint8_t* ib = ia + OA::BYTES;
+        const int nk = min(2, steps - 2 * s);
+        for (int k = 0; k < nk; ++k) {
+            v8i fa[2], fb[2];
+            int ca[2], cb[2];
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < 2; ++i) {
+                fa[i] = OA::frag(ia, wm * 64 + i * 32 + r, k, h);
+                fb[i] = OB::frag(ib, wn * 64 + i * 32 + r, k, h);
+                ca[i] = (int)(wa[i] >> (8 * (2 * k + h)));       // the matrix instruction takes the low byte
+                cb[i] = (int)(wb[i] >> (8 * (2 * k + h)));
+            }
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], FA, FB, 0, ca[i], 0, cb[j]);
+            for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int i = 0; i < 2; ++i) { fa[i] = na[i]; fb[i] = nb[i]; ca[i] = da[i]; cb[i] = db[i]; }
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], FA, FB, 0, ca[i], 0, cb[j]);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) { wa[i] = na[i]; wb[i] = nb[i]; }
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);                  // no direct-to-LDS load may outlive the workgroup
 
     // accumulator register e of lane (h, r) is C[8*(e/4) + 4*h + e%4][r] of its 32 x 32 block
     OutT* c = static_cast<OutT*>(g.c) + (int64_t)bz * g.M * g.ldc;
@@ -607,12 +691,25 @@ __global__ __launch_bounds__(256) void gemm_mx_general_kernel(GemmArgs g) {
         }
 }
 
+template <int FA, int FB, typename OutT>
+struct GeneralLds {
+    static inline const bool registered =
+        mpsa_register_lds_kernel(reinterpret_cast<const void*>(gemm_mx_general_kernel<FA, FB, OutT>), general_smem<FA, FB>());
+};
+
+template <int FA, int FB, typename OutT>
+void launch_general_kernel(const GemmArgs& g, dim3 grid, hipStream_t st) {
+    if (!GeneralLds<FA, FB, OutT>::registered) return;
+    constexpr int lds = general_smem<FA, FB>();
+    hipLaunchKernelGGL((gemm_mx_general_kernel<FA, FB, OutT>), grid, dim3(256), lds, st, g);
+}
+
 template <int FA, int FB>
 void launch_general_out(const GemmArgs& g, int c_dtype, dim3 grid, hipStream_t st) {
-    if (c_dtype == MPSA_BF16)        hipLaunchKernelGGL((gemm_mx_general_kernel<FA, FB, __bf16>), grid, dim3(256), 0, st, g);
-    else if (c_dtype == MPSA_F8E5M2) hipLaunchKernelGGL((gemm_mx_general_kernel<FA, FB, OutE5M2>), grid, dim3(256), 0, st, g);
-    else if (c_dtype == MPSA_F16)    hipLaunchKernelGGL((gemm_mx_general_kernel<FA, FB, _Float16>), grid, dim3(256), 0, st, g);
-    else                             hipLaunchKernelGGL((gemm_mx_general_kernel<FA, FB, float>), grid, dim3(256), 0, st, g);
+    if (c_dtype == MPSA_BF16)        launch_general_kernel<FA, FB, __bf16>(g, grid, st);
+    else if (c_dtype == MPSA_F8E5M2) launch_general_kernel<FA, FB, OutE5M2>(g, grid, st);
+    else if (c_dtype == MPSA_F16)    launch_general_kernel<FA, FB, _Float16>(g, grid, st);
+    else                             launch_general_kernel<FA, FB, float>(g, grid, st);
 }
 
 template <int FA>
