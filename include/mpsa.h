@@ -292,8 +292,8 @@ int mpsa_attn_fwd_q16_supported(int64_t B, int64_t Hq, int64_t Hkv, int64_t n, i
  * over the tile's valid query rows of the row maximum of S (after masking); tile 0 is always kept and sets the
  * reference value; tile j > 0 is kept iff stat(j) >= stat(0) * skip_thresh, and the diagonal tile of a causal run is
  * always kept (ours/online_routing.py:68-77: its stage starts a loop of its own); a skipped tile contributes nothing.
- * Arguments as mpsa_attn_fwd; mode MPSA_MODE_MXFP4, MPSA_MODE_MXFP8 or MPSA_MODE_DIAG (each tile's statistic is that
- * of the precision the tile runs in), plus
+ * Arguments as mpsa_attn_fwd; mode MPSA_MODE_MXFP4, MPSA_MODE_MXFP8, MPSA_MODE_MIXED or MPSA_MODE_DIAG (each tile's
+ * statistic is that of the precision the tile runs in), plus
  *   skip_thresh   the factor above (scores are in log2 units with sm_scale folded in, as in the reference)
  *   skipped       NULL, or int32 [B,Hq,ceil(n/tile)]: number of key tiles skipped for each query tile
  */

@@ -117,7 +117,6 @@ static int attn_entry(const RawQ* rq, const uint8_t* q4, const uint8_t* qs4, con
     }
     if (routed) return attn_routed_launch(a, pv_dtype, st);
     if (skip) {
-        if (mixed) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: tile skipping is built for the mxfp4, mxfp8 and diag modes only");
         if (!(skip_thresh == skip_thresh)) return mpsa_fail(MPSA_EINVAL, "attn: skip_thresh is NaN");
         if (skipped && (reinterpret_cast<uintptr_t>(skipped) & 3)) return mpsa_fail(MPSA_EALIGN, "attn: skipped must be 4-byte aligned");
         return attn_skip_launch(a, pv_dtype, st);

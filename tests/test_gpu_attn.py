@@ -283,7 +283,8 @@ def _robust_thresh(q, k, v, **kw):
                                                   ("diag", True, 448, 64, 64), ("diag_e5", True, 640, 128, 64),
                                                   ("diag", False, 1024, 128, 128), ("diag", False, 1000, 128, 128),
                                                   ("diag_e5", False, 448, 64, 64), ("diag", False, 520, 128, 64),
-                                                  ("diag", False, 256, 128, 128)])
+                                                  ("diag", False, 256, 128, 128), ("mixed", True, 640, 128, 128),
+                                                  ("mixed_e5", False, 448, 64, 64)])
 def test_tile_skipping_follows_the_reference_rule(mode, causal, N, D, tile):
     """skip_thresh: key tile 0 always kept; tile j kept iff mean-of-row-maxima(j) >= skip_thresh * that of tile 0.  The kernel must skip
     exactly the tiles the oracle skips (counted per query tile) and match its output."""
@@ -296,8 +297,7 @@ def test_tile_skipping_follows_the_reference_rule(mode, causal, N, D, tile):
     q = q + 1.0                                                    # a common direction in q, a per-tile amount of it in k:
     k = k + torch.rand(nt, generator=g).repeat_interleave(tile)[:N].view(1, 1, N, 1) * 0.5     # tile statistics spread out
     q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
-    kw = dict(tile=tile, causal=causal, mode="diag" if mode.startswith("diag") else mode,
-              fmt8=O.FMT_E5M2 if mode.endswith("e5") else O.FMT_E4M3)
+    kw = dict(tile=tile, causal=causal, mode=mode.replace("_e5", ""), fmt8=O.FMT_E5M2 if mode.endswith("e5") else O.FMT_E4M3)
     th = _robust_thresh(q, k, v, **kw)
     want, want_sk = O.attn_mx(q, k, v, skip_thresh=th, return_skipped=True, **kw)
     got, sparsity = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=causal, block_scale_type=mode, tile=tile,
