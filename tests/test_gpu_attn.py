@@ -159,6 +159,52 @@ def test_step_under_hip_graph_capture_replays_like_eager():
         assert torch.equal(replayed, eager), f"replay {r}"
 
 
+def test_two_host_threads_on_two_streams():
+    """Distinct host threads may call the library on distinct streams: it keeps no pointers and no state besides a
+    thread-local error text.  Two threads run attention and a matmul side by side, 20 rounds each, on their own
+    streams and inputs; every result equals the one the same call gives alone.  An error raised in one thread leaves
+    the other thread's error text alone."""
+    import threading
+    from ours import _lib
+    from ours.block_scaled_matmul import block_scaled_matmul, quantize_block_scaled_from_tensor
+    jobs = []
+    for n, (N, mode) in enumerate([(1024, "diag"), (640, "mxfp4")]):
+        q, k, v = (t.to(DEV) for t in make_qkv(1, 8, 2, N, 128, seed=900 + n))
+        a = torch.randn(256, 512, generator=torch.Generator().manual_seed(n)).bfloat16().to(DEV)
+        ops = quantize_block_scaled_from_tensor(a, a, "mxfp8" if n else "mxfp4")
+        alone = mxfp_attn_kernel(q, k, v, is_causal=True, block_scale_type=mode, output_dtype=torch.bfloat16)
+        alone_mm = block_scaled_matmul(*ops[:4], torch.float32, 256, 256, 512, ops[4])
+        jobs.append((q, k, v, mode, ops, alone, alone_mm))
+    torch.cuda.synchronize()
+    failures = []
+
+    def worker(job):
+        q, k, v, mode, ops, alone, alone_mm = job
+        stream = torch.cuda.Stream()
+        try:
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    got = mxfp_attn_kernel(q, k, v, is_causal=True, block_scale_type=mode, output_dtype=torch.bfloat16)
+                    mm = block_scaled_matmul(*ops[:4], torch.float32, 256, 256, 512, ops[4])
+                    stream.synchronize()
+                    if not (torch.equal(got, alone) and torch.equal(mm, alone_mm)):
+                        failures.append(mode)
+                if mode == "diag":                                   # an argument error: this thread's text only
+                    rc = _lib.lib().mpsa_e2m1_decode(None, 4, None, None)
+                    assert rc != 0 and b"null" in _lib.lib().mpsa_last_error().lower()
+                else:
+                    assert _lib.lib().mpsa_last_error() in (b"", None) or b"null" not in _lib.lib().mpsa_last_error().lower()
+        except Exception as e:                                       # noqa: BLE001 -- reported by the main thread
+            failures.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(j,)) for j in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures
+
+
 def test_c4_long_context_full_shape():
     """B=1 Hq=32 Hkv=8 N=131072 D=128 causal with the outlier-channel scheme (seed 3), 128x128 tiles, diag: the whole
     problem runs on the GPU (16384 workgroups of the paired-tile kernel, 1024 key tiles deep).  The oracle checks
