@@ -60,29 +60,36 @@ WORKLOADS = {
     "c5": (1, 40, 40, 32760, 128, 128, 4, "C5 video-DiT B1 H40 N32760 (21 frames x 1560) D128 non-causal tile128 diag, sigma 0.5 + per-frame offsets"),
 }
 NON_CAUSAL = {"c5"}
+PLAIN_DRAWS = {"c1"}          # N(0,1) without outlier channels
+ROUTE_THRESH_DEFAULT = 0.9
 
 
-def make_inputs(B, Hq, Hkv, N, D, seed, device, dit_frames=0):
-    g = torch.Generator(device=device).manual_seed(seed)
+def make_inputs(B, Hq, Hkv, N, D, seed, device, dit_frames=0, outliers=True):
+    """The workload's q, k, v: drawn on the CPU from one seeded generator in float32, cast to bf16, copied to the device
+    -- bit for bit the tensors the parity tests hand to the CPU oracle and to the kernels (tests/conftest.py::make_qkv;
+    the video-DiT offsets as in tests/test_gpu_route.py).  Causal workloads: N(0,1) draws, and (``outliers``: C3, C4) per
+    head one channel (1 % of 128, rounded) of q and of k multiplied by 20.  ``dit_frames``: sigma 0.5 draws plus one sigma-0.5 offset per
+    frame and channel on q and on k (generator seed + 1)."""
+    g = torch.Generator().manual_seed(seed)
+    sigma = 0.5 if dit_frames else 1.0
+    q = torch.randn(B, Hq, N, D, generator=g) * sigma
+    k = torch.randn(B, Hkv, N, D, generator=g) * sigma
+    v = torch.randn(B, Hkv, N, D, generator=g) * sigma
+    if outliers and not dit_frames:
+        n_out = max(1, round(0.01 * D))
+        for t, H in ((q, Hq), (k, Hkv)):
+            for h in range(H):
+                idx = torch.randint(0, D, (n_out,), generator=g)
+                t[:, h, :, idx] *= 20.0
+    q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
     if dit_frames:
-        # video-DiT statistics: sigma 0.5 draws plus one offset per frame and channel on q and k
-        q = 0.5 * torch.randn(B, Hq, N, D, generator=g, device=device)
-        k = 0.5 * torch.randn(B, Hkv, N, D, generator=g, device=device)
-        v = 0.5 * torch.randn(B, Hkv, N, D, generator=g, device=device)
-        off = 0.5 * torch.randn(dit_frames, 1, D, generator=g, device=device)
-        q = (q.view(B, Hq, dit_frames, N // dit_frames, D) + off).view(B, Hq, N, D)
-        k = (k.view(B, Hkv, dit_frames, N // dit_frames, D) + off).view(B, Hkv, N, D)
-        return q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
-    q = torch.randn(B, Hq, N, D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
-    k = torch.randn(B, Hkv, N, D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
-    v = torch.randn(B, Hkv, N, D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
-    n_out = max(1, round(0.01 * D))
-    gc = torch.Generator().manual_seed(seed)
-    for t, H in ((q, Hq), (k, Hkv)):
-        for h in range(H):
-            idx = torch.randint(0, D, (n_out,), generator=gc).to(device)
-            t[:, h, :, idx] *= 20.0
-    return q, k, v
+        g2 = torch.Generator().manual_seed(seed + 1)
+        per = -(-N // dit_frames)
+        frame = torch.arange(N) // per
+        for t in (q, k):
+            off = 0.5 * torch.randn(dit_frames, 1, D, generator=g2)
+            t += off[frame].reshape(1, 1, N, D).to(t.dtype)
+    return q.to(device), k.to(device), v.to(device)
 
 
 def composite_peak_tflops(nt, causal=True):
@@ -196,6 +203,54 @@ def secondary_c4(device):
     }
 
 
+def secondary_c5(device):
+    """The video-DiT configuration (non-causal, N = 32760, 40 heads) next to the headline line: the diag mode's kernel and
+    whole step, and the routed mode (tile router on the scale bytes + routed attention) at the default thresholds with
+    the shares of tiles it sends to each precision."""
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, route_tiles
+    B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS["c5"]
+    q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 21)
+    out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
+    flops = 4.0 * B * Hq * N * N * D
+    comp = composite_peak_tflops((N + tile - 1) // tile, False)
+    iters = 10
+    res = {"workload": desc, "steps": iters}
+    for mode in ("diag", "routed"):
+        routed = mode == "routed"
+        ops = prepare_operands(q, k, v, tile, mode)
+        route = route_tiles(ops, False, ROUTE_THRESH_DEFAULT, None) if routed else None
+        attention_from_operands(ops, out, False, route=route)
+        torch.cuda.synchronize()
+        attn_ms = time_events(lambda: attention_from_operands(ops, out, False, route=route), iters)
+
+        def step():
+            o = prepare_operands(q, k, v, tile, mode, reuse=ops)
+            r = route_tiles(o, False, ROUTE_THRESH_DEFAULT, None) if routed else None
+            attention_from_operands(o, out, False, route=r)
+
+        step()
+        wait_for_device()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            step()
+        wait_for_device()
+        step_ms = (time.perf_counter() - t0) * 1e3 / iters
+        ktf, stf = flops / attn_ms / 1e9, flops / step_ms / 1e9
+        r = {"kernel_ms": round(attn_ms, 3), "kernel_TFLOP/s": round(ktf, 1), "kernel_frac_mxfp4_peak": round(ktf / PEAK_FP4_TFLOPS, 5),
+             "ms_per_step": round(step_ms, 3), "TFLOP/s": round(stf, 1), "frac_mxfp4_peak": round(stf / PEAK_FP4_TFLOPS, 5)}
+        if routed:
+            cls = route[0]
+            visited = float((cls != 255).sum())
+            r["route_thresh"] = ROUTE_THRESH_DEFAULT
+            r["tile_shares"] = {"mxfp8": round(float((cls == 2).sum()) / visited, 4), "mxfp4": round(float((cls == 1).sum()) / visited, 4),
+                                "skipped": round(float((cls == 0).sum()) / visited, 4)}
+        else:
+            r["kernel_frac_composite"] = round(ktf / comp, 5)
+        res[mode] = r
+        del ops, route
+    return res
+
+
 def secondary(device, quick):
     """Quantizer GB/s on the 8192x8192 GEMM operand and block-scaled GEMM TFLOP/s at 8192^3."""
     from ours import _lib
@@ -216,9 +271,12 @@ def secondary(device, quick):
     ms = time_events(lambda: quantize_mx_dual(a, 1.0), it)
     gbs = M * K * (2 + 0.5 + 1 + 2 / 32) / ms / 1e6
     out["quant_dual"] = {"GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4), "ms": round(ms, 4)}
-    for bst, fmt, peak in (("mxfp4", _lib.FMT_E2M1, PEAK_FP4_TFLOPS), ("mxfp8", _lib.FMT_E4M3, PEAK_FP8_TFLOPS)):
+    # "mixed" = the reference's 8-bit A against 4-bit B (ours/block_scaled_matmul.py:318-324); the matrix instruction runs
+    # it at the 8-bit rate
+    for bst, fmt, fmt_b, peak in (("mxfp4", _lib.FMT_E2M1, _lib.FMT_E2M1, PEAK_FP4_TFLOPS), ("mxfp8", _lib.FMT_E4M3, _lib.FMT_E4M3, PEAK_FP8_TFLOPS),
+                                  ("mixed", _lib.FMT_E4M3, _lib.FMT_E2M1, PEAK_FP8_TFLOPS)):
         ac, asc = quantize_mx(a, 1.0, fmt)
-        bc, bsc = quantize_mx(b, 1.0, fmt)
+        bc, bsc = quantize_mx(b, 1.0, fmt_b)
         cfg = make_configs(bst)
         # scales in the reference's packed form, packed outside the timed region as in the reference's own benchmark
         # (ours/block_scaled_matmul.py:299-406 packs, :409-441 times the matmul alone)
@@ -235,14 +293,23 @@ def mfma_stream_rates(device, seconds=0.05):
     operands and operands with random bits, for the bf16, MXFP4 and MXFP8 instructions the path uses."""
     import ctypes
     from ours import _lib
-    L = _lib.lib()
+    # the measurement kernel lives in a shared object of its own, next to the library (built by build.py)
+    path = os.path.join(os.path.dirname(_lib.LIB_PATH), "libmpsa_bench.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with `python mp-sparse-attn_amd/build.py`")
+    L = ctypes.CDLL(path)
+    L.bench_mfma_stream.restype = ctypes.c_int
+    L.bench_mfma_stream.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
     sink = torch.zeros(4, dtype=torch.float32, device=device)
     cus = torch.cuda.get_device_properties(device).multi_processor_count
     out = {}
     for name, kind, peak in (("bf16", 0, PEAK_BF16_TFLOPS), ("mxfp4", 1, PEAK_FP4_TFLOPS), ("mxfp8", 2, PEAK_FP8_TFLOPS)):
         for label, rnd in (("constant", 0), ("random", 1)):
             flop = ctypes.c_double(0.0)
-            run = lambda n: _lib.check(L.mpsa_bench_mfma_stream(kind, rnd, n, cus, _lib.ptr(sink), ctypes.byref(flop), _lib.stream_ptr(device)))
+            def run(n):
+                rc = L.bench_mfma_stream(kind, rnd, n, cus, _lib.ptr(sink), ctypes.byref(flop), _lib.stream_ptr(device))
+                if rc != 0:
+                    raise RuntimeError(f"bench_mfma_stream failed with {rc}")
             ms = time_events(lambda: run(2000), 2)
             iters = max(2000, int(2000 * seconds * 1e3 / max(ms, 1e-3)))
             ms = time_events(lambda: run(iters), 3)
@@ -268,7 +335,7 @@ def run_only(args, device):
     elif args.only == "attn":
         B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
         causal = args.workload not in NON_CAUSAL
-        q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21)
+        q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21, args.workload not in PLAIN_DRAWS)
         if args.operands != "random":     # every element the same: the clock the kernel gets without the operands' bit toggling
             q, k, v = (torch.full_like(t, 1.0 if args.operands == "ones" else 0.0) for t in (q, k, v))
         out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
@@ -318,13 +385,14 @@ def main():
     ap.add_argument("--mode", default="diag", choices=["diag", "mxfp4", "mxfp8", "routed"],
                     help="per-tile precision: diag (the headline configuration), one precision everywhere, or routed "
                          "(tile router on the scale bytes, thresholds below)")
-    ap.add_argument("--route-thresh", type=float, default=0.9, help="routed: 8-bit at or above this share of the row's largest tile statistic")
+    ap.add_argument("--route-thresh", type=float, default=ROUTE_THRESH_DEFAULT, help="routed: 8-bit at or above this share of the row's largest tile statistic")
     ap.add_argument("--skip-thresh", type=float, default=None, help="routed: skipped below this share")
     ap.add_argument("--spinup-ms", type=float, default=80.0, help="untimed device spin-up (steps run for this long) before the warm-up steps")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--no-fuse-q", action="store_true", help="with --only attn: hand the kernel quantized Q operands")
     ap.add_argument("--no-c4", action="store_true", help="leave the long-context figures out of `secondary`")
+    ap.add_argument("--no-c5", action="store_true", help="leave the video-DiT figures out of `secondary`")
     ap.add_argument("--eager", action="store_true", help="time plain launches instead of replaying the step as a HIP graph")
     ap.add_argument("--operands", default="random", choices=["random", "ones", "zeros"],
                     help="--only gemm4|gemm8|attn: the workload's random operands (default) or constant ones (the clock then stays up)")
@@ -358,7 +426,7 @@ def main():
         return
     B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
     causal = args.workload not in NON_CAUSAL
-    q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21)
+    q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21, args.workload not in PLAIN_DRAWS)
     out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
 
     routed = args.mode == "routed"
@@ -398,9 +466,11 @@ def main():
     # clock, and `--warmup 5` steps of 0.4 ms do not bring it up (measured: 20 timed steps read 0.42 ms/step without
     # this and 0.37 with it, the same as 500 timed steps).
     t_spin = time.perf_counter()
+    spin_steps = 0
     while (time.perf_counter() - t_spin) * 1e3 < args.spinup_ms:
         for _ in range(10):
             run_step()
+        spin_steps += 10
         wait_for_device()
     for _ in range(args.warmup):
         run_step()
@@ -411,6 +481,17 @@ def main():
     wait_for_device()
     dt = time.perf_counter() - t0
     ms_per_step = dt * 1e3 / args.steps
+    # the same steps as plain launches (no graph), for comparison with figures taken that way
+    eager_ms = None
+    if run_step is not step:
+        for _ in range(args.warmup):
+            step()
+        wait_for_device()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        wait_for_device()
+        eager_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     flops = (2.0 if causal else 4.0) * B * Hq * N * N * D
     tflops = flops / (ms_per_step * 1e-3) / 1e12
 
@@ -446,12 +527,14 @@ def main():
     result = {
         "metric": "MXFP attn TFLOPS + % of scaled-MFMA peak, causal N=8K/128K D=128, 1 GPU",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "warmup_effective_steps": args.warmup + spin_steps,
+        "ms_per_step": round(ms_per_step, 4), "ms_per_step_eager": None if eager_ms is None else round(eager_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "mxfp4/mxfp8 scores (E2M1/E4M3 + E8M0), bf16 P.V, f32 accumulate", "data": "synthetic",
         "config": {"workload": desc, "B": B, "Hq": Hq, "Hkv": Hkv, "N": N, "D": D, "tile": tile, "mode": args.mode,
                    "step": ("quantize K (dual) + V repack + fused attention with Q quantized in the kernel" if fuse_q else
                             "quantize Q,K (dual) + V repack + " + ("tile router + " if routed else "") + "fused attention"),
-                   "launch": launch, "spinup_ms": args.spinup_ms},
+                   "launch": launch, "spinup_ms": args.spinup_ms, "spinup_steps": spin_steps,
+                   "inputs": "CPU draw (torch.Generator seed %d), bit-identical to the parity tests' tensors" % seed},
         "frac_mxfp4_peak": round(tflops / PEAK_FP4_TFLOPS, 5),
         "roofline": roofline,
     }
@@ -470,6 +553,8 @@ def main():
             del ops, route
             state.clear()
             result["secondary"]["c4"] = secondary_c4(device)
+        if args.workload == "c3" and args.mode == "diag" and not args.no_c5:
+            result["secondary"]["c5"] = secondary_c5(device)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(q, k, v, tile, D, causal)
     else:

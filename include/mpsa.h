@@ -178,8 +178,9 @@ int mpsa_seq_mean_static(const void* x, int x_dtype, int64_t B, int64_t H, int64
  *            nearest even, overflow to infinity - the reference's output dtypes are f32, f16 and e5m2,
  *            ours/block_scaled_matmul.py:185-190, :273-280), leading dimension ldc elements
  *   M, N >= 1 (edge tiles are masked, as in the reference's kernel), K % 64 == 0.  Equal formats with M % 256 == 0,
- *   N % 256 == 0 and K % 128 == 0 run on the LDS-staged 256 x 256 kernel, every other case on a 128 x 128 kernel
- *   that reads its operands straight from L2 (same results; MPSA_GEMM_GENERAL=1 in the environment forces it).
+ *   N % 256 == 0 and K % 128 == 0, and an 8-bit A against a 4-bit B with K % 256 == 0 besides, run on the LDS-staged
+ *   256 x 256 kernel; every other case on a 128 x 128 kernel with masked edge tiles, LDS-staged too (two buffers,
+ *   direct-to-LDS loads).  Same results either way; MPSA_GEMM_GENERAL=1 in the environment forces the second.
  */
 int mpsa_gemm_mx(const uint8_t* a, const uint8_t* sa, int fmt_a, const uint8_t* b, const uint8_t* sb, int fmt_b,
                  int64_t M, int64_t N, int64_t K, void* c, int c_dtype, int64_t ldc, mpsa_stream_t stream);
@@ -341,16 +342,6 @@ int mpsa_attn_fwd_routed(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q
                          const void* v_tiles, int pv_dtype, void* o, int o_dtype, const int64_t o_strides[4],
                          int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t nk, int64_t D, int tile, int causal,
                          const int32_t* order, const int32_t* counts, mpsa_stream_t stream);
-
-/*
- * Measurement aid (no counterpart in the reference): a register-resident stream of matrix instructions, two waves per
- * SIMD, `blocks` workgroups, iters x 16 instructions per wave.  kind 0: v_mfma_f32_32x32x16_bf16; 1:
- * v_mfma_scale_f32_32x32x64_f8f6f4 on E2M1 operands; 2: the same on E4M3 operands.  random_bits != 0 fills the operand
- * registers with pseudo-random bits instead of one constant: the chip's power management then runs the same stream at
- * a lower clock, which is the rate a real matmul can at best sustain.  *flop receives the launch's FLOP count; time it
- * with events on `stream`.  sink: any 4 writable device bytes.
- */
-int mpsa_bench_mfma_stream(int kind, int random_bits, int iters, int blocks, float* sink, double* flop, mpsa_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -142,13 +142,14 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                     amax = max_lane_pair(amax);                                // the other half of the block sits in lane ^ 32
                     const bool zero = mpsa_f2u(amax) == 0u;
                     const int se = block_exponent(amax) - 7;                   // emax of the 8-bit formats: ours/quant_mxint8.py:191
-                    // (the quantizer clamps to the format's maximum here; with the block maximum scaled into
-                    // [128, 256) that clamp never changes a value, so it is left out)
+                    // the quantizer's clamp to the format's maximum (quantize_kernel.h): finite blocks scale into
+                    // [128, 256) and never meet it, a block with an infinity saturates there instead of giving NaN codes
+                    const float lim = (FMT8 == MPSA_FMT_E4M3) ? 448.0f : 57344.0f;
 #pragma unroll
                     for (int c = 0; c < 2; ++c) {
                         float y[8];
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) y[e] = ldexpf(x[c][e], -se);
+                        for (int e = 0; e < 8; ++e) y[e] = __builtin_fminf(__builtin_fmaxf(ldexpf(x[c][e], -se), -lim), lim);
                         w[4 * blk + 2 * c] = zero ? 0 : (int)fp8_pack4<FMT8, false>(y[0], y[1], y[2], y[3]);
                         w[4 * blk + 2 * c + 1] = zero ? 0 : (int)fp8_pack4<FMT8, false>(y[4], y[5], y[6], y[7]);
                     }

@@ -2,8 +2,15 @@
 // chip -- the practical ceiling next to the datasheet peaks that the rooflines are quoted against.  MI355X manages its
 // clock by power: the same instruction stream runs near 2.4 GHz on constant operands and several hundred MHz lower on
 // operands with random bits, so a kernel's distance from the datasheet peak is partly not the kernel's.  No counterpart in
-// the reference; bench.py --only mfma uses it.
-#include "mpsa_common.h"
+// the reference.  Built into its own shared object (lib/libmpsa_bench.so), which only bench.py loads: it is a
+// measurement, not part of the library's interface.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 namespace {
 
@@ -52,14 +59,15 @@ __global__ __launch_bounds__(512, 1) void mfma_stream_kernel(float* sink, int it
 }  // namespace
 
 // Launches `blocks` workgroups of 8 waves (two per SIMD); every wave issues iters x 16 matrix instructions.
-// Returns the FLOP of the launch through *flop (2 x 32 x 32 x K per instruction).
-extern "C" int mpsa_bench_mfma_stream(int kind, int random_bits, int iters, int blocks, float* sink, double* flop, mpsa_stream_t stream) {
-    if (kind < 0 || kind > 2 || iters <= 0 || blocks <= 0 || !sink) return mpsa_fail(MPSA_EINVAL, "mfma_stream: bad argument");
+// Returns 0, -1 for a bad argument or -4 for a failed launch, and the FLOP of the launch through *flop
+// (2 x 32 x 32 x K per instruction).
+extern "C" int bench_mfma_stream(int kind, int random_bits, int iters, int blocks, float* sink, double* flop, void* stream) {
+    if (kind < 0 || kind > 2 || iters <= 0 || blocks <= 0 || !sink) return -1;
     hipStream_t st = (hipStream_t)stream;
     if (kind == 0)      hipLaunchKernelGGL(mfma_stream_kernel<0>, dim3(blocks), dim3(512), 0, st, sink, iters, random_bits);
     else if (kind == 1) hipLaunchKernelGGL(mfma_stream_kernel<1>, dim3(blocks), dim3(512), 0, st, sink, iters, random_bits);
     else                hipLaunchKernelGGL(mfma_stream_kernel<2>, dim3(blocks), dim3(512), 0, st, sink, iters, random_bits);
-    MPSA_CHECK_LAUNCH("mfma_stream");
+    if (hipGetLastError() != hipSuccess) return -4;
     if (flop) *flop = (double)blocks * 8.0 * iters * 16.0 * 2.0 * 32 * 32 * (kind == 0 ? 16 : 64);
-    return MPSA_OK;
+    return 0;
 }

@@ -94,14 +94,21 @@ __device__ __forceinline__ void load_to_lds(uint32_t lane_off, const uint8_t* wa
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(base), "v"(lane_off), "s"(gb) : "memory", "m0");
 }
 
-template <int FMT, typename OutT, bool WIDE, bool PK, bool PAIR>
+// FMT: element format of A (and of B, unless FMTB says otherwise).  FMTB == E2M1 under an 8-bit FMT is the reference's
+// "mixed" type (ours/block_scaled_matmul.py:318-324): everything follows the 8-bit geometry -- a stage is 64 elements
+// of K, a unit 128 -- except B's codes, which are half as wide: 32 bytes per row and stage, a unit's image 64-byte rows.
+template <int FMT, int FMTB, typename OutT, bool WIDE, bool PK, bool PAIR>
 __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     static_assert(!(WIDE && PK), "packed scales use the per-stage scale area");
     static_assert(NSTAGE == 4, "PAIR: the ring is two units of two stages");
     constexpr bool FP4 = (FMT == MPSA_FMT_E2M1);
+    constexpr bool B4 = !FP4 && (FMTB == MPSA_FMT_E2M1);       // 8-bit A against 4-bit B
+    static_assert(FMT == FMTB || B4, "the operands share a format, or A is 8-bit and B is E2M1");
+    static_assert(!B4 || PAIR, "mixed formats: K % 128 == 0, so the stage count is even");
     constexpr int STAGE_BYTES = stage_bytes<WIDE>();
     constexpr int GROUP = FP4 ? 4 : 8;                 // stages covered by 16 scale bytes of a row
-    const int row_bytes = FP4 ? g.K / 2 : g.K;         // code bytes per matrix row
+    const int row_bytes = FP4 ? g.K / 2 : g.K;         // code bytes per matrix row (of A)
+    const int row_bytes_b = B4 ? g.K / 2 : row_bytes;  // and of B
     const int srow_bytes = g.K / 32;
     const int KT = row_bytes / ROWB;
 
@@ -141,7 +148,7 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     const int64_t zb = (int64_t)bb * g.heads_b + ha / (g.heads_a / g.heads_b);
     g.a += (int64_t)bz * g.M * row_bytes;
     g.sa += (int64_t)bz * g.M * srow_bytes;
-    g.b += zb * g.N * row_bytes;
+    g.b += zb * g.N * row_bytes_b;
     g.sb += zb * g.N * srow_bytes;
     // lane offsets inside a tile's operand (the same for A and B) and inside its scale rows; tile bases are scalar
     // PAIR: a unit = two consecutive stages = 128 code bytes per row, fetched as whole cache lines: an instruction
@@ -166,9 +173,20 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
             lo[c] = (uint32_t)row * (uint32_t)row_bytes + cb * 16;
         }
     }
+    // mixed formats: a unit of B is 64 bytes per row, fetched like a stage of the stage-by-stage ring (four
+    // instructions per wave, row's piece c at slot c ^ ((row >> 2) & 3))
+    uint32_t lob[4] = {0, 0, 0, 0};
+    if constexpr (B4) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int p = (wave * 4 + c) * 64 + lane;
+            const int row = p >> 2, slot = p & 3;
+            lob[c] = (uint32_t)row * (uint32_t)row_bytes_b + (slot ^ ((row >> 2) & 3)) * 16;
+        }
+    }
     const uint32_t los = (uint32_t)(wave * 64 + lane) * (uint32_t)srow_bytes;
     const uint8_t* const a_base = g.a + (int64_t)m0 * row_bytes;
-    const uint8_t* const b_base = g.b + (int64_t)n0 * row_bytes;
+    const uint8_t* const b_base = g.b + (int64_t)n0 * row_bytes_b;
     const uint8_t* const sa_base = g.sa + (int64_t)m0 * srow_bytes;
     const uint8_t* const sb_base = g.sb + (int64_t)n0 * srow_bytes;
     // packed scales (the reference's [rows/128, K/128, 32, 4, 4] form, ours/mxfp_attn_kernel.py:56-57): the scale bytes
@@ -192,8 +210,9 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
             const int c2 = part * 2 + q, x = wave * 8 + c2;
             const int64_t go = (int64_t)uc * (2 * ROWB) + (int64_t)x * 8 * row_bytes;
             load_to_lds<16>(lo[q], a_base + go, ub + x * 1024);
-            load_to_lds<16>(lo[q], b_base + go, ub + 2 * OP_BYTES + x * 1024);
+            if constexpr (!B4) load_to_lds<16>(lo[q], b_base + go, ub + 2 * OP_BYTES + x * 1024);
         }
+        if constexpr (B4) load_to_lds<16>(lob[part], b_base + (int64_t)uc * ROWB, ub + 2 * OP_BYTES + (wave * 4 + part) * 1024);
         if (part != 3) return;
         uint8_t* sc = ub + 4 * OP_BYTES;
         if constexpr (PK) {
@@ -272,7 +291,10 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int ra_ = wm * 128 + i * 32 + r, rb_ = wn * 128 + i * 32 + r;
-        if constexpr (PAIR) {
+        if constexpr (B4) {
+            offa[i] = ra_ * 2 * ROWB; swz_a[i] = (ra_ >> 1) & 7;
+            offb[i] = rb_ * ROWB; swz_b[i] = (rb_ >> 2) & 3;
+        } else if constexpr (PAIR) {
             offa[i] = ra_ * 2 * ROWB; swz_a[i] = (ra_ >> 1) & 7;
             offb[i] = rb_ * 2 * ROWB; swz_b[i] = (rb_ >> 1) & 7;
         } else {
@@ -338,6 +360,10 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
             if constexpr (FP4) {
                 const v4i x = *reinterpret_cast<const v4i*>(lx + off + (((c0 + 2 * s + h) ^ swz) * 16));
                 fx = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+            } else if (B4 && isb) {
+                // the 4-bit operand of a mixed product: stage hh of the unit is pieces 2hh, 2hh + 1 of the 64-byte row
+                const v4i x = *reinterpret_cast<const v4i*>(lx + off + (((2 * hh + h) ^ swz) * 16));
+                fx = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
             } else {
                 // 8-bit operands: registers 0-3 of both lane halves form MX block 0 (scaled by the byte
                 // lane half 0 supplies), registers 4-7 form block 1 (scaled by lane half 1's byte)
@@ -351,8 +377,8 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     auto multiply_row = [&](const Frag& f, int i, bool odd) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            if (odd) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMT, 2, f.sa[i], 2, f.sb[j]);
-            else     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMT, 0, f.sa[i], 0, f.sb[j]);
+            if (odd) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMTB, 2, f.sa[i], 2, f.sb[j]);
+            else     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.a[i], f.b[j], acc[i][j], FMT, FMTB, 0, f.sa[i], 0, f.sb[j]);
         }
     };
     // One step: the 16 matrix instructions on operand set `cur`, in four rows.  Between them go the LDS reads
@@ -419,7 +445,7 @@ __global__ __launch_bounds__(256, 1) void gemm_mx_kernel(GemmArgs g) {
     {
         // stages 1 .. NSTAGE-1 stay in flight (packed 8-bit: only stage 2 of them carries scale loads)
         // PAIR: unit 1 stays in flight (16 code loads and its scale loads: none, one, or four)
-        constexpr int KEEP = PAIR ? 2 * CODE_LOADS + (WIDE ? 0 : PK ? 1 : 4)
+        constexpr int KEEP = PAIR ? (B4 ? CODE_LOADS + CODE_LOADS / 2 : 2 * CODE_LOADS) + (WIDE ? 0 : PK ? 1 : 4)
                            : WIDE ? (NSTAGE - 1) * CODE_LOADS : PK ? (FP4 ? (NSTAGE - 1) * (CODE_LOADS + 1) : (NSTAGE - 1) * CODE_LOADS + 1) : (NSTAGE - 1) * (CODE_LOADS + 2);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(wait_imm(KEEP));
@@ -734,43 +760,43 @@ bool force_general() {
     return on;
 }
 
-template <int FMT, typename OutT, bool WIDE, bool PK, bool PAIR>
+template <int FMT, int FMTB, typename OutT, bool WIDE, bool PK, bool PAIR>
 struct GemmLds {
     static inline const bool registered =
-        mpsa_register_lds_kernel(reinterpret_cast<const void*>(gemm_mx_kernel<FMT, OutT, WIDE, PK, PAIR>), smem_bytes<WIDE>());
+        mpsa_register_lds_kernel(reinterpret_cast<const void*>(gemm_mx_kernel<FMT, FMTB, OutT, WIDE, PK, PAIR>), smem_bytes<WIDE>());
 };
 
-template <int FMT, typename OutT, bool WIDE, bool PK, bool PAIR>
+template <int FMT, int FMTB, typename OutT, bool WIDE, bool PK, bool PAIR>
 void launch_kernel(const GemmArgs& g, dim3 grid, hipStream_t st) {
-    if (!GemmLds<FMT, OutT, WIDE, PK, PAIR>::registered) return;
-    hipLaunchKernelGGL((gemm_mx_kernel<FMT, OutT, WIDE, PK, PAIR>), grid, dim3(256), smem_bytes<WIDE>(), st, g);
+    if (!GemmLds<FMT, FMTB, OutT, WIDE, PK, PAIR>::registered) return;
+    hipLaunchKernelGGL((gemm_mx_kernel<FMT, FMTB, OutT, WIDE, PK, PAIR>), grid, dim3(256), smem_bytes<WIDE>(), st, g);
 }
 
-template <int FMT, typename OutT, bool PAIR>
+template <int FMT, int FMTB, typename OutT, bool PAIR>
 void launch_scales(const GemmArgs& g, dim3 grid, hipStream_t st) {
-    if (g.packed)            launch_kernel<FMT, OutT, false, true, PAIR>(g, grid, st);
-    else if (g.K % 512 == 0) launch_kernel<FMT, OutT, true, false, PAIR>(g, grid, st);
-    else                     launch_kernel<FMT, OutT, false, false, PAIR>(g, grid, st);
+    if (g.packed)            launch_kernel<FMT, FMTB, OutT, false, true, PAIR>(g, grid, st);
+    else if (g.K % 512 == 0) launch_kernel<FMT, FMTB, OutT, true, false, PAIR>(g, grid, st);
+    else                     launch_kernel<FMT, FMTB, OutT, false, false, PAIR>(g, grid, st);
 }
 
-template <int FMT, typename OutT>
+template <int FMT, int FMTB, typename OutT>
 void launch_one(const GemmArgs& g, dim3 grid, hipStream_t st) {
     // whole cache lines per row (two stages at a time) need an even number of stages: always so with 8-bit codes
     // (K % 128 == 0), with 4-bit codes when K % 256 == 0
     if constexpr (FMT != MPSA_FMT_E2M1) {
-        launch_scales<FMT, OutT, true>(g, grid, st);
+        launch_scales<FMT, FMTB, OutT, true>(g, grid, st);
     } else {
-        if (g.K % 256 == 0) launch_scales<FMT, OutT, true>(g, grid, st);
-        else                launch_scales<FMT, OutT, false>(g, grid, st);
+        if (g.K % 256 == 0) launch_scales<FMT, FMTB, OutT, true>(g, grid, st);
+        else                launch_scales<FMT, FMTB, OutT, false>(g, grid, st);
     }
 }
 
-template <int FMT>
+template <int FMT, int FMTB>
 void launch_fmt(const GemmArgs& g, int c_dtype, dim3 grid, hipStream_t st) {
-    if (c_dtype == MPSA_BF16)      launch_one<FMT, __bf16>(g, grid, st);
-    else if (c_dtype == MPSA_F8E5M2) launch_one<FMT, OutE5M2>(g, grid, st);
-    else if (c_dtype == MPSA_F16)  launch_one<FMT, _Float16>(g, grid, st);
-    else                           launch_one<FMT, float>(g, grid, st);
+    if (c_dtype == MPSA_BF16)      launch_one<FMT, FMTB, __bf16>(g, grid, st);
+    else if (c_dtype == MPSA_F8E5M2) launch_one<FMT, FMTB, OutE5M2>(g, grid, st);
+    else if (c_dtype == MPSA_F16)  launch_one<FMT, FMTB, _Float16>(g, grid, st);
+    else                           launch_one<FMT, FMTB, float>(g, grid, st);
 }
 
 }  // namespace
@@ -800,12 +826,14 @@ static int gemm_entry(const uint8_t* a, const uint8_t* sa, int fmt_a, const uint
     hipStream_t st = (hipStream_t)stream;
     const int rc = mpsa_ensure_init();
     if (rc != MPSA_OK) return rc;
-    // whole 256 x 256 tiles of one element format: the LDS-staged kernel; everything else: the general one
-    if (fmt_a == fmt_b && M % BM == 0 && N % BN == 0 && K % 128 == 0 && !force_general()) {
+    // whole 256 x 256 tiles of one element format, or of an 8-bit A against a 4-bit B (the reference's "mixed" type):
+    // the LDS-staged kernel; everything else: the general one
+    const bool mixed = fmt_a != MPSA_FMT_E2M1 && fmt_b == MPSA_FMT_E2M1;
+    if ((fmt_a == fmt_b || mixed) && M % BM == 0 && N % BN == 0 && K % 128 == 0 && !force_general()) {
         dim3 grid((unsigned)((M / BM) * (N / BN)), (unsigned)(batch * heads_a));
-        if (fmt_a == MPSA_FMT_E2M1)      launch_fmt<MPSA_FMT_E2M1>(g, c_dtype, grid, st);
-        else if (fmt_a == MPSA_FMT_E4M3) launch_fmt<MPSA_FMT_E4M3>(g, c_dtype, grid, st);
-        else                             launch_fmt<MPSA_FMT_E5M2>(g, c_dtype, grid, st);
+        if (fmt_a == MPSA_FMT_E2M1)      launch_fmt<MPSA_FMT_E2M1, MPSA_FMT_E2M1>(g, c_dtype, grid, st);
+        else if (fmt_a == MPSA_FMT_E4M3) mixed ? launch_fmt<MPSA_FMT_E4M3, MPSA_FMT_E2M1>(g, c_dtype, grid, st) : launch_fmt<MPSA_FMT_E4M3, MPSA_FMT_E4M3>(g, c_dtype, grid, st);
+        else                             mixed ? launch_fmt<MPSA_FMT_E5M2, MPSA_FMT_E2M1>(g, c_dtype, grid, st) : launch_fmt<MPSA_FMT_E5M2, MPSA_FMT_E5M2>(g, c_dtype, grid, st);
     } else {
         dim3 grid((unsigned)(((M + 127) / 128) * ((N + 127) / 128)), (unsigned)(batch * heads_a));
         launch_general(g, fmt_a, fmt_b, c_dtype, grid, st);

@@ -53,7 +53,6 @@ SIGNATURES = {
     "mpsa_attn_fwd_q16_supported": (_int, [_i64, _i64, _i64, _i64, _i64, _int, _int, _int]),
     "mpsa_attn_fwd_skip": (_int, [_vp] * 8 + [_int, _vp, _int, _vp, _int, _p64,
                                   _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _vp, _vp]),
-    "mpsa_bench_mfma_stream": (_int, [_int, _int, _int, _int, _vp, ctypes.POINTER(ctypes.c_double), _vp]),
     "mpsa_route_workspace": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
     "mpsa_route_tiles": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _f32, _f32, _vp, _vp, _vp, _vp, _vp]),
     "mpsa_attn_fwd_routed": (_int, [_vp] * 8 + [_int, _vp, _int, _vp, _int, _p64,
@@ -85,14 +84,14 @@ def lib():
             fn.restype = res
             fn.argtypes = args
         _lib = handle
-        # per-device set-up up front, so that even a caller's first launch can be captured into a HIP graph
-        # (no device here means no set-up: the entry points report their own errors)
+        # set-up of the current device up front, so that even a caller's first launch there can be captured into a HIP
+        # graph.  Other devices are set up by the entry points on their first use (mpsa_ensure_init); a caller that wants
+        # to capture a first call on another device calls mpsa_init() with that device current.  (No device here means no
+        # set-up: the entry points report their own errors.)
         if torch.cuda.is_available():
-            for dev in range(torch.cuda.device_count()):
-                with torch.cuda.device(dev):
-                    status = handle.mpsa_init()
-                if status != 0:
-                    raise MpsaError(status, handle.mpsa_last_error().decode("utf-8", "replace"))
+            status = handle.mpsa_init()
+            if status != 0:
+                raise MpsaError(status, handle.mpsa_last_error().decode("utf-8", "replace"))
     return _lib
 
 

@@ -13,6 +13,9 @@ import torch
 
 from . import _lib
 from .block_scaled_matmul import VEC_SIZE, _fmts_of, unpack_scale_5d
+# the reference defines the batched packaging here (ours/batched_block_scaled_matmul.py:239) and again, identically, next
+# to its attention kernel (ours/mxfp_attn_kernel.py:426); both names are one function in this package
+from .mxfp_attn_kernel import initialize_block_scaled_batched_from_tensor  # noqa: F401
 
 
 def block_scaled_batched_matmul(a, a_scale, b, b_scale, dtype_dst, B, H, M, N, K, configs):

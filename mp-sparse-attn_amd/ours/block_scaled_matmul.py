@@ -120,16 +120,33 @@ def fp8_cast(x, fmt8):
     return out
 
 
+E4M3_MAX = 448.0
+
+
 def _package_operand(t, four_bit, fmt8):
     """One operand of the reference's packaging: 8-bit -> the elementwise FP8 cast (ours/block_scaled_matmul.py:334-336);
     4-bit -> ``MXFP4Tensor`` codes packed two per byte along K (:338-345; uint8 input is taken as ready-made codes, one
-    per byte, which is what the reference's constructor call accepts; float input is encoded first)."""
+    per byte, which is what the reference's constructor call accepts; float input is encoded first).  Returns
+    ``(bytes for the kernel, decoded float32 values)`` -- the second is what the reference calls ``a_ref``.
+
+    The reference's 8-bit cast is E5M2 (largest finite value 57344); under this package's ``"mxfp8"`` / ``"mixed"``
+    the cast is E4M3, where torch's cast -- and ``mpsa_fp8_encode`` -- turns every magnitude above 464 into NaN, so
+    float input beyond +-448 is refused here with a pointer to the E5M2 types instead of being packaged as NaN."""
     if not four_bit:
-        if t.dtype in (torch.float8_e5m2, torch.float8_e4m3fn, torch.uint8):
-            return t.view(torch.uint8)
-        return fp8_cast(t, fmt8)
-    codes = MXFP4Tensor(data=t, dtype=torch.uint8) if t.dtype == torch.uint8 else MXFP4Tensor(data=t.to(torch.float32))
-    return codes.to_packed_tensor(dim=t.dim() - 1)
+        if t.dtype in (torch.float8_e5m2, torch.float8_e4m3fn):
+            want = torch.float8_e5m2 if fmt8 == _lib.FMT_E5M2 else torch.float8_e4m3fn
+            assert t.dtype == want, f"operand is {t.dtype} but the block scale type asks for {want}"
+            codes = t.view(torch.uint8)
+        elif t.dtype == torch.uint8:
+            codes = t
+        else:
+            if fmt8 == _lib.FMT_E4M3 and bool((t.abs() > E4M3_MAX).any()):
+                raise ValueError("values beyond +-448 do not fit E4M3 (this package's \"mxfp8\" / \"mixed\"); the "
+                                 "reference casts to E5M2: use block_scale_type \"mxfp8e5\" / \"mixed_e5\"")
+            codes = fp8_cast(t, fmt8)
+        return codes, lambda: codes.view(torch.float8_e5m2 if fmt8 == _lib.FMT_E5M2 else torch.float8_e4m3fn).to(torch.float32)
+    fp4 = MXFP4Tensor(data=t, dtype=torch.uint8) if t.dtype == torch.uint8 else MXFP4Tensor(data=t.to(torch.float32))
+    return fp4.to_packed_tensor(dim=t.dim() - 1), lambda: fp4.to(torch.float32)
 
 
 def _package_scale(s):
@@ -140,6 +157,15 @@ def _package_scale(s):
     return MXScaleTensor(s.to(torch.float32)).data
 
 
+def _expanded_scales(packed_bytes, K):
+    """E8M0 bytes in the packed layout -> float32 factors, one per element: ``unpack_scale`` + ``repeat_interleave``
+    of the reference (ours/block_scaled_matmul.py:382-388), on the device (``mpsa_scales_from_5d``,
+    ``mpsa_e8m0_decode``)."""
+    holder = MXScaleTensor(size=(1,), device=packed_bytes.device)
+    holder.data = unpack_scale_5d(packed_bytes)
+    return holder.to(torch.float32).repeat_interleave(VEC_SIZE, dim=-1)[..., :K]
+
+
 def initialize_block_scaled_from_tensor(a_tensor, b_tensor, a_scale, b_scale, block_scale_type="mxfp4", compute_reference=False):
     """Operand packaging with the reference's signature (ours/block_scaled_matmul.py:299-406).
 
@@ -148,14 +174,13 @@ def initialize_block_scaled_from_tensor(a_tensor, b_tensor, a_scale, b_scale, bl
     (encoded to E8M0 with ``MXScaleTensor``) or uint8.  ``block_scale_type``: ``"mxfp4"``, ``"mxfp8"`` (E4M3),
     ``"mixed"`` (8-bit A x 4-bit B), ``"mxfp8e5"`` / ``"mixed_e5"`` (E5M2, the reference's cast).  ``"nvfp4"`` (16-element
     blocks with FP8 scales) has no counterpart on the CDNA4 scaled matrix cores and raises.
-    Returns ``(a, a_scale, b, b_scale, configs, None)``; ``compute_reference=True`` raises -- the library carries no
-    second implementation to compare with."""
+    Returns ``(a, a_scale, b, b_scale, configs, reference)``; ``reference`` is None, or with ``compute_reference`` the
+    reference's triple ``(dq(A) @ dq(B)^T, dq(A), dq(B))`` in float32 (:376-392, :404), computed on the device from
+    the packaged bytes: codes decoded, E8M0 bytes decoded and repeated over their 32 elements, ``torch.matmul``."""
     if block_scale_type == "nvfp4":
         raise NotImplementedError("nvfp4 (16-element blocks, FP8 scale factors) is not available: the gfx950 scaled matrix "
                                   "instructions take one E8M0 scale per 32 elements")
     assert block_scale_type in _TYPES, f"Invalid block scale type: {block_scale_type}"
-    if compute_reference:
-        raise NotImplementedError("compute_reference is not available: use the test-suite's CPU oracle")
     M, K = a_tensor.shape
     N, K_b = b_tensor.shape
     assert K == K_b, f"matrix dimensions do not match: A.shape[1]={K} != B.shape[1]={K_b}"
@@ -166,9 +191,32 @@ def initialize_block_scaled_from_tensor(a_tensor, b_tensor, a_scale, b_scale, bl
     configs = make_configs(block_scale_type)
     fmt_a, fmt_b = _fmts_of(configs)
     f8 = fmt_a if fmt_a != _lib.FMT_E2M1 else _lib.FMT_E4M3
-    a = _package_operand(a_tensor, fmt_a == _lib.FMT_E2M1, f8)
-    b = _package_operand(b_tensor, fmt_b == _lib.FMT_E2M1, f8)
-    return a, _package_scale(a_scale), b, _package_scale(b_scale), configs, None
+    a, a_ref = _package_operand(a_tensor, fmt_a == _lib.FMT_E2M1, f8)
+    b, b_ref = _package_operand(b_tensor, fmt_b == _lib.FMT_E2M1, f8)
+    a_scale, b_scale = _package_scale(a_scale), _package_scale(b_scale)
+    reference = None
+    if compute_reference:
+        a_dq = a_ref() * _expanded_scales(a_scale, K)
+        b_dq = b_ref() * _expanded_scales(b_scale, K)
+        reference = (torch.matmul(a_dq, b_dq.T), a_dq, b_dq)
+    return a, a_scale, b, b_scale, configs, reference
+
+
+def validate_block_scaled_from_tensor(M, N, K, block_scale_type="mxfp4", device="cuda"):
+    """The reference's self-check (ours/block_scaled_matmul.py:409-441): random fp16 operands and float scale factors
+    ``rand + 1e-8`` in the packed layout, packaged with ``compute_reference=True``, multiplied to fp16, and compared
+    with the fake-quant product under the reference's bound (``assert_close``, atol = rtol = 1e-3).  Returns
+    ``(reference, output)``."""
+    a_tensor = torch.randn((M, K), dtype=torch.float16, device=device)
+    b_tensor = torch.randn((N, K), dtype=torch.float16, device=device)
+    epsilon = 1e-8
+    a_scale_tensor = torch.rand((M // 128, K // VEC_SIZE // 4, 32, 4, 4), device=device) + epsilon
+    b_scale_tensor = torch.rand((N // 128, K // VEC_SIZE // 4, 32, 4, 4), device=device) + epsilon
+    a_desc, a_scale, b_desc, b_scale, configs, reference = initialize_block_scaled_from_tensor(
+        a_tensor, b_tensor, a_scale_tensor, b_scale_tensor, block_scale_type, compute_reference=True)
+    output = block_scaled_matmul(a_desc, a_scale, b_desc, b_scale, torch.float16, M, N, K, configs)
+    torch.testing.assert_close(reference[0], output.to(torch.float32), atol=1e-3, rtol=1e-3)
+    return reference[0], output
 
 
 def quantize_block_scaled_from_tensor(a_tensor, b_tensor, block_scale_type="mxfp4", packed_scales=False):

@@ -157,14 +157,15 @@ def initialize_block_scaled_batched_from_tensor(a_tensor, b_tensor, a_scale, b_s
     code per byte, or FP8 bytes) or float values, which are cast element by element; ``a_scale`` / ``b_scale``:
     ``[B,H,rows/128,K/128,32,4,4]`` scale factors, uint8 E8M0 bytes (taken as they are, :505-506) or float (encoded
     with ``MXScaleTensor``).  4-bit codes are packed two per byte along K (the last dim).  Returns
-    ``(a, a_scale, b, b_scale, configs, (None, None, None))``; ``compute_reference=True`` raises."""
-    from .block_scaled_matmul import _TYPES, _fmts_of, _package_operand, _package_scale, make_configs, VEC_SIZE
+    ``(a, a_scale, b, b_scale, configs, reference)``; ``reference`` is ``(None, None, None)``, or with
+    ``compute_reference`` the reference's triple (:508-551): the float32 scores ``dq(A) @ dq(B)^T`` ``[B,H,M,N]`` (codes
+    decoded, E8M0 bytes decoded and repeated over their 32 elements, ``torch.matmul``, all on the device) and the
+    decoded codes of A and B without their scale factors, as the reference returns them."""
+    from .block_scaled_matmul import _TYPES, _fmts_of, _package_operand, _package_scale, _expanded_scales, make_configs, VEC_SIZE
     if block_scale_type == "nvfp4":
         raise NotImplementedError("nvfp4 (16-element blocks, FP8 scale factors) is not available: the gfx950 scaled matrix "
                                   "instructions take one E8M0 scale per 32 elements")
     assert block_scale_type in _TYPES, f"Invalid block scale type: {block_scale_type}"
-    if compute_reference:
-        raise NotImplementedError("compute_reference is not available: use the test-suite's CPU oracle")
     B, H, M, K = a_tensor.shape
     B_b, H_b, N, K_b = b_tensor.shape
     assert B == B_b, f"batch sizes do not match: A.shape[0]={B} != B.shape[0]={B_b}"
@@ -178,9 +179,16 @@ def initialize_block_scaled_batched_from_tensor(a_tensor, b_tensor, a_scale, b_s
     configs["BLOCK_SIZE_M"] = configs["BLOCK_SIZE_N"] = 128
     fmt_a, fmt_b = _fmts_of(configs)
     f8 = fmt_a if fmt_a != _lib.FMT_E2M1 else _lib.FMT_E4M3
-    a = _package_operand(a_tensor, fmt_a == _lib.FMT_E2M1, f8)
-    b = _package_operand(b_tensor, fmt_b == _lib.FMT_E2M1, f8)
-    return a, _package_scale(a_scale), b, _package_scale(b_scale), configs, (None, None, None)
+    a, a_ref = _package_operand(a_tensor, fmt_a == _lib.FMT_E2M1, f8)
+    b, b_ref = _package_operand(b_tensor, fmt_b == _lib.FMT_E2M1, f8)
+    a_scale, b_scale = _package_scale(a_scale), _package_scale(b_scale)
+    reference = (None, None, None)
+    if compute_reference:
+        a_dec, b_dec = a_ref(), b_ref()
+        a_dq = a_dec * _expanded_scales(a_scale, K)
+        b_dq = (b_dec * _expanded_scales(b_scale, K)).repeat_interleave(H // H_b, dim=1)     # grouped heads
+        reference = (torch.matmul(a_dq, b_dq.transpose(-1, -2)), a_dec, b_dec)
+    return a, a_scale, b, b_scale, configs, reference
 
 
 def block_scaled_batched_attn(a_desc, a_scale, b_desc, b_scale, v_ori, dtype_dst, B, H, M, N, K, configs, STAGE=1, skip_thresh=None):

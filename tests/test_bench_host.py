@@ -43,3 +43,27 @@ def test_traffic_comes_from_the_profile_summary():
     assert b.measured_traffic("c3", "no-such-mode") == (None, None)
     lines = [l for l in open(b.TRAFFIC_FILE) if l.startswith("#@ traffic")]
     assert len(lines) >= 1 and all("commit=" in l for l in lines)
+
+
+def test_benchmark_inputs_are_the_parity_tests_tensors():
+    """bench.py::make_inputs draws on the CPU from one seeded generator: bit for bit what tests/conftest.py::make_qkv (and,
+    for the video-DiT workload, tests/test_gpu_route.py::_frames on top of it) hands to the oracle and the kernels."""
+    import torch
+    from conftest import make_qkv
+    b = _bench()
+    for seed in (2, 3):                                                  # C3 / C4 scheme: outlier channels
+        q, k, v = b.make_inputs(1, 8, 2, 384, 128, seed, "cpu")
+        q2, k2, v2 = make_qkv(1, 8, 2, 384, 128, seed=seed, outliers=True)
+        assert torch.equal(q, q2) and torch.equal(k, k2) and torch.equal(v, v2)
+    q, k, v = b.make_inputs(1, 8, 8, 1024, 64, 0, "cpu", outliers=False)   # C1: plain N(0,1) draws
+    q2, k2, v2 = make_qkv(1, 8, 8, 1024, 64, seed=0)
+    assert torch.equal(q, q2) and torch.equal(k, k2) and torch.equal(v, v2)
+    # C5 scheme: sigma 0.5 and per-frame offsets (21 frames) from a second generator seeded seed + 1
+    N, frames = 21 * 20, 21
+    q, k, v = b.make_inputs(1, 4, 4, N, 128, 4, "cpu", frames)
+    q2, k2, v2 = make_qkv(1, 4, 4, N, 128, seed=4, sigma=0.5)
+    g = torch.Generator().manual_seed(5)
+    for t in (q2, k2):
+        off = 0.5 * torch.randn(frames, 1, 128, generator=g)
+        t += off[torch.arange(N) // (N // frames)].reshape(1, 1, N, 128).to(t.dtype)
+    assert torch.equal(q, q2) and torch.equal(k, k2) and torch.equal(v, v2)

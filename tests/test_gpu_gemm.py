@@ -17,7 +17,7 @@ import torch
 import oracle as O
 from conftest import make_qkv
 from ours import _lib
-from ours.block_scaled_matmul import block_scaled_matmul, quantize_block_scaled_from_tensor, make_configs
+from ours.block_scaled_matmul import block_scaled_matmul, quantize_block_scaled_from_tensor, make_configs, pack_scale_5d
 from ours.mxfp import MXFP4Tensor, MXScaleTensor
 
 pytestmark = pytest.mark.gpu
@@ -273,10 +273,78 @@ def test_reference_validate_call_sequence(bst):
         # the reference's own bound holds where a 4-bit operand keeps the products short
         assert (err <= 1e-3 + 1e-3 * want.abs()).all(), err.max()
     assert (err <= (1e-3 + 2 ** -10) * want.abs() + 3e-5 * mag).all(), (err / mag).max()
-    with pytest.raises(NotImplementedError):
-        initialize_block_scaled_from_tensor(a_tensor.to(DEV), b_tensor.to(DEV), a_scale_tensor.to(DEV), b_scale_tensor.to(DEV), bst, True)
     with pytest.raises(NotImplementedError, match="nvfp4"):
         initialize_block_scaled_from_tensor(a_tensor.to(DEV), b_tensor.to(DEV), a_scale_tensor.to(DEV), b_scale_tensor.to(DEV), "nvfp4")
+    # compute_reference=True (ours/block_scaled_matmul.py:376-392, :404): the same packaged operands plus the triple
+    # (fake-quant product, dq(A), dq(B)) in float32, made on the device from the packaged bytes.  The device reference
+    # is itself pinned here: against the oracle's dequantization (exactly) and its float64 product.
+    a2, sa2, b2, sb2, cfg2, reference = initialize_block_scaled_from_tensor(
+        a_tensor.to(DEV), b_tensor.to(DEV), a_scale_tensor.to(DEV), b_scale_tensor.to(DEV), bst, compute_reference=True)
+    assert torch.equal(a2, a_desc) and torch.equal(b2, b_desc) and torch.equal(sa2, a_scale) and torch.equal(sb2, b_scale) and cfg2 == configs
+    ref, a_dq, b_dq = reference
+    assert ref.dtype == torch.float32 and ref.shape == (M, N) and a_dq.shape == (M, K) and b_dq.shape == (N, K)
+    assert torch.equal(a_dq.cpu(), O.dequantize_mx(a_codes, sa_lin, fa, torch.float32))
+    assert torch.equal(b_dq.cpu(), O.dequantize_mx(b_codes, sb_lin, fb, torch.float32))
+    assert ((ref.cpu().double() - want).abs() <= 1e-5 * mag).all()          # float32 accumulation of 256 products
+    # the reference's own comparison (ours/block_scaled_matmul.py:440)
+    if fa == O.FMT_E2M1 or fb == O.FMT_E2M1:
+        torch.testing.assert_close(ref, output.to(torch.float32), atol=1e-3, rtol=1e-3)
+
+
+@pytest.mark.parametrize("bst", ["mxfp4", "mixed", "mxfp8", "mixed_e5", "mxfp8e5"])
+def test_validate_block_scaled_from_tensor_runs_the_reference_self_check(bst):
+    """validate_block_scaled_from_tensor at the reference's own shape and seed (ours/block_scaled_matmul.py:498-501):
+    packaging with compute_reference=True, the kernel's fp16 product, assert_close(atol = rtol = 1e-3) -- and the
+    fake-quant reference it compares with is checked here against the oracle's float64 product of the same operands,
+    which are regenerated on the CPU from the same seed."""
+    from ours.block_scaled_matmul import validate_block_scaled_from_tensor
+    M, N, K = 128, 256, 256
+    torch.manual_seed(42)
+    reference, output = validate_block_scaled_from_tensor(M, N, K, bst, device=DEV)
+    assert reference.shape == (M, N) and output.dtype == torch.float16
+    # the self-check drew its operands from the device generator; draw them again and rebuild them for the oracle
+    torch.manual_seed(42)
+    a_tensor = torch.randn((M, K), dtype=torch.float16, device=DEV).cpu()
+    b_tensor = torch.randn((N, K), dtype=torch.float16, device=DEV).cpu()
+    sa = (torch.rand((M // 128, K // 32 // 4, 32, 4, 4), device=DEV) + 1e-8).cpu()
+    sb = (torch.rand((N // 128, K // 32 // 4, 32, 4, 4), device=DEV) + 1e-8).cpu()
+    f8 = O.FMT_E5M2 if bst.endswith("e5") else O.FMT_E4M3
+    a_codes, fa = _oracle_operand(a_tensor, bst == "mxfp4", f8)
+    b_codes, fb = _oracle_operand(b_tensor, bst in ("mxfp4", "mixed", "mixed_e5"), f8)
+    sa_lin, sb_lin = O.scales_from_5d(O.encode_e8m0(sa)), O.scales_from_5d(O.encode_e8m0(sb))
+    want = O.gemm_mx(a_codes, sa_lin, b_codes, sb_lin, fa, fb, acc_dtype=torch.float64)
+    mag = O.dequantize_mx(a_codes, sa_lin, fa, torch.float64).abs() @ O.dequantize_mx(b_codes, sb_lin, fb, torch.float64).abs().T
+    assert ((reference.cpu().double() - want).abs() <= 1e-5 * mag).all()
+
+
+def test_packaging_refuses_values_beyond_e4m3_and_casts_them_in_e5m2():
+    """The reference's 8-bit cast is E5M2 (ours/block_scaled_matmul.py:334-336: finite up to 57344); this package's
+    "mxfp8" / "mixed" cast to E4M3, where torch's cast makes NaN of magnitudes above 464: such input is refused with a
+    pointer to the E5M2 types, under which the bytes are torch's E5M2 cast."""
+    from ours.block_scaled_matmul import initialize_block_scaled_from_tensor
+    M, N, K = 128, 128, 128
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(M, K, generator=g).to(torch.float16)
+    b = torch.randn(N, K, generator=g).to(torch.float16)
+    a[3, 7], a[100, 5], b[9, 9] = 1000.0, -30000.0, 449.0
+    sa = torch.rand((1, 1, 32, 4, 4), generator=g) + 1e-8
+    sb = torch.rand((1, 1, 32, 4, 4), generator=g) + 1e-8
+    for bst in ("mxfp8", "mixed"):
+        with pytest.raises(ValueError, match="mxfp8e5"):
+            initialize_block_scaled_from_tensor(a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV), bst)
+    a_desc, a_scale, b_desc, b_scale, configs, reference = initialize_block_scaled_from_tensor(
+        a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV), "mxfp8e5", compute_reference=True)
+    assert torch.equal(a_desc.cpu(), a.float().to(torch.float8_e5m2).view(torch.uint8))
+    assert torch.equal(b_desc.cpu(), b.float().to(torch.float8_e5m2).view(torch.uint8))
+    out = block_scaled_matmul(a_desc, a_scale, b_desc, b_scale, torch.float32, M, N, K, configs)
+    assert torch.isfinite(out).all() and torch.isfinite(reference[0]).all()
+    mag = reference[1].abs() @ reference[2].abs().T
+    assert ((out - reference[0]).abs() <= 1e-3 * reference[0].abs() + 3e-5 * mag).all()
+    # exactly +-448 still fits E4M3
+    a2 = a.clamp(-448, 448)
+    b2 = b.clamp(-448, 448)
+    a_desc, *_ = initialize_block_scaled_from_tensor(a2.to(DEV), b2.to(DEV), sa.to(DEV), sb.to(DEV), "mxfp8")
+    assert torch.equal(a_desc.cpu(), a2.float().to(torch.float8_e4m3fn).view(torch.uint8))
 
 
 @pytest.mark.parametrize("fa,fb", [(O.FMT_E2M1, O.FMT_E2M1), (O.FMT_E4M3, O.FMT_E4M3), (O.FMT_E5M2, O.FMT_E5M2),
@@ -308,16 +376,40 @@ def test_edge_tiles_and_mixed_formats_against_oracle(fa, fb, M, N, K):
     assert (err <= bound).all(), f"worst err/mag {(err / mag.clamp_min(1e-30)).max().item():.3e}"
 
 
-@pytest.mark.parametrize("bst", ["mxfp4", "mxfp8"])
-def test_general_kernel_equals_the_staged_kernel_on_its_shapes(bst):
+@pytest.mark.parametrize("K", [1024, 384])         # 16 scale bytes per row at a time (K % 512 == 0), and 4 per stage
+@pytest.mark.parametrize("bst", ["mxfp4", "mxfp8", "mixed", "mixed_e5"])
+def test_general_kernel_equals_the_staged_kernel_on_its_shapes(bst, K):
     """A 512 x 256 product computed whole (LDS-staged 256 x 256 kernel) and as two row slabs of 384 and 128 rows (the
-    general kernel: 384 is not a multiple of 256): same K order, same matrix instruction, same bits."""
-    M, N, K = 512, 256, 1024
+    general kernel: 384 is not a multiple of 256): same K order, same matrix instruction, same bits -- for equal
+    formats and for the reference's "mixed" type (8-bit A x 4-bit B, ours/block_scaled_matmul.py:318-324), with
+    row-major and with packed scales."""
+    M, N = 512, 256
     a, b, (ac, asc, bc, bsc, cfg) = _operands(M, N, K, bst, seed=77)
     whole = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg)
     top = block_scaled_matmul(ac[:384].contiguous(), asc[:384].contiguous(), bc, bsc, torch.float32, 384, N, K, cfg)
     bottom = block_scaled_matmul(ac[384:].contiguous(), asc[384:].contiguous(), bc, bsc, torch.float32, 128, N, K, cfg)
     assert torch.equal(whole, torch.cat([top, bottom]))
+    if K % 128 == 0:
+        packed = block_scaled_matmul(ac, pack_scale_5d(asc), bc, pack_scale_5d(bsc), torch.float32, M, N, K, cfg)
+        assert torch.equal(whole, packed)
+    for dt in (torch.bfloat16, torch.float16):
+        assert torch.equal(block_scaled_matmul(ac, asc, bc, bsc, dt, M, N, K, cfg), whole.to(dt))
+
+
+@pytest.mark.parametrize("bst", ["mixed", "mixed_e5"])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 768, 1024), (256, 512, 640), (768, 256, 2048)])
+def test_mixed_formats_on_the_staged_kernel_against_oracle(bst, M, N, K):
+    """8-bit A x 4-bit B on whole 256 x 256 tiles (the LDS-staged kernel's mixed variant) against the float64 oracle."""
+    f8 = O.FMT_E5M2 if bst.endswith("e5") else O.FMT_E4M3
+    a, b, (ac, asc, bc, bsc, cfg) = _operands(M, N, K, bst, seed=M + N + K)
+    oa, osa = O.quantize_mx(a, 1.0, f8)
+    ob, osb = O.quantize_mx(b, 1.0, O.FMT_E2M1)
+    assert torch.equal(ac.cpu(), oa) and torch.equal(bc.cpu(), ob) and torch.equal(asc.cpu(), osa) and torch.equal(bsc.cpu(), osb)
+    want = O.gemm_mx(oa, osa, ob, osb, f8, O.FMT_E2M1, acc_dtype=torch.float64)
+    mag = O.dequantize_mx(oa, osa, f8, torch.float64).abs() @ O.dequantize_mx(ob, osb, O.FMT_E2M1, torch.float64).abs().T
+    got = block_scaled_matmul(ac, asc, bc, bsc, torch.float32, M, N, K, cfg).cpu()
+    err = (got.double() - want).abs()
+    assert (err <= 1e-3 * want.abs() + 3e-5 * mag).all(), f"worst err/mag {(err / mag.clamp_min(1e-30)).max().item():.3e}"
 
 
 def test_batched_mixed_formats_with_grouped_heads():

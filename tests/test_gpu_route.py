@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import oracle as O
-from conftest import make_qkv, attention_close
+from conftest import make_qkv, attention_close, check_attention
 from ours import _lib
 from ours.mxfp_attn import mxfp_attn
 from ours.mxfp_attn_kernel import prepare_operands, route_tiles, attention_from_operands, mxfp_attn_kernel
@@ -111,20 +111,22 @@ def test_routed_attention_against_oracle(D, tile, causal):
     ops, route = _route_gpu(q, k, v, tile, causal, 0.5, 0.2)
     cls = route[0].cpu().numpy()
     assert {0, 1, 2} <= set(np.unique(cls).tolist())
-    out = torch.empty((1, 4, N, D), dtype=torch.bfloat16, device=DEV)
-    attention_from_operands(ops, out, causal, route=route)
-    want = O.attn_mx(q, k, v, tile=tile, causal=causal, mode="routed", route=cls)
-    _compare(out, want, f"routed D={D} tile={tile} causal={causal}")
+    def run(dt):
+        out = torch.empty((1, 4, N, D), dtype=dt, device=DEV)
+        return attention_from_operands(ops, out, causal, route=route)
+    want = O.attn_mx(q, k, v, tile=tile, causal=causal, mode="routed", route=cls, out_dtype=torch.float32)
+    check_attention(run, want, f"routed D={D} tile={tile} causal={causal}", torch.bfloat16)
 
 
 def test_routed_entry_point_and_sparsity():
     q, k, v = _inputs(1, 4, 4, 640, 128, seed=360)
-    got, sparsity = mxfp_attn(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=False, smooth_k=False,
-                              output_dtype=torch.bfloat16, block_scale_type="routed", route_thresh=0.5,
-                              skip_thresh=0.2, return_sparsity=True)
+    run = lambda dt: mxfp_attn(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=False, smooth_k=False, output_dtype=dt,
+                               block_scale_type="routed", route_thresh=0.5, skip_thresh=0.2, return_sparsity=True)
+    got, sparsity = run(torch.bfloat16)
     ops, route = _route_gpu(q, k, v, 128, False, 0.5, 0.2)
     cls = route[0].cpu().numpy()
-    _compare(got, O.attn_mx(q, k, v, tile=128, causal=False, mode="routed", route=cls), "mxfp_attn routed")
+    check_attention(lambda dt: run(dt)[0], O.attn_mx(q, k, v, tile=128, causal=False, mode="routed", route=cls, out_dtype=torch.float32),
+                    "mxfp_attn routed", torch.bfloat16)
     assert abs(float(sparsity) - float((cls == 0).mean())) < 1e-6
     with pytest.raises(ValueError):
         mxfp_attn(q.to(DEV), k.to(DEV), v.to(DEV), block_scale_type="mxfp4", route_thresh=0.5, smooth_k=False)
@@ -139,19 +141,18 @@ def test_routed_e5m2_smooth_k_fp16_and_nhd_layout():
     ops = prepare_operands(q.to(DEV), ks.to(DEV), v.to(DEV), 64, "routed_e5")
     cls = route_tiles(ops, True, 0.5, 0.2)[0].cpu().numpy()
     assert {1, 2} <= set(np.unique(cls).tolist())
-    want = O.attn_mx(q, ks, v, tile=64, causal=True, mode="routed", route=cls, fmt8=O.FMT_E5M2)
-    got = mxfp_attn_kernel(q.transpose(1, 2).contiguous().to(DEV), ks.transpose(1, 2).contiguous().to(DEV),
-                           v.transpose(1, 2).contiguous().to(DEV), is_causal=True, tensor_layout="NHD",
-                           output_dtype=torch.float16, block_scale_type="routed_e5", tile=64, route_thresh=0.5,
-                           skip_thresh=0.2)
-    assert got.shape == (1, N, 4, 64)
-    _compare(got.transpose(1, 2), want, "routed_e5 NHD")
+    want = O.attn_mx(q, ks, v, tile=64, causal=True, mode="routed", route=cls, fmt8=O.FMT_E5M2, out_dtype=torch.float32)
+    run = lambda dt: mxfp_attn_kernel(q.transpose(1, 2).contiguous().to(DEV), ks.transpose(1, 2).contiguous().to(DEV),
+                                      v.transpose(1, 2).contiguous().to(DEV), is_causal=True, tensor_layout="NHD",
+                                      output_dtype=dt, block_scale_type="routed_e5", tile=64, route_thresh=0.5, skip_thresh=0.2)
+    assert run(torch.float16).shape == (1, N, 4, 64)
+    check_attention(lambda dt: run(dt).transpose(1, 2), want, "routed_e5 NHD", torch.float16)
     # smoothing inside the wrapper: same map inputs up to the 16-bit mean's last place, so compare the output only
-    got2 = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=True, smooth_k=True, output_dtype=torch.float16,
-                            block_scale_type="routed_e5", tile=64, route_thresh=0.5, skip_thresh=None)
-    want2 = O.attn_mx(q, k, v, tile=64, causal=True, mode="routed", smooth_k=True, fmt8=O.FMT_E5M2,
+    want2 = O.attn_mx(q, k, v, tile=64, causal=True, mode="routed", smooth_k=True, fmt8=O.FMT_E5M2, out_dtype=torch.float32,
                       route=O.route_tiles(*_oracle_scales(q, O.smooth_k(k), 64), 64, True, 0.5, None))
-    _compare(got2, want2, "routed_e5 smooth_k")
+    check_attention(lambda dt: mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=True, smooth_k=True, output_dtype=dt,
+                                                block_scale_type="routed_e5", tile=64, route_thresh=0.5, skip_thresh=None),
+                    want2, "routed_e5 smooth_k", torch.float16)
 
 
 def _oracle_scales(q, k, tile):
@@ -194,12 +195,12 @@ def test_routed_lists_are_clamped_and_empty_rows_give_zeros():
     counts[0, 1, 2] = torch.tensor([1 << 30, -5, 1 << 30, 7])      # run lengths beyond the row: clamped to nt tiles
     order[0, 1, 3, 0] = 1 << 20                            # tile index beyond the sequence: clamped to the last tile
     order[0, 1, 3, 1] = -9                                 # and below it: clamped to tile 0
-    out = torch.empty((1, 2, 384, 64), dtype=torch.bfloat16, device=DEV)
+    out = torch.empty((1, 2, 384, 64), dtype=torch.float32, device=DEV)
     attention_from_operands(ops, out, False, route=(cls, order, counts))
     torch.cuda.synchronize()
-    assert torch.isfinite(out.float()).all()
+    assert torch.isfinite(out).all()
     assert (out[0, 0, 64:128] == 0).all()
-    want = O.attn_mx(q, k, v, tile=64, causal=False, mode="mxfp4")
+    want = O.attn_mx(q, k, v, tile=64, causal=False, mode="mxfp4", out_dtype=torch.float32)
     _compare(out[:, :1, :64], want[:, :1, :64], "untouched rows")
     _compare(out[:, 1:, 256:], want[:, 1:, 256:], "untouched rows")
 

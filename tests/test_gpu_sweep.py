@@ -9,7 +9,7 @@ import pytest
 import torch
 
 import oracle as O
-from conftest import make_qkv, attention_close
+from conftest import make_qkv, attention_close, check_attention
 from ours.block_scaled_matmul import block_scaled_matmul, quantize_block_scaled_from_tensor
 from ours.mxfp_attn_kernel import prepare_operands, route_tiles, attention_from_operands, mxfp_attn_kernel
 from ours.quant_mxint8 import quantize_mx, quantize_mx_dual
@@ -53,15 +53,18 @@ def test_attention_sweep(sweep_seed):
             cls = route[0].cpu().numpy()
             want_cls = O.route_tiles(ops["qs4"].cpu().numpy(), ops["ks4"].cpu().numpy(), p["tile"], p["causal"], p["hi"], p["lo"])
             assert np.array_equal(cls, want_cls), what
-            out = torch.empty((1, p["Hq"], p["N"], p["D"]), dtype=p["dt"], device=DEV)
-            attention_from_operands(ops, out, p["causal"], route=route)
-            want = O.attn_mx(q, k, v, tile=p["tile"], causal=p["causal"], mode="routed", route=cls, fmt8=fmt8)
+            def run(dt):
+                out = torch.empty((1, p["Hq"], p["N"], p["D"]), dtype=dt, device=DEV)
+                return attention_from_operands(ops, out, p["causal"], route=route)
+            want = O.attn_mx(q, k, v, tile=p["tile"], causal=p["causal"], mode="routed", route=cls, fmt8=fmt8, out_dtype=torch.float32)
         else:
-            out = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=p["causal"], block_scale_type=p["mode"],
-                                   tile=p["tile"], output_dtype=p["dt"])
+            def run(dt):
+                return mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=p["causal"], block_scale_type=p["mode"],
+                                        tile=p["tile"], output_dtype=dt)
             want = O.attn_mx(q, k, v, tile=p["tile"], causal=p["causal"], mode={"mxfp8e5": "mxfp8"}.get(p["mode"], p["mode"]),
-                             fmt8=fmt8)
-        attention_close(out, want, what)
+                             fmt8=fmt8, out_dtype=torch.float32)
+        # the bar on the float32 outputs; the 16-bit output of the case's dtype is the rounded float32 one
+        check_attention(run, want, what, p["dt"])
 
 
 def test_paired_tile_kernel_sweep():
