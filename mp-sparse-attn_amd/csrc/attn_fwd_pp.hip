@@ -11,8 +11,9 @@
 // instructions S(t+1), then the 32 matrix instructions of P.V(t) with the softmax of tile t+1 placed in the gaps
 // between them -- measured on MI355X, vector instructions of the *other* wave of a SIMD get almost no issue slots
 // while a wave streams matrix instructions, but a few vector instructions between a wave's own matrix instructions
-// are free.  The registers of a 16-key group of P(t) take the new P(t+1) as soon as the four instructions that
-// consume the group have been issued.  The exponentials are taken without a maximum pass: the (lazy) running maximum
+// are free.  The exponentials run in place over the score registers, one pair per gap from the first matrix instruction
+// on; the registers of a 16-key group of P(t) take the new P(t+1) as soon as the four instructions that consume the
+// group have been issued.  The exponentials are taken without a maximum pass: the (lazy) running maximum
 // only has to move when a score exceeds it by more than a threshold, which the tile's row sum then shows; the wave
 // does such a tile again the careful way (scores from the K tile still in LDS, maximum, rebase of row sum and output
 // accumulators -- P.V(t), relative to the old maximum, is through by then -- and exponentials).
@@ -419,8 +420,15 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         l_run += tot;
     };
 
-    // P.V(t) with the softmax of tile t+1 (whose scores are in st) in the gaps between its matrix instructions: after the
-    // four instructions that consume one 16-key group of P(t), that group's registers take the new P(t+1).
+    // P.V(t) with the softmax of tile t+1 (whose scores are in st) in the gaps between its matrix instructions.  The work
+    // of score pair e (two of a lane's 64 scores) is spread over three gaps so that no instruction waits for the one
+    // before it: the exponentials are taken in place in the gap of matrix instruction e; the row-sum additions follow one
+    // gap later (the exponential unit's latency is over by then); the conversion into the P registers follows four gaps
+    // later -- the four matrix instructions that consume a 16-key group of P(t) are out, so the group's registers take
+    // the new P(t+1).  Only the last addition and the last group's four conversions are left behind the last matrix
+    // instruction (with exponentials, additions and conversions of a pair all in one gap, the wave stalled on the
+    // exponentials' results in every gap and a whole group's softmax ran after the last matrix instruction: 6 % more
+    // cycles per step at a fixed clock).
     auto pv_exp = [&](int t) __attribute__((always_inline)) {
         constexpr int PRE = 8;
         const uint8_t* vl = vbuf0 + (t & 1) * V_BYTES + lane * 16;
@@ -440,22 +448,42 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             const int f = (krow >> SH4) & (CPR4 - 1);
             kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * ROW4 + (((2 * s + h) ^ f) * 16));
         };
+        // score pair e = 4 g + j: registers 8c + 2j, 8c + 2j + 1 of key block kb, with g = 2 kb + c the 16-key group
+        auto do_exp = [&](int e) __attribute__((always_inline)) {
+            const int g = e >> 2, j = e & 3, kb = g >> 1, c = g & 1;
+            st[kb][8 * c + 2 * j] = __builtin_amdgcn_exp2f(st[kb][8 * c + 2 * j]);
+            st[kb][8 * c + 2 * j + 1] = __builtin_amdgcn_exp2f(st[kb][8 * c + 2 * j + 1]);
+        };
+        auto do_add = [&](int e) __attribute__((always_inline)) {
+            const int g = e >> 2, j = e & 3, kb = g >> 1, c = g & 1;
+            ps0 += st[kb][8 * c + 2 * j];
+            ps1 += st[kb][8 * c + 2 * j + 1];
+        };
+        auto do_cvt = [&](int e) __attribute__((always_inline)) {
+            const int g = e >> 2, j = e & 3, kb = g >> 1, c = g & 1;
+            const typename P::v2 pp = P::pack(st[kb][8 * c + 2 * j], st[kb][8 * c + 2 * j + 1]);
+            int word = __builtin_bit_cast(int, pp);
+            // pin the conversion here, between the matrix instructions: the redo path overwrites pk, so the compiler
+            // would otherwise sink all 32 conversions behind the check, where nothing overlaps them
+            asm volatile("" : "+v"(word));
+            pk[kb][c][j] = word;
+        };
 #pragma unroll
-        for (int kc = 0; kc < 2 * KB; ++kc)
+        for (int idx = 0; idx < NV; ++idx) {
+            const int d = idx % NDB, kc = idx / NDB;
+            mm(idx);
+            do_exp(idx);
+            if (idx >= 1) do_add(idx - 1);
+            if (idx >= NDB) do_cvt(idx - NDB);
+            if (kc >= KB && d < SST) kfrag(kc - KB, d);   // K fragments of tile t+2 (the score MFMAs are long gone)
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+        }
+        do_add(NV - 1);
 #pragma unroll
-            for (int d = 0; d < NDB; ++d) {
-                mm(kc * NDB + d);
-                if (kc > 0) ex(kc - 1, d, ps0, ps1);
-                if (kc >= KB && d < SST) kfrag(kc - KB, d);   // K fragments of tile t+2 (the score MFMAs are long gone)
-                if (kc > 0) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
-                }
-            }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) ex(2 * KB - 1, j, ps0, ps1);
+        for (int e = NV - NDB; e < NV; ++e) do_cvt(e);
         finish_tile(t, ps0, ps1);
     };
 
