@@ -61,7 +61,7 @@ WORKLOADS = {
 }
 NON_CAUSAL = {"c5"}
 PLAIN_DRAWS = {"c1"}          # N(0,1) without outlier channels
-ROUTE_THRESH_DEFAULT = 0.9
+ROUTE_THRESH_DEFAULT = 0.97        # on the C5 inputs: about 8 % of the tiles in MXFP8 (see profiles/attn_c5_router_study.txt)
 
 
 def make_inputs(B, Hq, Hkv, N, D, seed, device, dit_frames=0, outliers=True):
@@ -318,12 +318,73 @@ def mfma_stream_rates(device, seconds=0.05):
     return out
 
 
+def router_study(args, device):
+    """What per-tile precision routing buys on a workload: for the fixed-precision modes and for the routed mode at a few
+    thresholds, the attention kernel's time on the first ``--heads`` heads and the error of its float32 output against
+    exact attention (float64 softmax(q k^T) v of the unquantized 16-bit inputs, computed with torch on the device) on
+    sampled query tiles."""
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, route_tiles
+    from ours.quant_mxint8 import pre_scale_q
+    B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
+    causal = args.workload not in NON_CAUSAL
+    q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21, args.workload not in PLAIN_DRAWS)
+    group = Hq // Hkv
+    hq = min(args.heads, Hq)
+    hq -= hq % group if hq >= group else 0
+    hq = max(hq, group)
+    q, k, v = q[:, :hq].contiguous(), k[:, :hq // group].contiguous(), v[:, :hq // group].contiguous()
+    nt = (N + tile - 1) // tile
+    tiles = sorted({0, nt // 5, nt // 2, (4 * nt) // 5, nt - 1})
+    rows = torch.cat([torch.arange(t * tile, min((t + 1) * tile, N)) for t in tiles]).to(device)
+    pre = pre_scale_q(D)                                   # sm_scale * log2(e): scores in log2 units
+    exact = torch.empty((B, hq, rows.numel(), D), dtype=torch.float64, device=device)
+    for h in range(hq):
+        sc = (q[0, h, rows].double() @ k[0, h // group].double().T) * pre
+        if causal:
+            sc = sc.masked_fill(torch.arange(N, device=device)[None, :] > rows[:, None], float("-inf"))
+        pr = torch.exp2(sc - sc.amax(dim=1, keepdim=True))
+        exact[0, h] = (pr / pr.sum(dim=1, keepdim=True)) @ v[0, h // group].double()
+    out = torch.empty((B, hq, N, D), dtype=torch.float32, device=device)
+    cases = [("mxfp4", None, None), ("diag", None, None), ("mxfp8", None, None)]
+    cases += [("routed", t, None) for t in (0.99, 0.97, 0.95, 0.9, 0.8, 0.5)]
+    cases += [("routed", 0.95, 0.5), ("routed", None, 0.5), ("routed", None, 0.8)]
+    table = []
+    for mode, hi, lo in cases:
+        ops = prepare_operands(q, k, v, tile, mode)
+        route = route_tiles(ops, causal, hi, lo) if mode == "routed" else None
+        attention_from_operands(ops, out, causal, route=route)
+        torch.cuda.synchronize()
+        t_spin = time.perf_counter()                       # clocks up before the timed launches, the same for every case
+        while (time.perf_counter() - t_spin) * 1e3 < args.spinup_ms:
+            attention_from_operands(ops, out, causal, route=route)
+            wait_for_device()
+        ms = time_events(lambda: attention_from_operands(ops, out, causal, route=route), args.steps)
+        got = out[:, :, rows].double()
+        err = (got - exact).abs()
+        row = {"mode": mode, "route_thresh": hi, "skip_thresh": lo, "kernel_ms": round(ms, 4),
+               "cos": round(torch.nn.functional.cosine_similarity(got.flatten(), exact.flatten(), dim=0).item(), 7),
+               "max_abs": float("%.4g" % err.max().item()), "rmse": float("%.4g" % err.pow(2).mean().sqrt().item()),
+               "rel_l1": float("%.4g" % (err.sum() / exact.abs().sum()).item())}
+        if route is not None:
+            cls = route[0]
+            visited = float((cls != 255).sum())
+            row["tile_shares"] = {"mxfp8": round(float((cls == 2).sum()) / visited, 4), "mxfp4": round(float((cls == 1).sum()) / visited, 4),
+                                  "skipped": round(float((cls == 0).sum()) / visited, 4)}
+        table.append(row)
+        del ops, route
+    print(json.dumps({"kernel": "router study", "workload": desc, "heads": hq, "sampled_query_tiles": tiles,
+                      "reference": "float64 softmax(q k^T * scale) v of the unquantized inputs (torch, on the device)", "cases": table}))
+
+
 def run_only(args, device):
     """Launch one kernel repeatedly (for rocprofv3 --pmc / --kernel-trace runs)."""
     from ours import _lib
     from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, route_tiles
     from ours.quant_mxint8 import quantize_mx, quantize_mx_dual
     from ours.block_scaled_matmul import block_scaled_matmul, make_configs, pack_scale_5d
+    if args.only == "router":
+        router_study(args, device)
+        return
     if args.only == "mfma":
         print(json.dumps({"kernel": "matrix-instruction stream", "rates": mfma_stream_rates(device, 0.2)}))
         return
@@ -359,9 +420,10 @@ def run_only(args, device):
         else:          # every code and scale byte the same: what the kernel does when power management leaves the clock alone
             a = torch.full((1, 1, M, K), 1.0 if args.operands == "ones" else 0.0, dtype=torch.bfloat16, device=device)
             b = a.clone()
-        bst, fmt = ("mxfp4", _lib.FMT_E2M1) if args.only == "gemm4" else ("mxfp8", _lib.FMT_E4M3)
+        bst, fmt, fmt_b = {"gemm4": ("mxfp4", _lib.FMT_E2M1, _lib.FMT_E2M1), "gemm8": ("mxfp8", _lib.FMT_E4M3, _lib.FMT_E4M3),
+                           "gemm48": ("mixed", _lib.FMT_E4M3, _lib.FMT_E2M1)}[args.only]
         ac, asc = quantize_mx(a, 1.0, fmt)
-        bc, bsc = quantize_mx(b, 1.0, fmt)
+        bc, bsc = quantize_mx(b, 1.0, fmt_b)
         cfg = make_configs(bst)
         sa2, sb2 = (asc[0, 0], bsc[0, 0]) if args.linear_scales else (pack_scale_5d(asc[0, 0]), pack_scale_5d(bsc[0, 0]))
         fn = lambda: block_scaled_matmul(ac[0, 0], sa2, bc[0, 0], sb2, torch.bfloat16, M, N, K, cfg)
@@ -392,13 +454,14 @@ def main():
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--no-fuse-q", action="store_true", help="with --only attn: hand the kernel quantized Q operands")
     ap.add_argument("--no-c4", action="store_true", help="leave the long-context figures out of `secondary`")
+    ap.add_argument("--heads", type=int, default=4, help="--only router: query heads of the workload to run")
     ap.add_argument("--no-c5", action="store_true", help="leave the video-DiT figures out of `secondary`")
     ap.add_argument("--eager", action="store_true", help="time plain launches instead of replaying the step as a HIP graph")
     ap.add_argument("--operands", default="random", choices=["random", "ones", "zeros"],
                     help="--only gemm4|gemm8|attn: the workload's random operands (default) or constant ones (the clock then stays up)")
     ap.add_argument("--linear-scales", action="store_true",
                     help="with --only gemm4/gemm8: row-major [rows, K/32] scales instead of the reference's packed form")
-    ap.add_argument("--only", default=None, choices=["attn", "copy", "quant", "gemm4", "gemm8", "mfma"],
+    ap.add_argument("--only", default=None, choices=["attn", "copy", "quant", "gemm4", "gemm8", "gemm48", "mfma", "router"],
                     help="profiling aid: launch just this kernel --steps times and exit (copy = 1 GiB torch copy, "
                          "the calibration kernel for HBM counters)")
     args = ap.parse_args()
