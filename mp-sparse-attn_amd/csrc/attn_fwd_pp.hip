@@ -21,8 +21,9 @@
 //
 // Staging is the one of attn_fwd.hip: 4-bit K tiles (XOR-swizzled rows) and V tiles (operand order) arrive by
 // direct-to-LDS loads, one barrier per key tile; K has three buffers (the tile whose fragments are being pulled into
-// registers is two steps ahead of the P.V tile), V two; the single 8-bit (diagonal) tile of a "diag" run is read
-// straight from global memory.  The running maximum rides in the score MFMA's C operand.
+// registers is two steps ahead of the P.V tile), V two; the two 8-bit (diagonal) K tiles of a "diag" run's pair are staged
+// once, in the prologue, into an LDS area of their own (read straight from global memory at the diagonal step their
+// latency sat on the wave's critical path).  The running maximum rides in the score MFMA's C operand.
 #include "attn_common.h"
 #include "quantize_kernel.h"
 
@@ -37,6 +38,9 @@ constexpr int NKBUF = 3;                        // K tiles in LDS: one being mul
 constexpr int SMEM = NKBUF * K_BYTES + 2 * V_BYTES;
 constexpr int Q8_BYTES = 512 * 64;              // fused-quantizer variants: every lane's 8-bit Q fragments (64 bytes), parked until the diagonal tile
 constexpr int SMEM_QRAW = SMEM + Q8_BYTES;
+constexpr int K8_BYTES = TILE * ROW8;           // "diag" runs: the two 8-bit diagonal K tiles of the pair (X's, then Y's), staged in the prologue
+constexpr int CPR8 = ROW8 / 16;
+constexpr int smem_bytes(bool qraw, int mode) { return (qraw ? SMEM_QRAW : SMEM) + (mode == MPSA_MODE_DIAG ? 2 * K8_BYTES : 0); }
 constexpr int NWAVES = 8;
 constexpr int VI = V_BYTES / 1024 / NWAVES;     // direct-load instructions per wave for one V tile (4)
 constexpr int NV = KB * 2 * NDB;                // P.V matrix instructions per tile (32)
@@ -81,6 +85,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
 
     uint8_t* const kbuf0 = smem;
     uint8_t* const vbuf0 = smem + NKBUF * K_BYTES;
+    uint8_t* const k8d0 = smem + (QRAW ? SMEM_QRAW : SMEM);     // the pair's two 8-bit diagonal K tiles: tile 2I+1, tile 2I
 
     // ---- operands in registers ----
     v8i qf[SST];
@@ -94,79 +99,69 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         const uint32_t ef = ab >> 23;
         return ef ? (int)ef - 127 : (31 - __builtin_clz(ab | 1u)) - 149;
     };
-    auto load_q_raw = [&](bool is8) __attribute__((always_inline)) {
+    // Both precisions from one pass over the lane's query row: lane half h owns MX blocks h and 2 + h of the row's four
+    // (the 4-bit operand layout), so a block's maximum and shared exponent are lane-local and serve both formats (the
+    // element exponent limits differ: 3 and 7).  The 8-bit operand wants 16 bytes of EVERY block in each lane half
+    // (registers 0-3: block 2s, 4-7: block 2s + 1), so the two lanes of a query trade halves of their blocks afterwards:
+    // one v_permlane32_swap per register pair.  q8f receives the 8-bit fragments when WANT8 is set.
+    auto load_q_raw = [&](auto want8_c, v8i (&q8f)[SST]) __attribute__((always_inline)) {
 #pragma clang fp contract(off)        // the quantizer's arithmetic, operation by operation
-        // this lane's query row, unquantized; lane half h owns MX blocks h and 2+h of the row's four in the 4-bit
-        // layout, and one half (16 elements) of every block in the 8-bit layout
+        constexpr bool WANT8 = decltype(want8_c)::value;
         const char* row = static_cast<const char*>(a.q_raw) +
                           2 * ((int64_t)b * a.q_sb + (int64_t)hq * a.q_sh + ((int64_t)i * TILE + q_local) * a.q_sn);
-        uint32_t sbytes = 0;
-        if (!is8) {
+        uint32_t sbytes = 0, sbytes8 = 0;
 #pragma unroll
-            for (int s = 0; s < SST; ++s) {
-                float x[4][8];
-                float amax = 0.0f;
+        for (int s = 0; s < SST; ++s) {
+            float x[4][8];
+            float amax = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                load8<PVT>(row + 2 * (32 * (2 * s + h) + 8 * c), x[c]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    x[c][e] = x[c][e] * a.q_pre;
+                    amax = __builtin_fmaxf(amax, __builtin_fabsf(x[c][e]));
+                }
+            }
+            const bool zero = mpsa_f2u(amax) == 0u;
+            const int ex = block_exponent(amax);
+            const int se = ex - 3;                                             // emax of E2M1: ours/quant_mxint8.py:303
+            int w[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) w[c] = zero ? 0 : (int)e2m1_pack8<true>(x[c], se, false);
+            qf[s] = (v8i){w[0], w[1], w[2], w[3], 0, 0, 0, 0};
+            sbytes |= (uint32_t)(zero ? 0 : min(max(se + 127, 0), 254)) << (16 * s);
+            if constexpr (WANT8) {
+                const int se8 = ex - 7;                                        // emax of the 8-bit formats: ours/quant_mxint8.py:191
+                // the quantizer's clamp to the format's maximum (quantize_kernel.h): finite blocks scale into
+                // [128, 256) and never meet it, a block with an infinity saturates there instead of giving NaN codes
+                const float lim = (FMT8 == MPSA_FMT_E4M3) ? 448.0f : 57344.0f;
+                int w8[8];
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    load8<PVT>(row + 2 * (32 * (2 * s + h) + 8 * c), x[c]);
+                    float y[8];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        x[c][e] = x[c][e] * a.q_pre;
-                        amax = __builtin_fmaxf(amax, __builtin_fabsf(x[c][e]));
-                    }
+                    for (int e = 0; e < 8; ++e) y[e] = __builtin_fminf(__builtin_fmaxf(ldexpf(x[c][e], -se8), -lim), lim);
+                    w8[2 * c] = zero ? 0 : (int)fp8_pack4<FMT8, false>(y[0], y[1], y[2], y[3]);
+                    w8[2 * c + 1] = zero ? 0 : (int)fp8_pack4<FMT8, false>(y[4], y[5], y[6], y[7]);
                 }
-                const bool zero = mpsa_f2u(amax) == 0u;
-                const int se = block_exponent(amax) - 3;                       // emax of E2M1: ours/quant_mxint8.py:303
-                int w[4];
+                // w8[0..3] = bytes 0-15, w8[4..7] = bytes 16-31 of block 2s + h.  Lane half 0 keeps its low half in
+                // registers 0-3 and takes block 2s + 1's low half from its partner into 4-7; lane half 1 keeps its high
+                // half in 4-7 and takes block 2s's high half into 0-3: swap (lanes 32-63 of register i) with (lanes 0-31 of
+                // register 4 + i).
 #pragma unroll
-                for (int c = 0; c < 4; ++c) w[c] = zero ? 0 : (int)e2m1_pack8<true>(x[c], se, false);
-                qf[s] = (v8i){w[0], w[1], w[2], w[3], 0, 0, 0, 0};
-                sbytes |= (uint32_t)(zero ? 0 : min(max(se + 127, 0), 254)) << (16 * s);
-            }
-        } else {
-#pragma unroll
-            for (int s = 0; s < SST; ++s) {
-                int w[8];
-#pragma unroll
-                for (int blk = 0; blk < 2; ++blk) {                             // MX block 2s + blk: this lane's 16 of its 32 elements
-                    float x[2][8];
-                    float amax = 0.0f;
-#pragma unroll
-                    for (int c = 0; c < 2; ++c) {
-                        load8<PVT>(row + 2 * (64 * s + 32 * blk + 16 * h + 8 * c), x[c]);
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) {
-                            x[c][e] = x[c][e] * a.q_pre;
-                            amax = __builtin_fmaxf(amax, __builtin_fabsf(x[c][e]));
-                        }
-                    }
-                    amax = max_lane_pair(amax);                                // the other half of the block sits in lane ^ 32
-                    const bool zero = mpsa_f2u(amax) == 0u;
-                    const int se = block_exponent(amax) - 7;                   // emax of the 8-bit formats: ours/quant_mxint8.py:191
-                    // the quantizer's clamp to the format's maximum (quantize_kernel.h): finite blocks scale into
-                    // [128, 256) and never meet it, a block with an infinity saturates there instead of giving NaN codes
-                    const float lim = (FMT8 == MPSA_FMT_E4M3) ? 448.0f : 57344.0f;
-#pragma unroll
-                    for (int c = 0; c < 2; ++c) {
-                        float y[8];
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) y[e] = __builtin_fminf(__builtin_fmaxf(ldexpf(x[c][e], -se), -lim), lim);
-                        w[4 * blk + 2 * c] = zero ? 0 : (int)fp8_pack4<FMT8, false>(y[0], y[1], y[2], y[3]);
-                        w[4 * blk + 2 * c + 1] = zero ? 0 : (int)fp8_pack4<FMT8, false>(y[4], y[5], y[6], y[7]);
-                    }
-                    // lane half h hands the matrix core the scale byte of block 2s + h
-                    if (blk == h) sbytes |= (uint32_t)(zero ? 0 : min(max(se + 127, 0), 254)) << (16 * s);
-                }
-                qf[s] = (v8i){w[0], w[1], w[2], w[3], w[4], w[5], w[6], w[7]};
+                for (int q = 0; q < 4; ++q)
+                    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(w8[q]), "+v"(w8[4 + q]));
+                q8f[s] = (v8i){w8[0], w8[1], w8[2], w8[3], w8[4], w8[5], w8[6], w8[7]};
+                // lane half h hands the matrix core the scale byte of block 2s + h: its own
+                sbytes8 |= (uint32_t)(zero ? 0 : min(max(se8 + 127, 0), 254)) << (16 * s);
             }
         }
         qsc = (int)sbytes;
+        qsc8 = (int)sbytes8;
     };
     auto load_q = [&](bool is8) __attribute__((always_inline)) {
-        if constexpr (QRAW) {
-            load_q_raw(is8);
-            return;
-        }
+        if constexpr (QRAW) return;                   // the fused-quantizer variants fill the fragments in the prologue
         if (is8) {
 #pragma unroll
             for (int s = 0; s < SST; ++s) {
@@ -284,13 +279,17 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     };
     auto s_special = [&](int t) __attribute__((always_inline)) {
         if constexpr (MODE == MPSA_MODE_DIAG) {
+            // this wave's 8-bit diagonal K tile has been in LDS since the prologue (rows XOR-swizzled like the 4-bit ones)
+            const uint8_t* kl = k8d0 + role * K8_BYTES;
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
-                const uint8_t* src = a.k8 + (khead_row + (int64_t)t * TILE + 32 * kb + r) * ROW8 + h * 16;
+                const int krow = 32 * kb + r;
+                const int f = (krow >> 1) & (CPR8 - 1);
 #pragma unroll
                 for (int s = 0; s < SST; ++s) {
-                    const v4i x0 = *reinterpret_cast<const v4i*>(src + s * 64);
-                    const v4i x1 = *reinterpret_cast<const v4i*>(src + s * 64 + 32);
+                    // 8-bit operand: registers 0-3 hold 16 bytes of MX block 2s, registers 4-7 of block 2s+1
+                    const v4i x0 = *reinterpret_cast<const v4i*>(kl + krow * ROW8 + (((4 * s + h) ^ f) * 16));
+                    const v4i x1 = *reinterpret_cast<const v4i*>(kl + krow * ROW8 + (((4 * s + h + 2) ^ f) * 16));
                     const v8i kd = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
                     st[kb] = score_mfma8<FMT8>(kd, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
                 }
@@ -492,20 +491,40 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     issue_k4(0);
     issue_k4(1);
     if (nsteps > 2) issue_k4(2);
-    if constexpr (QRAW && MODE == MPSA_MODE_DIAG) {
-        // The diagonal tile's 8-bit Q is quantized now, while the first K/V tiles are on their way, and parked in LDS
-        // (each lane reads back only what it wrote itself): at the diagonal tile the loads and the conversion would
-        // sit on the wave's critical path.
-        load_q(true);
-        qsc8 = qsc;
-        uint8_t* park = smem + SMEM + tid * 16;
+    if constexpr (MODE == MPSA_MODE_DIAG) {
+        // the pair's two diagonal tiles in 8 bits (X's: key tile 2I+1, Y's: 2I), 16 one-KiB pieces each, two per wave:
+        // piece position p = 8 row + slot holds the row's 16-byte chunk slot ^ ((row >> 1) & 7)
 #pragma unroll
-        for (int s = 0; s < SST; ++s) {
-            *reinterpret_cast<v4i*>(park + (2 * s) * 8192) = (v4i){qf[s][0], qf[s][1], qf[s][2], qf[s][3]};
-            *reinterpret_cast<v4i*>(park + (2 * s + 1) * 8192) = (v4i){qf[s][4], qf[s][5], qf[s][6], qf[s][7]};
+        for (int x = 0; x < 2; ++x) {
+            const uint8_t* src = a.k8 + (khead_row + (int64_t)(2 * pair + 1 - x) * TILE) * ROW8;
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const int p = (w * 2 + c) * 64 + lane;
+                const int row = p / CPR8, slot = p % CPR8;
+                const int cb = slot ^ ((row >> 1) & (CPR8 - 1));
+                load16_to_lds_sv((uint32_t)(row * ROW8 + cb * 16), src, k8d0 + x * K8_BYTES + (wu * 2 + c) * 1024);
+            }
         }
     }
-    load_q(false);
+    if constexpr (QRAW) {
+        // Q is quantized now, while the first K/V tiles are on their way.  The diagonal tile's 8-bit fragments come out
+        // of the same pass and are parked in LDS (each lane reads back only what it wrote itself): at the diagonal tile
+        // the loads and the conversion would sit on the wave's critical path.
+        v8i q8f[SST];
+        if constexpr (MODE == MPSA_MODE_DIAG) {
+            load_q_raw(std::true_type{}, q8f);
+            uint8_t* park = smem + SMEM + tid * 16;
+#pragma unroll
+            for (int s = 0; s < SST; ++s) {
+                *reinterpret_cast<v4i*>(park + (2 * s) * 8192) = (v4i){q8f[s][0], q8f[s][1], q8f[s][2], q8f[s][3]};
+                *reinterpret_cast<v4i*>(park + (2 * s + 1) * 8192) = (v4i){q8f[s][4], q8f[s][5], q8f[s][6], q8f[s][7]};
+            }
+        } else {
+            load_q_raw(std::false_type{}, q8f);
+        }
+    } else {
+        load_q(false);
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
 
@@ -602,7 +621,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
 
 template <int PVT, int FMT8, int MODE, bool QRAW>
 struct PpLds {
-    static inline const bool registered = mpsa_register_lds_kernel(reinterpret_cast<const void*>(attn_pp_kernel<PVT, FMT8, MODE, QRAW>), QRAW ? SMEM_QRAW : SMEM);
+    static inline const bool registered = mpsa_register_lds_kernel(reinterpret_cast<const void*>(attn_pp_kernel<PVT, FMT8, MODE, QRAW>), smem_bytes(QRAW, MODE));
 };
 
 template <int PVT, int FMT8, int MODE, bool QRAW>
@@ -611,7 +630,7 @@ int launch_pp(const AttnArgs& a, hipStream_t st) {
     const int rc = mpsa_ensure_init();
     if (rc != MPSA_OK) return rc;
     dim3 grid((unsigned)(a.B * a.Hq * (a.nt / 2)));
-    hipLaunchKernelGGL((attn_pp_kernel<PVT, FMT8, MODE, QRAW>), grid, dim3(512), QRAW ? SMEM_QRAW : SMEM, st, a);
+    hipLaunchKernelGGL((attn_pp_kernel<PVT, FMT8, MODE, QRAW>), grid, dim3(512), smem_bytes(QRAW, MODE), st, a);
     MPSA_CHECK_LAUNCH("attn(pp)");
     return MPSA_OK;
 }
