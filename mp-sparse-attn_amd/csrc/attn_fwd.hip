@@ -111,8 +111,8 @@ static int attn_entry(const RawQ* rq, const uint8_t* q4, const uint8_t* qs4, con
     if (rq) {
         a.q_raw = rq->q; a.q_sb = rq->strides[0]; a.q_sh = rq->strides[1]; a.q_sn = rq->strides[2]; a.q_pre = rq->pre;
         if (!attn_pp_supported(a, pv_dtype))
-            return mpsa_fail(MPSA_EUNSUPPORTED, "attn: unquantized q needs the paired-tile kernel's shape (causal, D = 128, tile = 128, "
-                                                "sequence a multiple of 256); quantize q with mpsa_attn_prepare and call mpsa_attn_fwd");
+            return mpsa_fail(MPSA_EUNSUPPORTED, "attn: unquantized q needs the paired-tile kernel's shape (D = 128, tile = 128, an even number of tiles; "
+                                                "causal: sequence a multiple of 256; unmasked: at least six tiles); quantize q with mpsa_attn_prepare and call mpsa_attn_fwd");
         return attn_pp_launch(a, pv_dtype, st);
     }
     if (routed) return attn_routed_launch(a, pv_dtype, st);
@@ -170,5 +170,6 @@ extern "C" int mpsa_attn_fwd_q16_supported(int64_t B, int64_t Hq, int64_t Hkv, i
     AttnArgs a = {};
     a.B = (int)B; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.n = (int)n; a.d = (int)D; a.tile = tile; a.causal = causal ? 1 : 0; a.mode = mode;
     a.nt = (int)((n + tile - 1) / (tile > 0 ? tile : 1)); a.n_pad = a.nt * tile;
+    a.nq = a.n; a.ntq = a.nt; a.nq_pad = a.n_pad;
     return (tile == 64 || tile == 128) && attn_pp_supported(a, MPSA_BF16) ? 1 : 0;
 }

@@ -1,4 +1,5 @@
-// Paired-tile ("ping-pong") fused MXFP attention forward for gfx950: causal, D = 128, 128x128 tiles.
+// Paired-tile ("ping-pong") fused MXFP attention forward for gfx950: D = 128, 128x128 tiles, causal or (self-attention of
+// six tiles or more) unmasked.
 //
 // Same arithmetic as attn_fwd.hip (see there for the operand layouts and the reference citations:
 // ours/mxfp_attn_kernel.py:216-359 for the loop, ours/online_routing.py:68-77, :113-118, :160-171 for the causal
@@ -17,7 +18,8 @@
 // only has to move when a score exceeds it by more than a threshold, which the tile's row sum then shows; the wave
 // does such a tile again the careful way (scores from the K tile still in LDS, maximum, rebase of row sum and output
 // accumulators -- P.V(t), relative to the old maximum, is through by then -- and exponentials).
-// The wave's diagonal tile runs as straight-line code after the loop; Y, one tile short of X, idles in the last step.
+// The wave's diagonal tile runs as straight-line code after the loop; in a causal run Y, one tile short of X, idles in
+// the last step.
 //
 // Staging is the one of attn_fwd.hip: 4-bit K tiles (XOR-swizzled rows) and V tiles (operand order) arrive by
 // direct-to-LDS loads, one barrier per key tile; K has three buffers (the tile whose fragments are being pulled into
@@ -40,7 +42,11 @@ constexpr int Q8_BYTES = 512 * 64;              // fused-quantizer variants: eve
 constexpr int SMEM_QRAW = SMEM + Q8_BYTES;
 constexpr int K8_BYTES = TILE * ROW8;           // "diag" runs: the two 8-bit diagonal K tiles of the pair (X's, then Y's), staged in the prologue
 constexpr int CPR8 = ROW8 / 16;
-constexpr int smem_bytes(bool qraw, int mode) { return (qraw ? SMEM_QRAW : SMEM) + (mode == MPSA_MODE_DIAG ? 2 * K8_BYTES : 0); }
+constexpr int Q4_BYTES = 256 * 32;              // fused-quantizer "diag" runs without the causal mask: Y's 4-bit Q fragments, parked while the 8-bit ones are in use
+constexpr int smem_bytes(bool qraw, int mode, bool causal) {
+    return (qraw ? SMEM_QRAW : SMEM) + (mode == MPSA_MODE_DIAG ? 2 * K8_BYTES : 0) + (qraw && mode == MPSA_MODE_DIAG && !causal ? Q4_BYTES : 0);
+}
+static_assert(smem_bytes(true, MPSA_MODE_DIAG, false) <= 160 * 1024, "LDS of a CU");
 constexpr int NWAVES = 8;
 constexpr int VI = V_BYTES / 1024 / NWAVES;     // direct-load instructions per wave for one V tile (4)
 constexpr int NV = KB * 2 * NDB;                // P.V matrix instructions per tile (32)
@@ -49,7 +55,12 @@ static_assert(K_BYTES / 1024 == NWAVES, "one K direct-load instruction per wave"
 // QRAW: Q arrives unquantized (in the P.V dtype) and is MX-quantized here, in registers, with the quantizer's own device
 // functions -- the bits are those mpsa_quantize_mx would have written (ours/quant_mxint8.py:276-351, :164-219 with
 // sm_scale*log2(e) folded in, :479-494), but the codes and scales never travel through HBM.
-template <int PVT, int FMT8, int MODE, bool QRAW>
+//
+// CAUSAL = false: every query tile visits every key tile.  The steps then walk the key tiles in an order of the
+// workgroup's own: first the tiles both groups take in 4 bits, pipelined as above; then, as straight-line steps, the
+// ragged last tile (keys beyond the sequence masked) and the pair's two diagonal tiles 2I (8 bits for Y) and 2I+1
+// (8 bits for X).  Softmax does not care about the order of the keys.
+template <int PVT, int FMT8, int MODE, bool QRAW, bool CAUSAL>
 __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     typedef PV<PVT> P;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -74,9 +85,25 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     const int hq = (unit % a.Hkv) * group + (rem - rank * group);
     const int b = unit / a.Hkv;
     const int kvh = unit % a.Hkv;
-    const int pair = npairs - 1 - rank;
+    const int pair = CAUSAL ? npairs - 1 - rank : rank;
     const int i = 2 * pair + (1 - role);         // this wave's query tile
-    const int nsteps = 2 * pair + 2;             // key tiles 0 .. 2*pair+1, step t visits tile t
+    const int nsteps = CAUSAL ? 2 * pair + 2 : a.nt;      // causal: key tiles 0 .. 2*pair+1, step t visits tile t
+    // Without the mask: steps 0 .. n_plain-1 visit the tiles everybody takes in 4 bits and unmasked, in ascending order; the
+    // remaining steps visit [the ragged last tile, unless the pair holds it,] tile 2I, tile 2I+1 (a run in 4 bits throughout
+    // keeps the natural order and has only its last tile there).
+    const int d0 = 2 * pair, d1 = 2 * pair + 1;
+    const bool ragged = !CAUSAL && a.n < a.n_pad;
+    const int n_plain = CAUSAL ? i
+                        : MODE == MPSA_MODE_DIAG ? a.nt - 2 - ((ragged && d1 != a.nt - 1) ? 1 : 0)
+                                                 : a.nt - 1;       // the last tile, ragged or not, gets the straight-line step
+    auto tile_at = [&](int t) __attribute__((always_inline)) {
+        if constexpr (CAUSAL || MODE != MPSA_MODE_DIAG) {
+            return t;
+        } else {
+            if (t < n_plain) return t + (t >= d0 ? 2 : 0);
+            return t == a.nt - 1 ? d1 : t == a.nt - 2 ? d0 : a.nt - 1;
+        }
+    };
 
     const int64_t qhead_row = ((int64_t)b * a.Hq + hq) * a.n_pad;
     const int64_t khead_row = ((int64_t)b * a.Hkv + kvh) * a.n_pad;
@@ -107,8 +134,11 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     auto load_q_raw = [&](auto want8_c, v8i (&q8f)[SST]) __attribute__((always_inline)) {
 #pragma clang fp contract(off)        // the quantizer's arithmetic, operation by operation
         constexpr bool WANT8 = decltype(want8_c)::value;
+        // rows beyond the sequence (ragged last tile) quantize as zeros, as the standalone quantizer pads them
+        const bool row_ok = CAUSAL || i * TILE + q_local < a.nq;
+        const int64_t row_idx = row_ok ? (int64_t)i * TILE + q_local : (int64_t)a.nq - 1;
         const char* row = static_cast<const char*>(a.q_raw) +
-                          2 * ((int64_t)b * a.q_sb + (int64_t)hq * a.q_sh + ((int64_t)i * TILE + q_local) * a.q_sn);
+                          2 * ((int64_t)b * a.q_sb + (int64_t)hq * a.q_sh + row_idx * a.q_sn);
         uint32_t sbytes = 0, sbytes8 = 0;
 #pragma unroll
         for (int s = 0; s < SST; ++s) {
@@ -119,7 +149,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                 load8<PVT>(row + 2 * (32 * (2 * s + h) + 8 * c), x[c]);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    x[c][e] = x[c][e] * a.q_pre;
+                    x[c][e] = CAUSAL ? x[c][e] * a.q_pre : (row_ok ? x[c][e] * a.q_pre : 0.0f);
                     amax = __builtin_fmaxf(amax, __builtin_fabsf(x[c][e]));
                 }
             }
@@ -180,8 +210,8 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         const uint8_t* qs = (is8 ? a.qs8 : a.qs4) + q_row * (D / 32);
         qsc = (int)(*reinterpret_cast<const uint32_t*>(qs) >> (8 * h));
     };
-    auto load_kscales = [&](int t, bool is8) __attribute__((always_inline)) {
-        const uint8_t* sp = (is8 ? a.ks8 : a.ks4) + (khead_row + (int64_t)t * TILE + r) * (D / 32);
+    auto load_kscales = [&](int tile, bool is8) __attribute__((always_inline)) {
+        const uint8_t* sp = (is8 ? a.ks8 : a.ks4) + (khead_row + (int64_t)tile * TILE + r) * (D / 32);
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
             ksc[kb] = (int)(*reinterpret_cast<const uint32_t*>(sp + kb * 32 * (D / 32)) >> (8 * h));
@@ -207,11 +237,11 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         koff = (uint32_t)(row * ROW4 + cb * 16);
     }
     auto issue_k4 = [&](int t) __attribute__((always_inline)) {
-        const uint8_t* src = a.k4 + (khead_row + (int64_t)t * TILE) * ROW4;
+        const uint8_t* src = a.k4 + (khead_row + (int64_t)tile_at(t) * TILE) * ROW4;
         load16_to_lds_sv(koff, src, kbuf0 + (t % NKBUF) * K_BYTES + wu * 1024);
     };
     auto issue_v = [&](int t) __attribute__((always_inline)) {
-        const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)t * TILE) * (D * 2);
+        const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)tile_at(t) * TILE) * (D * 2);
         uint8_t* dst = vbuf0 + (t & 1) * V_BYTES;
 #pragma unroll
         for (int c = 0; c < VI; ++c) {
@@ -244,13 +274,13 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     v16f st[KB];
     v4i pk[KB][2];
 
-    auto prep_plain = [&](int t) __attribute__((always_inline)) {
-        load_kscales(t, false);
+    auto prep_plain = [&](int t) __attribute__((always_inline)) {       // step t's tile in 4 bits
+        load_kscales(tile_at(t), false);
         read_kf4(t);
     };
-    auto prep_special = [&](int t) __attribute__((always_inline)) {      // this wave's diagonal tile
+    auto prep_special = [&](int t) __attribute__((always_inline)) {      // this wave's diagonal tile (key tile i) at step t
         if constexpr (MODE == MPSA_MODE_DIAG) {
-            load_kscales(t, true);
+            load_kscales(i, true);
             if constexpr (QRAW) {
                 const uint8_t* park = smem + SMEM + tid * 16;
 #pragma unroll
@@ -265,6 +295,21 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             }
         } else {
             prep_plain(t);
+        }
+    };
+    // Y without the causal mask takes a 4-bit tile (2I+1) after its 8-bit one (2I): back to the 4-bit Q fragments
+    int qsc4 = 0;
+    auto restore_q4 = [&]() __attribute__((always_inline)) {
+        if constexpr (QRAW) {
+            const uint8_t* park4 = k8d0 + 2 * K8_BYTES + (tid & 255) * 16;
+#pragma unroll
+            for (int s = 0; s < SST; ++s) {
+                const v4i x = *reinterpret_cast<const v4i*>(park4 + s * 4096);
+                qf[s] = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+            }
+            qsc = qsc4;
+        } else {
+            load_q(false);
         }
     };
     auto s_plain = [&]() __attribute__((always_inline)) {
@@ -298,15 +343,17 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             s_plain();
         }
     };
-    auto softmax = [&](bool first, auto masked_c) __attribute__((always_inline)) {
+    // masked: keys from `limit` on are dead (the causal diagonal tile: the keys after the query; the ragged last tile:
+    // the keys beyond the sequence)
+    auto softmax = [&](bool first, auto masked_c, int limit) __attribute__((always_inline)) {
         __builtin_amdgcn_s_setprio(0);
-        if constexpr (decltype(masked_c)::value) {      // diagonal tile: keys after the query are dead
+        if constexpr (decltype(masked_c)::value) {
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int key = 32 * kb + 8 * (e >> 2) + 4 * h + (e & 3);
-                    if (key > q_local) st[kb][e] = -__builtin_inff();
+                    if (key >= limit) st[kb][e] = -__builtin_inff();
                 }
         }
         float mx = st[0][0];
@@ -513,6 +560,15 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         v8i q8f[SST];
         if constexpr (MODE == MPSA_MODE_DIAG) {
             load_q_raw(std::true_type{}, q8f);
+            if constexpr (!CAUSAL) {
+                qsc4 = qsc;
+                if (role == 1) {
+                    uint8_t* park4 = k8d0 + 2 * K8_BYTES + (tid & 255) * 16;
+#pragma unroll
+                    for (int s = 0; s < SST; ++s)
+                        *reinterpret_cast<v4i*>(park4 + s * 4096) = (v4i){qf[s][0], qf[s][1], qf[s][2], qf[s][3]};
+                }
+            }
             uint8_t* park = smem + SMEM + tid * 16;
 #pragma unroll
             for (int s = 0; s < SST; ++s) {
@@ -528,42 +584,78 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
 
-    // Step t (between barriers t and t+1): S(t+1), then P.V(t) with the softmax of t+1 in its gaps.  The wave's last
-    // key tile (the diagonal one, index i) gets straight-line code; Y, one tile short of X, idles through the last step.
-    const int last = i;
-    if (last == 0) {
-        prep_special(0);
-        s_special(0);
-        softmax(true, std::true_type{});
+    // Step t (between barriers t and t+1): S(t+1), then P.V(t) with the softmax of t+1 in its gaps.  The first `last`
+    // steps take plain tiles; the tiles after them get straight-line code.
+    const int last = n_plain;
+    if constexpr (CAUSAL) {
+        // the wave's last key tile is the diagonal one (index i); Y, one tile short of X, idles through the last step
+        if (last == 0) {
+            prep_special(0);
+            s_special(0);
+            softmax(true, std::true_type{}, q_local + 1);
+        } else {
+            prep_plain(0);
+            s_plain();
+            softmax(true, std::false_type{}, 0);
+            if (last >= 2) prep_plain(1);
+        }
     } else {
         prep_plain(0);
         s_plain();
-        softmax(true, std::false_type{});
+        softmax(true, std::false_type{}, 0);
         if (last >= 2) prep_plain(1);
     }
     for (int t = 0; t + 2 <= last; ++t) {
         sync_issue(t);
         s_plain();
-        load_kscales(t + 2, false);
+        load_kscales(tile_at(t + 2), false);
         pv_exp(t);
     }
-    if (last >= 1) {
-        const int t = last - 1;
-        sync_issue(t);
-        prep_special(t + 1);
-        pv(t);
-        s_special(t + 1);
-        softmax(false, std::true_type{});
+    if constexpr (CAUSAL) {
+        if (last >= 1) {
+            const int t = last - 1;
+            sync_issue(t);
+            prep_special(t + 1);
+            pv(t);
+            s_special(t + 1);
+            softmax(false, std::true_type{}, q_local + 1);
+        }
+        sync_issue(last);
+        pv(last);
+        if (role == 1) sync_issue(last + 1);
+    } else {
+        bool q_is8 = false;
+#pragma nounroll
+        for (int t = last - 1; t + 1 < nsteps; ++t) {          // P.V(t) is pending; step t+1's tile comes next
+            const int j = tile_at(t + 1);
+            const bool is8 = MODE == MPSA_MODE_DIAG && j == i;
+            const int limit = (ragged && j == a.nt - 1) ? a.n - j * TILE : TILE;
+            sync_issue(t);
+            if (is8) {
+                prep_special(t + 1);
+                q_is8 = true;
+            } else {
+                prep_plain(t + 1);
+                if (q_is8) restore_q4();
+                q_is8 = false;
+            }
+            pv(t);
+            if (is8) s_special(t + 1);
+            else s_plain();
+            softmax(false, std::true_type{}, limit);
+        }
+        sync_issue(nsteps - 1);
+        pv(nsteps - 1);
     }
-    sync_issue(last);
-    pv(last);
-    if (role == 1) sync_issue(last + 1);
     __builtin_amdgcn_s_waitcnt(0x0F70);                // no direct-to-LDS load may outlive the workgroup
 
     // ---- epilogue: O = acc / l ; register e of lane (h, r): dim 32*db + 8*(e/4) + 4*h + e%4 of query r ----
     const float l_tot = sum_lane_pair(l_run);
     const float inv = 1.0f / l_tot;
     const int q_global = i * TILE + q_local;
+    if constexpr (!CAUSAL) {
+        if (q_global >= a.nq) return;                   // a row of the ragged last tile's padding (both lanes of a query leave together)
+    }
     uint8_t* orow = static_cast<uint8_t*>(a.o);
     const int64_t off = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh + (int64_t)q_global * a.o_sn;
     if (a.o_dtype != MPSA_F32 && ((a.o_sn | a.o_sh | a.o_sb) & 7) == 0 && (reinterpret_cast<uintptr_t>(a.o) & 15) == 0) {
@@ -619,20 +711,25 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         }
 }
 
-template <int PVT, int FMT8, int MODE, bool QRAW>
+template <int PVT, int FMT8, int MODE, bool QRAW, bool CAUSAL>
 struct PpLds {
-    static inline const bool registered = mpsa_register_lds_kernel(reinterpret_cast<const void*>(attn_pp_kernel<PVT, FMT8, MODE, QRAW>), smem_bytes(QRAW, MODE));
+    static inline const bool registered = mpsa_register_lds_kernel(reinterpret_cast<const void*>(attn_pp_kernel<PVT, FMT8, MODE, QRAW, CAUSAL>), smem_bytes(QRAW, MODE, CAUSAL));
 };
 
-template <int PVT, int FMT8, int MODE, bool QRAW>
-int launch_pp(const AttnArgs& a, hipStream_t st) {
-    if (!PpLds<PVT, FMT8, MODE, QRAW>::registered) return mpsa_fail(MPSA_ELAUNCH, "attn: kernel not registered");
+template <int PVT, int FMT8, int MODE, bool QRAW, bool CAUSAL>
+int launch_pp_c(const AttnArgs& a, hipStream_t st) {
+    if (!PpLds<PVT, FMT8, MODE, QRAW, CAUSAL>::registered) return mpsa_fail(MPSA_ELAUNCH, "attn: kernel not registered");
     const int rc = mpsa_ensure_init();
     if (rc != MPSA_OK) return rc;
     dim3 grid((unsigned)(a.B * a.Hq * (a.nt / 2)));
-    hipLaunchKernelGGL((attn_pp_kernel<PVT, FMT8, MODE, QRAW>), grid, dim3(512), smem_bytes(QRAW, MODE), st, a);
+    hipLaunchKernelGGL((attn_pp_kernel<PVT, FMT8, MODE, QRAW, CAUSAL>), grid, dim3(512), smem_bytes(QRAW, MODE, CAUSAL), st, a);
     MPSA_CHECK_LAUNCH("attn(pp)");
     return MPSA_OK;
+}
+
+template <int PVT, int FMT8, int MODE, bool QRAW>
+int launch_pp(const AttnArgs& a, hipStream_t st) {
+    return a.causal ? launch_pp_c<PVT, FMT8, MODE, QRAW, true>(a, st) : launch_pp_c<PVT, FMT8, MODE, QRAW, false>(a, st);
 }
 
 template <int PVT, bool QRAW>
@@ -644,7 +741,8 @@ int launch_pp_mode(const AttnArgs& a, hipStream_t st) {
 
 }  // namespace
 
-// The paired-tile kernel covers causal runs over whole pairs of full 128-query tiles with D = 128.
+// The paired-tile kernel covers D = 128 with 128-key tiles over whole pairs of query tiles: causal runs of full tiles, and
+// self-attention without the mask from six tiles on (there the last tile may be ragged).
 // MPSA_ATTN_PP=0 in the environment switches it off (the general kernel then runs everything).
 bool attn_pp_supported(const AttnArgs& a, int pv_dtype) {
     static const bool enabled = [] {
@@ -652,8 +750,9 @@ bool attn_pp_supported(const AttnArgs& a, int pv_dtype) {
         return !(v && v[0] == '0');
     }();
     (void)pv_dtype;
-    return enabled && a.causal && a.d == 128 && a.tile == 128 && a.n == a.n_pad && (a.nt % 2) == 0 &&
-           (a.mode == MPSA_MODE_DIAG || a.mode == MPSA_MODE_MXFP4);
+    if (!enabled || a.d != 128 || a.tile != 128 || (a.nt % 2) != 0 || (a.mode != MPSA_MODE_DIAG && a.mode != MPSA_MODE_MXFP4)) return false;
+    if (a.causal) return a.n == a.n_pad;
+    return a.nq == a.n && a.nt >= 6;
 }
 
 int attn_pp_launch(const AttnArgs& a, int pv_dtype, hipStream_t st) {

@@ -531,7 +531,8 @@ def test_q_quantized_inside_the_attention_kernel_gives_the_same_bits(bst, N, sca
     qd = q.to(DEV).transpose(1, 2).contiguous().transpose(1, 2)   # [B,H,N,D] view of an [B,N,H,D] tensor
     kd, vd = k.to(DEV), v.to(DEV)
     assert not qd.is_contiguous() and q_fusable(qd, kd, 128, bst, True)
-    assert not q_fusable(qd, kd, 128, bst, False) and not q_fusable(qd, kd, 64, bst, True) and not q_fusable(qd, kd, 128, "mxfp8", True)
+    assert q_fusable(qd, kd, 128, bst, False) == (N >= 768)       # without the mask: from six tiles on
+    assert not q_fusable(qd, kd, 64, bst, True) and not q_fusable(qd, kd, 128, "mxfp8", True)
     a = torch.empty((2, 8, N, 128), dtype=dtype, device=DEV)
     b = torch.empty_like(a)
     attention_from_operands(prepare_operands(qd, kd, vd, 128, bst, scale), a, True)
@@ -545,6 +546,33 @@ def test_q_quantized_inside_the_attention_kernel_gives_the_same_bits(bst, N, sca
     want = O.attn_mx(q, k, v, tile=128, causal=True, mode="diag" if bst.startswith("diag") else "mxfp4", scale=scale,
                      fmt8=O.FMT_E5M2 if bst.endswith("e5") else O.FMT_E4M3, out_dtype=torch.float32)
     _compare(mxfp_attn_kernel(qd, kd, vd, is_causal=True, scale=scale, block_scale_type=bst, output_dtype=torch.float32), want, f"fused q {bst} N={N}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("bst", ["diag", "mxfp4", "diag_e5"])
+@pytest.mark.parametrize("N", [768, 1000, 1024, 1665, 2047])
+def test_paired_tile_kernel_without_the_causal_mask(bst, N, dtype):
+    """Self-attention without the mask on the paired-tile kernel (D = 128, 128-key tiles, an even number of tiles from
+    six on): whole tiles (768, 1024), a ragged last tile that is some pair's own diagonal tile and every other pair's
+    masked extra step (1000: 8 tiles; 2047: 16 tiles, one key short), and a last tile holding a single key (1665 = 13 * 128 + 1:
+    14 tiles).  Against the oracle at the float32 bar; Q quantized inside the kernel gives the bits of the prepared
+    route; grouped heads, outlier channels, all-zero MX blocks."""
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, q_fusable
+    q, k, v = make_qkv(1, 4, 2, N, 128, seed=900 + N, dtype=dtype, outliers=True)
+    q[0, 0, :40] = 0
+    q[0, 3, N - 1, 32:64] = 0
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    assert q_fusable(qd, kd, 128, bst, False)
+    mode = "diag" if bst.startswith("diag") else "mxfp4"
+    fmt8 = O.FMT_E5M2 if bst.endswith("e5") else O.FMT_E4M3
+    want = O.attn_mx(q, k, v, tile=128, causal=False, mode=mode, fmt8=fmt8, out_dtype=torch.float32)
+    _check(q, k, v, want, f"paired, no mask, {bst} N={N} {dtype}", out16=dtype, is_causal=False, block_scale_type=bst, tile=128)
+    a = torch.full((1, 4, N, 128), float("nan"), dtype=torch.float32, device=DEV)
+    b = torch.full_like(a, float("nan"))
+    attention_from_operands(prepare_operands(qd, kd, vd, 128, bst), a, False)
+    attention_from_operands(prepare_operands(qd, kd, vd, 128, bst, fuse_q=True), b, False)
+    assert torch.isfinite(a).all() and torch.equal(a, b)
+    _compare(a, want, f"paired, no mask, prepared route, {bst} N={N}")
 
 
 @pytest.mark.parametrize("bst", ["mxfp4", "mxfp8", "diag", "mixed_e5"])
@@ -595,7 +623,10 @@ def test_q_with_infinities_quantizes_to_the_same_codes_in_the_kernel(bst):
 def test_q16_entry_point_rejects_other_shapes():
     L = _lib.lib()
     assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 128, 128, 1, _lib.MODE_DIAG) == 1
-    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 128, 128, 0, _lib.MODE_DIAG) == 0      # not causal
+    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 128, 128, 0, _lib.MODE_DIAG) == 1      # no mask: six tiles or more,
+    assert L.mpsa_attn_fwd_q16_supported(1, 40, 40, 32760, 128, 128, 0, _lib.MODE_DIAG) == 1    # the last one may be ragged
+    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 512, 128, 128, 0, _lib.MODE_DIAG) == 0
+    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192 - 8, 128, 128, 1, _lib.MODE_DIAG) == 0  # causal: whole tiles only
     assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192 + 128, 128, 128, 1, _lib.MODE_DIAG) == 0  # an odd number of tiles
     assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 64, 128, 1, _lib.MODE_DIAG) == 0
     assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 128, 128, 1, _lib.MODE_MXFP8) == 0

@@ -67,42 +67,57 @@ def test_attention_sweep(sweep_seed):
         check_attention(run, want, what, p["dt"])
 
 
-def test_paired_tile_kernel_sweep():
-    """The paired-tile kernel's shapes (causal, D = 128, 128x128 tiles, whole tile pairs) with score profiles that
-    make its running maximum move at unpredictable places: per-64-row gains, scores climbing along the keys at
-    different rates, and random tiles towering over the rest."""
-    rnd = random.Random(21)
-    for c in range(40):
+def _paired_tile_sweep(causal, sweep_seed, cases):
+    rnd = random.Random(sweep_seed)
+    for c in range(cases):
         Hkv = rnd.choice([1, 2]); Hq = Hkv * rnd.choice([1, 2, 4])
-        N = 256 * rnd.randint(1, 6)
+        if causal:
+            N = 256 * rnd.randint(1, 6)
+        else:
+            N = 256 * rnd.randint(3, 7) - rnd.choice([0, 0, 1, 37, 100, 127])    # an even number of tiles, the last one ragged or not
         mode = rnd.choice(["mxfp4", "diag", "diag", "diag_e5"])
         dt = rnd.choice([torch.bfloat16, torch.float16])
         seed = rnd.randint(0, 10 ** 6)
         shape = rnd.choice(["gain", "ramp", "spikes"])
         rate = rnd.choice([0.5, 1.0, 3.0, 5.0]); height = rnd.choice([2.0, 6.0, 9.0])
-        what = f"paired sweep case {c}: Hq={Hq} Hkv={Hkv} N={N} mode={mode} {dt} seed={seed} {shape} rate={rate} height={height}"
+        what = f"paired sweep case {c}: causal={causal} Hq={Hq} Hkv={Hkv} N={N} mode={mode} {dt} seed={seed} {shape} rate={rate} height={height}"
         print(what, flush=True)
         q, k, v = make_qkv(1, Hq, Hkv, N, 128, seed=seed, dtype=dt)
         g = torch.Generator().manual_seed(seed + 7)
+        nt = (N + 127) // 128
         if shape == "gain":
             for t in (q, k):
-                gain = torch.exp2(torch.randint(-3, 3, (1, t.shape[1], N // 64, 1), generator=g).float())
-                t *= gain.repeat_interleave(64, dim=2).to(t.dtype)
+                gain = torch.exp2(torch.randint(-3, 3, (1, t.shape[1], 2 * nt, 1), generator=g).float())
+                t *= gain.repeat_interleave(64, dim=2)[:, :, :N].to(t.dtype)
         else:
             u = torch.sign(torch.randn(128, generator=g))
             if shape == "ramp":
                 gk = torch.arange(N, dtype=torch.float32) / 128 * rate
             else:
-                gk = (torch.rand(N // 128, generator=g) < 0.3).float().repeat_interleave(128) * height
+                gk = ((torch.rand(nt, generator=g) < 0.3).float().repeat_interleave(128) * height)[:N]
             q = (q.float() * 0.3 + u).to(dt)
             k = (k.float() * 0.3 + gk[:, None] * u).to(dt)
         fmt8 = O.FMT_E5M2 if mode.endswith("e5") else O.FMT_E4M3
-        got = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=True, block_scale_type=mode, tile=128,
+        got = mxfp_attn_kernel(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=causal, block_scale_type=mode, tile=128,
                                output_dtype=torch.float32)
-        want = O.attn_mx(q, k, v, tile=128, causal=True, mode="diag" if mode.startswith("diag") else mode, fmt8=fmt8,
+        want = O.attn_mx(q, k, v, tile=128, causal=causal, mode="diag" if mode.startswith("diag") else mode, fmt8=fmt8,
                          out_dtype=torch.float32)
         assert torch.isfinite(got).all(), what
         attention_close(got, want, what)
+
+
+def test_paired_tile_kernel_sweep():
+    """The paired-tile kernel's causal shapes (D = 128, 128x128 tiles, whole tile pairs) with score profiles that
+    make its running maximum move at unpredictable places: per-64-row gains, scores climbing along the keys at
+    different rates, and random tiles towering over the rest."""
+    _paired_tile_sweep(True, 21, 40)
+
+
+def test_paired_tile_kernel_sweep_without_the_mask():
+    """The same score profiles on the kernel's unmasked shapes (six tiles or more, an even number, the last one ragged in
+    most cases): the tiles are visited out of order there -- the pair's two diagonal tiles and the ragged tile last --
+    so a running maximum that moves in the late straight-line steps is covered too (the ramp peaks in the last tile)."""
+    _paired_tile_sweep(False, 22, 30)
 
 
 def test_matmul_sweep():
