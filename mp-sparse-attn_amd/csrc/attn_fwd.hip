@@ -111,8 +111,8 @@ static int attn_entry(const RawQ* rq, const uint8_t* q4, const uint8_t* qs4, con
     if (rq) {
         a.q_raw = rq->q; a.q_sb = rq->strides[0]; a.q_sh = rq->strides[1]; a.q_sn = rq->strides[2]; a.q_pre = rq->pre;
         if (!attn_pp_supported(a, pv_dtype))
-            return mpsa_fail(MPSA_EUNSUPPORTED, "attn: unquantized q needs the paired-tile kernel's shape (D = 128, tile = 128, an even number of tiles; "
-                                                "causal: sequence a multiple of 256; unmasked: at least six tiles); quantize q with mpsa_attn_prepare and call mpsa_attn_fwd");
+            return mpsa_fail(MPSA_EUNSUPPORTED, "attn: unquantized q needs the paired-tile kernel's shape (D = 128, tile = 128; "
+                                                "causal: at least two tiles, unmasked: at least six); quantize q with mpsa_attn_prepare and call mpsa_attn_fwd");
         return attn_pp_launch(a, pv_dtype, st);
     }
     if (routed) return attn_routed_launch(a, pv_dtype, st);

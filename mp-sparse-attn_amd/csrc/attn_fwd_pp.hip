@@ -73,7 +73,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     const int wq = wu & 3;
 
     // ---- which (batch, kv head, query head, query-tile pair) -- XCD-aware, heavy pairs first ----
-    const int npairs = a.nt >> 1;
+    const int npairs = (a.nt + 1) >> 1;          // an odd tile count leaves the last pair with its lower tile only
     const int group = a.Hq / a.Hkv;
     const int total = a.B * a.Hq * npairs;
     int L = blockIdx.x;
@@ -87,13 +87,16 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     const int kvh = unit % a.Hkv;
     const int pair = CAUSAL ? npairs - 1 - rank : rank;
     const int i = 2 * pair + (1 - role);         // this wave's query tile
-    const int nsteps = CAUSAL ? 2 * pair + 2 : a.nt;      // causal: key tiles 0 .. 2*pair+1, step t visits tile t
+    const bool lone = 2 * pair + 1 >= a.nt;      // the pair without an upper tile: X has no queries and only helps with the staging
+    const bool inactive = lone && role == 0;
+    const int nsteps = CAUSAL ? 2 * pair + (lone ? 1 : 2) : a.nt;      // causal: key tiles 0 .. 2*pair+1, step t visits tile t
     // Without the mask: steps 0 .. n_plain-1 visit the tiles everybody takes in 4 bits and unmasked, in ascending order; the
     // remaining steps visit [the ragged last tile, unless the pair holds it,] tile 2I, tile 2I+1 (a run in 4 bits throughout
     // keeps the natural order and has only its last tile there).
     const int d0 = 2 * pair, d1 = 2 * pair + 1;
     const bool ragged = !CAUSAL && a.n < a.n_pad;
     const int n_plain = CAUSAL ? i
+                        : lone ? a.nt - 1
                         : MODE == MPSA_MODE_DIAG ? a.nt - 2 - ((ragged && d1 != a.nt - 1) ? 1 : 0)
                                                  : a.nt - 1;       // the last tile, ragged or not, gets the straight-line step
     auto tile_at = [&](int t) __attribute__((always_inline)) {
@@ -101,6 +104,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             return t;
         } else {
             if (t < n_plain) return t + (t >= d0 ? 2 : 0);
+            if (lone) return d0;
             return t == a.nt - 1 ? d1 : t == a.nt - 2 ? d0 : a.nt - 1;
         }
     };
@@ -116,8 +120,8 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
 
     // ---- operands in registers ----
     v8i qf[SST];
-    int qsc = 0;
-    int qsc8 = 0;                                // fused-quantizer variants: scale bytes of the parked 8-bit Q fragments
+    int qsc = 0;                                 // Q's scale bytes (bytes 0 and 2 of the word; the fused-quantizer variants keep
+                                                 // those of the parked 8-bit fragments in bytes 1 and 3)
     v4i kf4[KB][SST];
     int ksc[KB];
     // shared exponent of an MX block from its largest magnitude, as the quantizer takes it (quantize_kernel.h)
@@ -134,8 +138,8 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     auto load_q_raw = [&](auto want8_c, v8i (&q8f)[SST]) __attribute__((always_inline)) {
 #pragma clang fp contract(off)        // the quantizer's arithmetic, operation by operation
         constexpr bool WANT8 = decltype(want8_c)::value;
-        // rows beyond the sequence (ragged last tile) quantize as zeros, as the standalone quantizer pads them
-        const bool row_ok = CAUSAL || i * TILE + q_local < a.nq;
+        // rows beyond the sequence (ragged last tile) read the last row instead and are zeroed below
+        const bool row_ok = i * TILE + q_local < a.nq;
         const int64_t row_idx = row_ok ? (int64_t)i * TILE + q_local : (int64_t)a.nq - 1;
         const char* row = static_cast<const char*>(a.q_raw) +
                           2 * ((int64_t)b * a.q_sb + (int64_t)hq * a.q_sh + row_idx * a.q_sn);
@@ -149,7 +153,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                 load8<PVT>(row + 2 * (32 * (2 * s + h) + 8 * c), x[c]);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    x[c][e] = CAUSAL ? x[c][e] * a.q_pre : (row_ok ? x[c][e] * a.q_pre : 0.0f);
+                    x[c][e] = x[c][e] * a.q_pre;
                     amax = __builtin_fmaxf(amax, __builtin_fabsf(x[c][e]));
                 }
             }
@@ -187,8 +191,17 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                 sbytes8 |= (uint32_t)(zero ? 0 : min(max(se8 + 127, 0), 254)) << (16 * s);
             }
         }
-        qsc = (int)sbytes;
-        qsc8 = (int)sbytes8;
+        qsc = (int)(sbytes | (sbytes8 << 8));
+        if (i * TILE + 32 * wq + 31 >= a.nq) {            // a wave of the ragged last tile: zero codes and scales for its padding
+#pragma unroll                                            // rows, as the standalone quantizer pads them
+            for (int s = 0; s < SST; ++s)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    qf[s][e] = row_ok ? qf[s][e] : 0;
+                    if constexpr (WANT8) q8f[s][e] = row_ok ? q8f[s][e] : 0;
+                }
+            qsc = row_ok ? qsc : 0;
+        }
     };
     auto load_q = [&](bool is8) __attribute__((always_inline)) {
         if constexpr (QRAW) return;                   // the fused-quantizer variants fill the fragments in the prologue
@@ -289,7 +302,6 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                     const v4i x1 = *reinterpret_cast<const v4i*>(park + (2 * s + 1) * 8192);
                     qf[s] = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
                 }
-                qsc = qsc8;
             } else {
                 load_q(true);
             }
@@ -298,7 +310,6 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         }
     };
     // Y without the causal mask takes a 4-bit tile (2I+1) after its 8-bit one (2I): back to the 4-bit Q fragments
-    int qsc4 = 0;
     auto restore_q4 = [&]() __attribute__((always_inline)) {
         if constexpr (QRAW) {
             const uint8_t* park4 = k8d0 + 2 * K8_BYTES + (tid & 255) * 16;
@@ -307,7 +318,6 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                 const v4i x = *reinterpret_cast<const v4i*>(park4 + s * 4096);
                 qf[s] = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
             }
-            qsc = qsc4;
         } else {
             load_q(false);
         }
@@ -326,6 +336,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         if constexpr (MODE == MPSA_MODE_DIAG) {
             // this wave's 8-bit diagonal K tile has been in LDS since the prologue (rows XOR-swizzled like the 4-bit ones)
             const uint8_t* kl = k8d0 + role * K8_BYTES;
+            const int qs8 = QRAW ? (int)((uint32_t)qsc >> 8) : qsc;
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
                 const int krow = 32 * kb + r;
@@ -336,7 +347,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                     const v4i x0 = *reinterpret_cast<const v4i*>(kl + krow * ROW8 + (((4 * s + h) ^ f) * 16));
                     const v4i x1 = *reinterpret_cast<const v4i*>(kl + krow * ROW8 + (((4 * s + h + 2) ^ f) * 16));
                     const v8i kd = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-                    st[kb] = score_mfma8<FMT8>(kd, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
+                    st[kb] = score_mfma8<FMT8>(kd, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qs8);
                 }
             }
         } else {
@@ -536,13 +547,14 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     // ---- prologue (all waves): V(0), K(0..2) on their way; Q into registers ----
     issue_v(0);
     issue_k4(0);
-    issue_k4(1);
+    if (nsteps > 1) issue_k4(1);
     if (nsteps > 2) issue_k4(2);
     if constexpr (MODE == MPSA_MODE_DIAG) {
         // the pair's two diagonal tiles in 8 bits (X's: key tile 2I+1, Y's: 2I), 16 one-KiB pieces each, two per wave:
         // piece position p = 8 row + slot holds the row's 16-byte chunk slot ^ ((row >> 1) & 7)
 #pragma unroll
         for (int x = 0; x < 2; ++x) {
+            if (lone && x == 0) continue;
             const uint8_t* src = a.k8 + (khead_row + (int64_t)(2 * pair + 1 - x) * TILE) * ROW8;
 #pragma unroll
             for (int c = 0; c < 2; ++c) {
@@ -553,7 +565,9 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             }
         }
     }
-    if constexpr (QRAW) {
+    if (inactive) {
+        // no queries here: this wave only issues its share of the staging loads and keeps the barriers' count
+    } else if constexpr (QRAW) {
         // Q is quantized now, while the first K/V tiles are on their way.  The diagonal tile's 8-bit fragments come out
         // of the same pass and are parked in LDS (each lane reads back only what it wrote itself): at the diagonal tile
         // the loads and the conversion would sit on the wave's critical path.
@@ -561,7 +575,6 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         if constexpr (MODE == MPSA_MODE_DIAG) {
             load_q_raw(std::true_type{}, q8f);
             if constexpr (!CAUSAL) {
-                qsc4 = qsc;
                 if (role == 1) {
                     uint8_t* park4 = k8d0 + 2 * K8_BYTES + (tid & 255) * 16;
 #pragma unroll
@@ -583,6 +596,12 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
+    if (inactive) {
+        const int nsync = CAUSAL ? nsteps + 1 : nsteps;
+        for (int t = 0; t < nsync; ++t) sync_issue(t);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        return;
+    }
 
     // Step t (between barriers t and t+1): S(t+1), then P.V(t) with the softmax of t+1 in its gaps.  The first `last`
     // steps take plain tiles; the tiles after them get straight-line code.
@@ -653,9 +672,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     const float l_tot = sum_lane_pair(l_run);
     const float inv = 1.0f / l_tot;
     const int q_global = i * TILE + q_local;
-    if constexpr (!CAUSAL) {
-        if (q_global >= a.nq) return;                   // a row of the ragged last tile's padding (both lanes of a query leave together)
-    }
+    if (q_global >= a.nq) return;                       // a row of the ragged last tile's padding (both lanes of a query leave together)
     uint8_t* orow = static_cast<uint8_t*>(a.o);
     const int64_t off = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh + (int64_t)q_global * a.o_sn;
     if (a.o_dtype != MPSA_F32 && ((a.o_sn | a.o_sh | a.o_sb) & 7) == 0 && (reinterpret_cast<uintptr_t>(a.o) & 15) == 0) {
@@ -721,7 +738,7 @@ int launch_pp_c(const AttnArgs& a, hipStream_t st) {
     if (!PpLds<PVT, FMT8, MODE, QRAW, CAUSAL>::registered) return mpsa_fail(MPSA_ELAUNCH, "attn: kernel not registered");
     const int rc = mpsa_ensure_init();
     if (rc != MPSA_OK) return rc;
-    dim3 grid((unsigned)(a.B * a.Hq * (a.nt / 2)));
+    dim3 grid((unsigned)(a.B * a.Hq * ((a.nt + 1) / 2)));
     hipLaunchKernelGGL((attn_pp_kernel<PVT, FMT8, MODE, QRAW, CAUSAL>), grid, dim3(512), smem_bytes(QRAW, MODE, CAUSAL), st, a);
     MPSA_CHECK_LAUNCH("attn(pp)");
     return MPSA_OK;
@@ -741,8 +758,9 @@ int launch_pp_mode(const AttnArgs& a, hipStream_t st) {
 
 }  // namespace
 
-// The paired-tile kernel covers D = 128 with 128-key tiles over whole pairs of query tiles: causal runs of full tiles, and
-// self-attention without the mask from six tiles on (there the last tile may be ragged).
+// The paired-tile kernel covers self-attention with D = 128 and 128-key tiles: causal runs from two tiles on, runs without
+// the mask from six tiles on; the last tile may be ragged, and with an odd number of tiles the last workgroup of a head
+// works on its one tile with half of its waves.
 // MPSA_ATTN_PP=0 in the environment switches it off (the general kernel then runs everything).
 bool attn_pp_supported(const AttnArgs& a, int pv_dtype) {
     static const bool enabled = [] {
@@ -750,9 +768,8 @@ bool attn_pp_supported(const AttnArgs& a, int pv_dtype) {
         return !(v && v[0] == '0');
     }();
     (void)pv_dtype;
-    if (!enabled || a.d != 128 || a.tile != 128 || (a.nt % 2) != 0 || (a.mode != MPSA_MODE_DIAG && a.mode != MPSA_MODE_MXFP4)) return false;
-    if (a.causal) return a.n == a.n_pad;
-    return a.nq == a.n && a.nt >= 6;
+    if (!enabled || a.d != 128 || a.tile != 128 || a.nq != a.n || (a.mode != MPSA_MODE_DIAG && a.mode != MPSA_MODE_MXFP4)) return false;
+    return a.nt >= (a.causal ? 2 : 6);
 }
 
 int attn_pp_launch(const AttnArgs& a, int pv_dtype, hipStream_t st) {

@@ -59,7 +59,7 @@ def _prepare(q, k, mode, scale, fmt8):
 
 def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=False,
             fmt8=FMT_E4M3, out_dtype=None, heads=None, q_tiles=None, skip_thresh=None, return_skipped=False,
-            ratios_out=None, route=None):
+            ratios_out=None, route=None, score8=None):
     """Tile-by-tile MXFP attention.  q ``[B,Hq,N,D]``, k/v ``[B,Hkv,N,D]`` in bf16 or fp16.
 
     P is rounded to v's dtype before P.V and the product of a tile is accumulated in float32
@@ -76,7 +76,11 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
     a list passed as ``ratios_out`` collects statistic(j) / statistic(0) of every tile j > 0 examined.
 
     ``mode="routed"``: ``route`` ``[B,Hq,tiles,key tiles]`` gives every tile's class (0 skip, 1 4-bit, 2 8-bit, 255 not
-    visited), see :mod:`oracle.mx_route`; a query row whose every tile is skipped returns zeros."""
+    visited), see :mod:`oracle.mx_route`; a query row whose every tile is skipped returns zeros.
+
+    ``score8``: optional callable ``(q_tile, k_tile) -> scores`` that replaces the float32 product ``q_tile @ k_tile.T`` for
+    tiles whose two operands are 8-bit -- the tests use it to put a model of a matrix unit's accumulation in place of the
+    exact product; the default is the reference's arithmetic."""
     B, Hq, N, D = q.shape
     Hkv, Nk = k.shape[1], k.shape[2]
     assert Hq % Hkv == 0
@@ -117,7 +121,10 @@ def attn_mx(q, k, v, tile=128, causal=True, mode="diag", scale=None, smooth_k=Fa
                     qtag, ktag = _tile_tags(mode, i, j, None if route is None else route[b, h])
                     qt = ops["q" + qtag][b, hi_, r0:r1]
                     kt = ops["k" + ktag][b, kvh, c0:c1]
-                    s = qt @ kt.T                                    # float32, already in log2 units
+                    if score8 is not None and qtag == "8" and ktag == "8":
+                        s = score8(qt, kt)
+                    else:
+                        s = qt @ kt.T                                # float32, already in log2 units
                     if causal and j == i:
                         rr = torch.arange(r0, r1).unsqueeze(1)
                         cc = torch.arange(c0, c1).unsqueeze(0)

@@ -67,14 +67,16 @@ def test_attention_sweep(sweep_seed):
         check_attention(run, want, what, p["dt"])
 
 
-def _paired_tile_sweep(causal, sweep_seed, cases):
+def _paired_tile_sweep(causal, sweep_seed, cases, any_length=False):
     rnd = random.Random(sweep_seed)
     for c in range(cases):
         Hkv = rnd.choice([1, 2]); Hq = Hkv * rnd.choice([1, 2, 4])
-        if causal:
+        if causal and any_length:
+            N = 128 * rnd.randint(2, 12) - rnd.choice([0, 1, 37, 100, 127])
+        elif causal:
             N = 256 * rnd.randint(1, 6)
         else:
-            N = 256 * rnd.randint(3, 7) - rnd.choice([0, 0, 1, 37, 100, 127])    # an even number of tiles, the last one ragged or not
+            N = 128 * rnd.randint(6, 14) - rnd.choice([0, 0, 1, 37, 100, 127])    # the last tile ragged or not
         mode = rnd.choice(["mxfp4", "diag", "diag", "diag_e5"])
         dt = rnd.choice([torch.bfloat16, torch.float16])
         seed = rnd.randint(0, 10 ** 6)
@@ -113,9 +115,13 @@ def test_paired_tile_kernel_sweep():
     _paired_tile_sweep(True, 21, 40)
 
 
+def test_paired_tile_kernel_sweep_causal_any_length():
+    """The same with lengths that leave the last tile ragged or the last pair with one tile."""
+    _paired_tile_sweep(True, 23, 30, any_length=True)
+
+
 def test_paired_tile_kernel_sweep_without_the_mask():
-    """The same score profiles on the kernel's unmasked shapes (six tiles or more, an even number, the last one ragged in
-    most cases): the tiles are visited out of order there -- the pair's two diagonal tiles and the ragged tile last --
+    """The same score profiles on the kernel's unmasked shapes (six tiles or more, the last one ragged in most cases): the tiles are visited out of order there -- the pair's two diagonal tiles and the ragged tile last --
     so a running maximum that moves in the late straight-line steps is covered too (the ramp peaks in the last tile)."""
     _paired_tile_sweep(False, 22, 30)
 
