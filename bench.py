@@ -207,7 +207,7 @@ def secondary_c5(device):
     """The video-DiT configuration (non-causal, N = 32760, 40 heads) next to the headline line: the diag mode's kernel and
     whole step, and the routed mode (tile router on the scale bytes + routed attention) at the default thresholds with
     the shares of tiles it sends to each precision."""
-    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, route_tiles
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, route_tiles, q_fusable
     B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS["c5"]
     q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 21)
     out = torch.empty((B, Hq, N, D), dtype=torch.bfloat16, device=device)
@@ -217,14 +217,17 @@ def secondary_c5(device):
     res = {"workload": desc, "steps": iters}
     for mode in ("diag", "routed"):
         routed = mode == "routed"
-        ops = prepare_operands(q, k, v, tile, mode)
+        # as the public entry point does: Q stays unquantized where the attention kernel quantizes it itself (the router
+        # reads Q's scale bytes, so a routed step quantizes Q beforehand)
+        fuse = not routed and q_fusable(q, k, tile, mode, False)
+        ops = prepare_operands(q, k, v, tile, mode, fuse_q=fuse)
         route = route_tiles(ops, False, ROUTE_THRESH_DEFAULT, None) if routed else None
         attention_from_operands(ops, out, False, route=route)
         torch.cuda.synchronize()
         attn_ms = time_events(lambda: attention_from_operands(ops, out, False, route=route), iters)
 
         def step():
-            o = prepare_operands(q, k, v, tile, mode, reuse=ops)
+            o = prepare_operands(q, k, v, tile, mode, reuse=ops, fuse_q=fuse)
             r = route_tiles(o, False, ROUTE_THRESH_DEFAULT, None) if routed else None
             attention_from_operands(o, out, False, route=r)
 
