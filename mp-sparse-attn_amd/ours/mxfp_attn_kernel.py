@@ -19,8 +19,8 @@ _MODES = {"mxfp4": _lib.MODE_MXFP4, "mxfp8": _lib.MODE_MXFP8, "mxfp8e5": _lib.MO
 
 def q_fusable(q, k, tile, block_scale_type, is_causal):
     """True when the attention kernel can take this Q unquantized and quantize it itself (``mpsa_attn_fwd_q16``: the
-    paired-tile kernel's shapes -- D = 128, tile = 128, whole pairs of tiles, diag / mxfp4 types; causal over full tiles, or
-    unmasked from six tiles on)."""
+    paired-tile kernel's shapes -- D = 128, tile = 128, diag / mxfp4 types; causal from two tiles on, unmasked from six
+    tiles on, any length)."""
     mode = _MODES.get(block_scale_type)
     if mode not in (_lib.MODE_DIAG, _lib.MODE_MXFP4) or q.shape[2] != k.shape[2]:
         return False

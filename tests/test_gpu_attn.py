@@ -50,7 +50,7 @@ def test_c1_cpu_plumbing_config(mode):
 
 
 @pytest.mark.parametrize("N", [512, 384])      # 4 and 3 tiles of 128: causal D=128/tile=128 runs the paired-tile
-@pytest.mark.parametrize("D,tile", [(128, 128), (64, 128), (128, 64), (64, 64)])   # kernel for 512, the general one for 384
+@pytest.mark.parametrize("D,tile", [(128, 128), (64, 128), (128, 64), (64, 64)])   # kernel, everything else the general one
 @pytest.mark.parametrize("causal", [True, False])
 def test_all_kernel_variants_gqa(D, tile, causal, N):
     q, k, v = make_qkv(2, 4, 2, N, D, seed=10 + D + tile)
@@ -74,13 +74,14 @@ def _rising_qkv(N, D, step, seed, spike_tile=None, tile=128):
 
 
 @pytest.mark.parametrize("pv", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("causal,N,tile", [(True, 1024, 128), (True, 1536, 128), (False, 1024, 128), (True, 640, 128), (True, 512, 64)])
+@pytest.mark.parametrize("causal,N,tile", [(True, 1024, 128), (True, 1536, 128), (False, 1024, 128), (True, 640, 128), (True, 512, 64), (False, 512, 128)])
 @pytest.mark.parametrize("shape", ["ramp", "spike"])
 def test_running_maximum_moves(shape, causal, N, tile, pv):
     """Scores that rise by far more than the lazy maximum's threshold from one key tile to the next (bf16: 60, fp16: 12,
     in log2 units), and a single tile towering over the rest: the running maximum has to move, in the paired-tile
-    kernel (causal, whole tile pairs), which takes the exponentials first and repeats a tile whose row sum shows that
-    the maximum must move, and in the general kernel."""
+    kernel (the 128-key tiles from N = 640 on; with and without the mask, an odd tile count among them), which takes the
+    exponentials first and repeats a tile whose row sum shows that the maximum must move, and in the general kernel (64-key
+    tiles; four tiles without the mask)."""
     D = 128
     if shape == "ramp":
         q, k, v = _rising_qkv(N, D, step=5.0, seed=N + tile, tile=tile)          # ~80 log2 units per tile
