@@ -447,7 +447,7 @@ def main():
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default: 500; 100 for c5, 30 for c4)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default: a tenth of --steps)")
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
-    ap.add_argument("--mode", default="diag", choices=["diag", "mxfp4", "mxfp8", "routed"],
+    ap.add_argument("--mode", default="diag", choices=["diag", "mxfp4", "mxfp8", "mixed", "routed"],
                     help="per-tile precision: diag (the headline configuration), one precision everywhere, or routed "
                          "(tile router on the scale bytes, thresholds below)")
     ap.add_argument("--route-thresh", type=float, default=ROUTE_THRESH_DEFAULT, help="routed: 8-bit at or above this share of the row's largest tile statistic")
@@ -573,7 +573,7 @@ def main():
     nt = (N + tile - 1) // tile
     comp = composite_peak_tflops(nt, causal)
     traffic, traffic_commit = measured_traffic(args.workload, args.mode)
-    paired = D == 128 and tile == 128 and nt >= (2 if causal else 6) and args.mode in ("diag", "mxfp4")
+    paired = D == 128 and tile == 128 and nt >= (2 if causal else 6) and args.mode in ("diag", "mxfp4", "mixed")
     roofline = {
         "bound": "mfma", "kernel": ("attn_pp_kernel" if paired else "attn_fwd_kernel") + " (fused attention)", "achieved": round(achieved, 2), "peak": PEAK_FP4_TFLOPS,
         "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP4_TFLOPS, 5),

@@ -167,6 +167,7 @@ extern "C" int mpsa_attn_fwd_q16(const void* q, const int64_t q_strides[4], int 
 
 extern "C" int mpsa_attn_fwd_q16_supported(int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode) {
     if (B <= 0 || Hq <= 0 || Hkv <= 0 || n <= 0 || Hq % Hkv || B * Hq * (n / 256 + 1) >= (int64_t(1) << 31)) return 0;
+    if (mode != MPSA_MODE_DIAG && mode != MPSA_MODE_MXFP4) return 0;
     AttnArgs a = {};
     a.B = (int)B; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.n = (int)n; a.d = (int)D; a.tile = tile; a.causal = causal ? 1 : 0; a.mode = mode;
     a.nt = (int)((n + tile - 1) / (tile > 0 ? tile : 1)); a.n_pad = a.nt * tile;

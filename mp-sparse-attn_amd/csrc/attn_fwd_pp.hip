@@ -329,7 +329,8 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             for (int s = 0; s < SST; ++s) {
                 const v4i x = kf4[kb][s];
                 const v8i k8v = (v8i){x[0], x[1], x[2], x[3], 0, 0, 0, 0};
-                st[kb] = score_mfma4(k8v, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
+                if constexpr (MODE == MPSA_MODE_MIXED) st[kb] = score_mfma48<FMT8>(k8v, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
+                else st[kb] = score_mfma4(k8v, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
             }
     };
     auto s_special = [&](int t) __attribute__((always_inline)) {
@@ -592,7 +593,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             load_q_raw(std::false_type{}, q8f);
         }
     } else {
-        load_q(false);
+        load_q(MODE == MPSA_MODE_MIXED);          // "mixed": 8-bit Q fragments for the whole run, against 4-bit K tiles
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
@@ -752,15 +753,20 @@ int launch_pp(const AttnArgs& a, hipStream_t st) {
 template <int PVT, bool QRAW>
 int launch_pp_mode(const AttnArgs& a, hipStream_t st) {
     if (a.mode == MPSA_MODE_MXFP4) return launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP4, QRAW>(a, st);
+    if constexpr (!QRAW) {
+        if (a.mode == MPSA_MODE_MIXED)
+            return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_MIXED, false>(a, st)
+                                           : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MIXED, false>(a, st);
+    }
     return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_DIAG, QRAW>(a, st)
                                    : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_DIAG, QRAW>(a, st);
 }
 
 }  // namespace
 
-// The paired-tile kernel covers self-attention with D = 128 and 128-key tiles: causal runs from two tiles on, runs without
-// the mask from six tiles on; the last tile may be ragged, and with an odd number of tiles the last workgroup of a head
-// works on its one tile with half of its waves.
+// The paired-tile kernel covers self-attention with D = 128 and 128-key tiles in the diag, mxfp4 and mixed modes: causal
+// runs from two tiles on, runs without the mask from six tiles on; the last tile may be ragged, and with an odd number of
+// tiles the last workgroup of a head works on its one tile with half of its waves.
 // MPSA_ATTN_PP=0 in the environment switches it off (the general kernel then runs everything).
 bool attn_pp_supported(const AttnArgs& a, int pv_dtype) {
     static const bool enabled = [] {
@@ -768,7 +774,8 @@ bool attn_pp_supported(const AttnArgs& a, int pv_dtype) {
         return !(v && v[0] == '0');
     }();
     (void)pv_dtype;
-    if (!enabled || a.d != 128 || a.tile != 128 || a.nq != a.n || (a.mode != MPSA_MODE_DIAG && a.mode != MPSA_MODE_MXFP4)) return false;
+    const bool mode_ok = a.mode == MPSA_MODE_DIAG || a.mode == MPSA_MODE_MXFP4 || (a.mode == MPSA_MODE_MIXED && !a.q_raw);
+    if (!enabled || a.d != 128 || a.tile != 128 || a.nq != a.n || !mode_ok) return false;
     return a.nt >= (a.causal ? 2 : 6);
 }
 

@@ -448,7 +448,8 @@ def test_error_behaviour():
 
 
 @pytest.mark.parametrize("fmt8", ["mixed", "mixed_e5"])
-@pytest.mark.parametrize("causal,N,D,tile", [(True, 512, 128, 128), (False, 300, 128, 128), (True, 384, 64, 64), (False, 256, 64, 128)])
+@pytest.mark.parametrize("causal,N,D,tile", [(True, 512, 128, 128), (False, 300, 128, 128), (True, 384, 64, 64), (False, 256, 64, 128),
+                                             (True, 1100, 128, 128), (False, 1100, 128, 128), (False, 1024, 128, 128)])   # the last three and the first: the paired-tile kernel
 def test_mixed_mode_8bit_q_against_4bit_k(fmt8, causal, N, D, tile):
     """The reference's "mixed" type (ours/mxfp_attn_kernel.py:264-269 with ELEM_PER_BYTE_A = 1, ELEM_PER_BYTE_B = 2):
     every tile multiplies 8-bit Q codes with 4-bit K codes."""
