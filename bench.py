@@ -573,7 +573,7 @@ def main():
     nt = (N + tile - 1) // tile
     comp = composite_peak_tflops(nt, causal)
     traffic, traffic_commit = measured_traffic(args.workload, args.mode)
-    paired = D == 128 and tile == 128 and nt >= (2 if causal else 6) and args.mode in ("diag", "mxfp4", "mixed")
+    paired = D == 128 and tile == 128 and nt >= (2 if causal else 6) and args.mode in ("diag", "mxfp4", "mxfp8", "mixed")
     roofline = {
         "bound": "mfma", "kernel": ("attn_pp_kernel" if paired else "attn_fwd_kernel") + " (fused attention)", "achieved": round(achieved, 2), "peak": PEAK_FP4_TFLOPS,
         "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP4_TFLOPS, 5),

@@ -116,6 +116,6 @@ int attn_skip_launch(const AttnArgs& a, int pv_dtype, hipStream_t st);
 // Routed variants of the general kernel (per-tile precision from a visiting list): attn_fwd_routed.hip
 int attn_routed_launch(const AttnArgs& a, int pv_dtype, hipStream_t st);
 
-// Paired-tile ("ping-pong") kernel for self-attention with D = 128, tile = 128 in the diag / mxfp4 / mixed modes: attn_fwd_pp.hip
+// Paired-tile ("ping-pong") kernel for self-attention with D = 128, tile = 128 in the diag / mxfp4 / mixed / mxfp8 modes: attn_fwd_pp.hip
 bool attn_pp_supported(const AttnArgs& a, int pv_dtype);
 int attn_pp_launch(const AttnArgs& a, int pv_dtype, hipStream_t st);       // a.q_raw != nullptr: the fused-quantizer variants

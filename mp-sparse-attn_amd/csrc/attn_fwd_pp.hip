@@ -25,7 +25,8 @@
 // direct-to-LDS loads, one barrier per key tile; K has three buffers (the tile whose fragments are being pulled into
 // registers is two steps ahead of the P.V tile), V two; the two 8-bit (diagonal) K tiles of a "diag" run's pair are staged
 // once, in the prologue, into an LDS area of their own (read straight from global memory at the diagonal step their
-// latency sat on the wave's critical path).  The running maximum rides in the score MFMA's C operand.
+// latency sat on the wave's critical path).  The running maximum rides in the score MFMA's C operand.  The "mixed" mode
+// (8-bit Q, 4-bit K) differs in the score instruction's operand formats only; the "mxfp8" mode's K ring holds 8-bit tiles.
 #include "attn_common.h"
 #include "quantize_kernel.h"
 
@@ -44,6 +45,7 @@ constexpr int K8_BYTES = TILE * ROW8;           // "diag" runs: the two 8-bit di
 constexpr int CPR8 = ROW8 / 16;
 constexpr int Q4_BYTES = 256 * 32;              // fused-quantizer "diag" runs without the causal mask: Y's 4-bit Q fragments, parked while the 8-bit ones are in use
 constexpr int smem_bytes(bool qraw, int mode, bool causal) {
+    if (mode == MPSA_MODE_MXFP8) return NKBUF * K8_BYTES + 2 * V_BYTES;      // every K tile in 8 bits: a ring of 16 KB tiles
     return (qraw ? SMEM_QRAW : SMEM) + (mode == MPSA_MODE_DIAG ? 2 * K8_BYTES : 0) + (qraw && mode == MPSA_MODE_DIAG && !causal ? Q4_BYTES : 0);
 }
 static_assert(smem_bytes(true, MPSA_MODE_DIAG, false) <= 160 * 1024, "LDS of a CU");
@@ -114,8 +116,12 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     const int q_local = 32 * wq + r;
     const int64_t q_row = qhead_row + (int64_t)i * TILE + q_local;
 
+    // MODE_MXFP8: every K tile is an 8-bit one (16 KB, 128-byte rows swizzled like the staged diagonal tiles); the fragment
+    // registers hold two of a tile's four key blocks at a time (the 4-bit tiles': all four)
+    constexpr bool K8ALL = MODE == MPSA_MODE_MXFP8;
+    constexpr int KT_BYTES = K8ALL ? K8_BYTES : K_BYTES;
     uint8_t* const kbuf0 = smem;
-    uint8_t* const vbuf0 = smem + NKBUF * K_BYTES;
+    uint8_t* const vbuf0 = smem + NKBUF * KT_BYTES;
     uint8_t* const k8d0 = smem + (QRAW ? SMEM_QRAW : SMEM);     // the pair's two 8-bit diagonal K tiles: tile 2I+1, tile 2I
 
     // ---- operands in registers ----
@@ -229,7 +235,26 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         for (int kb = 0; kb < KB; ++kb)
             ksc[kb] = (int)(*reinterpret_cast<const uint32_t*>(sp + kb * 32 * (D / 32)) >> (8 * h));
     };
+    // 8-bit tiles: fragment (key block kb0 + kbl, step s) = registers kf4[2 kbl][s] (bytes of MX block 2s) and kf4[2 kbl + 1][s]
+    // (of block 2s + 1)
+    auto read_kf8_pair = [&](int t, int kb0) __attribute__((always_inline)) {
+        const uint8_t* kl = kbuf0 + (t % NKBUF) * K8_BYTES;
+#pragma unroll
+        for (int kbl = 0; kbl < 2; ++kbl) {
+            const int krow = 32 * (kb0 + kbl) + r;
+            const int f = (krow >> 1) & (CPR8 - 1);
+#pragma unroll
+            for (int s = 0; s < SST; ++s) {
+                kf4[2 * kbl][s] = *reinterpret_cast<const v4i*>(kl + krow * ROW8 + (((4 * s + h) ^ f) * 16));
+                kf4[2 * kbl + 1][s] = *reinterpret_cast<const v4i*>(kl + krow * ROW8 + (((4 * s + h + 2) ^ f) * 16));
+            }
+        }
+    };
     auto read_kf4 = [&](int t) __attribute__((always_inline)) {
+        if constexpr (K8ALL) {
+            read_kf8_pair(t, 0);
+            return;
+        }
         const uint8_t* kl = kbuf0 + (t % NKBUF) * K_BYTES;
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
@@ -249,9 +274,22 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         const int cb = slot ^ ((row >> SH4) & (CPR4 - 1));
         koff = (uint32_t)(row * ROW4 + cb * 16);
     }
-    auto issue_k4 = [&](int t) __attribute__((always_inline)) {
-        const uint8_t* src = a.k4 + (khead_row + (int64_t)tile_at(t) * TILE) * ROW4;
-        load16_to_lds_sv(koff, src, kbuf0 + (t % NKBUF) * K_BYTES + wu * 1024);
+    uint32_t koff8[2];                                    // the same for an 8-bit tile's two pieces per wave
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const int p = (w * 2 + c) * 64 + lane;
+        const int row = p / CPR8, slot = p % CPR8;
+        koff8[c] = (uint32_t)(row * ROW8 + (slot ^ ((row >> 1) & (CPR8 - 1))) * 16);
+    }
+    auto issue_k4 = [&](int t) __attribute__((always_inline)) {           // step t's K tile, in the width the mode multiplies
+        if constexpr (K8ALL) {
+            const uint8_t* src = a.k8 + (khead_row + (int64_t)tile_at(t) * TILE) * ROW8;
+#pragma unroll
+            for (int c = 0; c < 2; ++c) load16_to_lds_sv(koff8[c], src, kbuf0 + (t % NKBUF) * K8_BYTES + (wu * 2 + c) * 1024);
+        } else {
+            const uint8_t* src = a.k4 + (khead_row + (int64_t)tile_at(t) * TILE) * ROW4;
+            load16_to_lds_sv(koff, src, kbuf0 + (t % NKBUF) * K_BYTES + wu * 1024);
+        }
     };
     auto issue_v = [&](int t) __attribute__((always_inline)) {
         const uint8_t* src = static_cast<const uint8_t*>(a.v) + (khead_row + (int64_t)tile_at(t) * TILE) * (D * 2);
@@ -287,8 +325,8 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     v16f st[KB];
     v4i pk[KB][2];
 
-    auto prep_plain = [&](int t) __attribute__((always_inline)) {       // step t's tile in 4 bits
-        load_kscales(tile_at(t), false);
+    auto prep_plain = [&](int t) __attribute__((always_inline)) {       // step t's tile in the mode's plain width
+        load_kscales(tile_at(t), K8ALL);
         read_kf4(t);
     };
     auto prep_special = [&](int t) __attribute__((always_inline)) {      // this wave's diagonal tile (key tile i) at step t
@@ -322,7 +360,26 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             load_q(false);
         }
     };
-    auto s_plain = [&]() __attribute__((always_inline)) {
+    auto s_plain = [&](int ts) __attribute__((always_inline)) {          // scores of step ts's tile
+        if constexpr (K8ALL) {
+            // key blocks 0, 1 are in the fragment registers; blocks 2, 3 follow into the same registers while the first
+            // four matrix instructions run
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                for (int kbl = 0; kbl < 2; ++kbl) {
+                    const int kb = 2 * half + kbl;
+#pragma unroll
+                    for (int s = 0; s < SST; ++s) {
+                        const v4i x0 = kf4[2 * kbl][s], x1 = kf4[2 * kbl + 1][s];
+                        const v8i kd = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+                        st[kb] = score_mfma8<FMT8>(kd, qf[s], s == 0 ? negm : st[kb], s, ksc[kb], qsc);
+                    }
+                }
+                if (half == 0) read_kf8_pair(ts, 2);
+            }
+            return;
+        }
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -352,7 +409,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                 }
             }
         } else {
-            s_plain();
+            s_plain(t);
         }
     };
     // masked: keys from `limit` on are dead (the causal diagonal tile: the keys after the query; the ragged last tile:
@@ -446,7 +503,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
         float tot = ps0 + ps1;
         if (__any(!(tot < P::OPTIMISTIC_LIMIT))) {
             prep_plain(t + 1);
-            s_plain();
+            s_plain(t + 1);
             float mx = st[0][0];
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb)
@@ -500,11 +557,17 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             acc[d] = P::mfma(cur, __builtin_bit_cast(typename P::vec, pk[kc >> 1][kc & 1]), acc[d]);
         };
         float ps0 = 0.0f, ps1 = 0.0f;
-        const uint8_t* kl = kbuf0 + ((t + 2) % NKBUF) * K_BYTES;
+        const uint8_t* kl = kbuf0 + ((t + 2) % NKBUF) * KT_BYTES;
         auto kfrag = [&](int kb, int s) __attribute__((always_inline)) {
-            const int krow = 32 * kb + r;
-            const int f = (krow >> SH4) & (CPR4 - 1);
-            kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * ROW4 + (((2 * s + h) ^ f) * 16));
+            if constexpr (K8ALL) {                       // register kf4[kb][s] of the 8-bit layout: key block kb / 2, half kb % 2
+                const int krow = 32 * (kb >> 1) + r;
+                const int f = (krow >> 1) & (CPR8 - 1);
+                kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * ROW8 + (((4 * s + h + 2 * (kb & 1)) ^ f) * 16));
+            } else {
+                const int krow = 32 * kb + r;
+                const int f = (krow >> SH4) & (CPR4 - 1);
+                kf4[kb][s] = *reinterpret_cast<const v4i*>(kl + krow * ROW4 + (((2 * s + h) ^ f) * 16));
+            }
         };
         // score pair e = 4 g + j: registers 8c + 2j, 8c + 2j + 1 of key block kb, with g = 2 kb + c the 16-key group
         auto do_exp = [&](int e) __attribute__((always_inline)) {
@@ -593,7 +656,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             load_q_raw(std::false_type{}, q8f);
         }
     } else {
-        load_q(MODE == MPSA_MODE_MIXED);          // "mixed": 8-bit Q fragments for the whole run, against 4-bit K tiles
+        load_q(MODE == MPSA_MODE_MIXED || K8ALL);  // "mixed" and "mxfp8": 8-bit Q fragments for the whole run
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
@@ -615,20 +678,20 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             softmax(true, std::true_type{}, q_local + 1);
         } else {
             prep_plain(0);
-            s_plain();
+            s_plain(0);
             softmax(true, std::false_type{}, 0);
             if (last >= 2) prep_plain(1);
         }
     } else {
         prep_plain(0);
-        s_plain();
+        s_plain(0);
         softmax(true, std::false_type{}, 0);
         if (last >= 2) prep_plain(1);
     }
     for (int t = 0; t + 2 <= last; ++t) {
         sync_issue(t);
-        s_plain();
-        load_kscales(tile_at(t + 2), false);
+        s_plain(t + 1);
+        load_kscales(tile_at(t + 2), K8ALL);
         pv_exp(t);
     }
     if constexpr (CAUSAL) {
@@ -661,7 +724,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             }
             pv(t);
             if (is8) s_special(t + 1);
-            else s_plain();
+            else s_plain(t + 1);
             softmax(false, std::true_type{}, limit);
         }
         sync_issue(nsteps - 1);
@@ -757,6 +820,9 @@ int launch_pp_mode(const AttnArgs& a, hipStream_t st) {
         if (a.mode == MPSA_MODE_MIXED)
             return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_MIXED, false>(a, st)
                                            : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MIXED, false>(a, st);
+        if (a.mode == MPSA_MODE_MXFP8)
+            return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_MXFP8, false>(a, st)
+                                           : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP8, false>(a, st);
     }
     return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_DIAG, QRAW>(a, st)
                                    : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_DIAG, QRAW>(a, st);
@@ -764,7 +830,7 @@ int launch_pp_mode(const AttnArgs& a, hipStream_t st) {
 
 }  // namespace
 
-// The paired-tile kernel covers self-attention with D = 128 and 128-key tiles in the diag, mxfp4 and mixed modes: causal
+// The paired-tile kernel covers self-attention with D = 128 and 128-key tiles in the diag, mxfp4, mixed and mxfp8 modes: causal
 // runs from two tiles on, runs without the mask from six tiles on; the last tile may be ragged, and with an odd number of
 // tiles the last workgroup of a head works on its one tile with half of its waves.
 // MPSA_ATTN_PP=0 in the environment switches it off (the general kernel then runs everything).
@@ -774,7 +840,7 @@ bool attn_pp_supported(const AttnArgs& a, int pv_dtype) {
         return !(v && v[0] == '0');
     }();
     (void)pv_dtype;
-    const bool mode_ok = a.mode == MPSA_MODE_DIAG || a.mode == MPSA_MODE_MXFP4 || (a.mode == MPSA_MODE_MIXED && !a.q_raw);
+    const bool mode_ok = a.mode == MPSA_MODE_DIAG || a.mode == MPSA_MODE_MXFP4 || ((a.mode == MPSA_MODE_MIXED || a.mode == MPSA_MODE_MXFP8) && !a.q_raw);
     if (!enabled || a.d != 128 || a.tile != 128 || a.nq != a.n || !mode_ok) return false;
     return a.nt >= (a.causal ? 2 : 6);
 }

@@ -652,6 +652,19 @@ def test_outlier_channels_on_rows_with_large_gains_and_the_8bit_matrix_instructi
     assert 2e-2 < err < 4e-2 and (got - modelled).abs().max().item() < 5e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("bst", ["mxfp8", "mxfp8e5"])
+@pytest.mark.parametrize("causal,N", [(True, 384), (True, 1100), (True, 2048), (False, 768), (False, 1100), (False, 1665)])
+def test_paired_tile_kernel_with_every_tile_in_8_bits(bst, causal, N, dtype):
+    """The reference's "mxfp8" type on the paired-tile kernel: the K ring holds 8-bit tiles, the fragment registers two of a
+    tile's four key blocks at a time (the other two are read while the first score instructions run).  Whole and ragged
+    lengths, odd tile counts, grouped heads, against the oracle at the float32 bar; the 16-bit output as its rounding."""
+    q, k, v = make_qkv(2, 4, 2, N, 128, seed=2500 + N, dtype=dtype)
+    fmt8 = O.FMT_E5M2 if bst.endswith("e5") else O.FMT_E4M3
+    want = O.attn_mx(q, k, v, tile=128, causal=causal, mode="mxfp8", fmt8=fmt8, out_dtype=torch.float32)
+    _check(q, k, v, want, f"paired, {bst} causal={causal} N={N} {dtype}", out16=dtype, is_causal=causal, block_scale_type=bst, tile=128)
+
+
 @pytest.mark.parametrize("bst", ["mxfp4", "mxfp8", "diag", "mixed_e5"])
 def test_public_entry_point_with_the_reference_self_check(bst):
     """mxfp_attn(..., compute_reference=True) (ours/mxfp_attn.py:52-69): the score product of the quantized operands is
