@@ -275,8 +275,9 @@ int mpsa_attn_fwd(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, cons
  * call for Q of the reference's wrapper (quant_mxfp4 / quant_mxfp8e5 on q, ours/mxfp_attn_kernel.py:43-50,
  * ours/quant_mxint8.py:479-494) and the attention launch (ours/mxfp_attn_kernel.py:66-70) in one; Q's codes and scales
  * never travel through HBM (at the B1 Hq32 N8192 shape that is 52 MB written and read back).  Same bits as
- * mpsa_attn_prepare + mpsa_attn_fwd.  Built for the paired-tile kernel's shapes only: D = 128, tile = 128, mode
- * MPSA_MODE_DIAG or MPSA_MODE_MXFP4; causal with at least two key tiles (n >= 129), or unmasked with at least six
+ * mpsa_attn_prepare + mpsa_attn_fwd.  Built for the paired-tile kernel's shapes only: D = 128, tile = 128, any mode but
+ * MPSA_MODE_ROUTED (MPSA_MODE_MIXED and MPSA_MODE_MXFP8 quantize Q to 8 bits only, MPSA_MODE_MXFP4 to 4 bits only, and
+ * the K operands a mode does not multiply may be NULL); causal with at least two key tiles (n >= 129), or unmasked with at least six
  * (n >= 641); n need not be a multiple of the tile -- mpsa_attn_fwd_q16_supported() says whether a shape qualifies (1)
  * or not (0); other shapes return MPSA_EUNSUPPORTED and go through mpsa_attn_prepare + mpsa_attn_fwd.
  *   q            [B,Hq,n,D] of q_dtype == pv_dtype (MPSA_BF16 | MPSA_F16), element strides q_strides[4], last dim

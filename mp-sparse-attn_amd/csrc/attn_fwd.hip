@@ -74,8 +74,9 @@ static int attn_entry(const RawQ* rq, const uint8_t* q4, const uint8_t* qs4, con
         if (rq->dtype != pv_dtype) return mpsa_fail(MPSA_EINVAL, "attn: unquantized q must have the P.V dtype (the dtype of v)");
         if (rq->strides[3] != 1 || !mpsa_aligned16(rq->q) || (rq->strides[0] % 8) || (rq->strides[1] % 8) || (rq->strides[2] % 8))
             return mpsa_fail(MPSA_EALIGN, "attn: q rows must be contiguous and 16-byte aligned");
-        if (mode != MPSA_MODE_DIAG && mode != MPSA_MODE_MXFP4) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: unquantized q is taken in the diag and mxfp4 modes only");
-        if ((need4 && (!k4 || !ks4)) || (need8 && (!k8 || !ks8))) return mpsa_fail(MPSA_EINVAL, "attn: K operands missing");
+        if (mode == MPSA_MODE_ROUTED) return mpsa_fail(MPSA_EUNSUPPORTED, "attn: unquantized q is not taken in the routed mode (the router reads Q's scale bytes)");
+        const bool k8_read = mode == MPSA_MODE_DIAG || mode == MPSA_MODE_MXFP8;       // the mixed mode multiplies 4-bit K only
+        if ((need4 && (!k4 || !ks4)) || (k8_read && (!k8 || !ks8))) return mpsa_fail(MPSA_EINVAL, "attn: K operands missing");
     } else if (mixed) {
         if (!q8 || !qs8 || !k4 || !ks4) return mpsa_fail(MPSA_EINVAL, "attn: the mixed mode needs 8-bit Q and 4-bit K operands");
     } else {
@@ -167,7 +168,7 @@ extern "C" int mpsa_attn_fwd_q16(const void* q, const int64_t q_strides[4], int 
 
 extern "C" int mpsa_attn_fwd_q16_supported(int64_t B, int64_t Hq, int64_t Hkv, int64_t n, int64_t D, int tile, int causal, int mode) {
     if (B <= 0 || Hq <= 0 || Hkv <= 0 || n <= 0 || Hq % Hkv || B * Hq * (n / 256 + 1) >= (int64_t(1) << 31)) return 0;
-    if (mode != MPSA_MODE_DIAG && mode != MPSA_MODE_MXFP4) return 0;
+    if (mode != MPSA_MODE_DIAG && mode != MPSA_MODE_MXFP4 && mode != MPSA_MODE_MIXED && mode != MPSA_MODE_MXFP8) return 0;
     AttnArgs a = {};
     a.B = (int)B; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.n = (int)n; a.d = (int)D; a.tile = tile; a.causal = causal ? 1 : 0; a.mode = mode;
     a.nt = (int)((n + tile - 1) / (tile > 0 ? tile : 1)); a.n_pad = a.nt * tile;

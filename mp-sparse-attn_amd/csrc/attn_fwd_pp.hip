@@ -46,7 +46,8 @@ constexpr int CPR8 = ROW8 / 16;
 constexpr int Q4_BYTES = 256 * 32;              // fused-quantizer "diag" runs without the causal mask: Y's 4-bit Q fragments, parked while the 8-bit ones are in use
 constexpr int smem_bytes(bool qraw, int mode, bool causal) {
     if (mode == MPSA_MODE_MXFP8) return NKBUF * K8_BYTES + 2 * V_BYTES;      // every K tile in 8 bits: a ring of 16 KB tiles
-    return (qraw ? SMEM_QRAW : SMEM) + (mode == MPSA_MODE_DIAG ? 2 * K8_BYTES : 0) + (qraw && mode == MPSA_MODE_DIAG && !causal ? Q4_BYTES : 0);
+    const bool diag = mode == MPSA_MODE_DIAG;                                 // the parked Q fragments and staged diagonal tiles are a diag run's
+    return (qraw && diag ? SMEM_QRAW : SMEM) + (diag ? 2 * K8_BYTES : 0) + (qraw && diag && !causal ? Q4_BYTES : 0);
 }
 static_assert(smem_bytes(true, MPSA_MODE_DIAG, false) <= 160 * 1024, "LDS of a CU");
 constexpr int NWAVES = 8;
@@ -144,6 +145,7 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
     auto load_q_raw = [&](auto want8_c, v8i (&q8f)[SST]) __attribute__((always_inline)) {
 #pragma clang fp contract(off)        // the quantizer's arithmetic, operation by operation
         constexpr bool WANT8 = decltype(want8_c)::value;
+        constexpr bool WANT4 = MODE != MPSA_MODE_MIXED && MODE != MPSA_MODE_MXFP8;   // those two multiply 8-bit Q everywhere
         // rows beyond the sequence (ragged last tile) read the last row instead and are zeroed below
         const bool row_ok = i * TILE + q_local < a.nq;
         const int64_t row_idx = row_ok ? (int64_t)i * TILE + q_local : (int64_t)a.nq - 1;
@@ -165,12 +167,14 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
             }
             const bool zero = mpsa_f2u(amax) == 0u;
             const int ex = block_exponent(amax);
-            const int se = ex - 3;                                             // emax of E2M1: ours/quant_mxint8.py:303
-            int w[4];
+            if constexpr (WANT4) {
+                const int se = ex - 3;                                         // emax of E2M1: ours/quant_mxint8.py:303
+                int w[4];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) w[c] = zero ? 0 : (int)e2m1_pack8<true>(x[c], se, false);
-            qf[s] = (v8i){w[0], w[1], w[2], w[3], 0, 0, 0, 0};
-            sbytes |= (uint32_t)(zero ? 0 : min(max(se + 127, 0), 254)) << (16 * s);
+                for (int c = 0; c < 4; ++c) w[c] = zero ? 0 : (int)e2m1_pack8<true>(x[c], se, false);
+                qf[s] = (v8i){w[0], w[1], w[2], w[3], 0, 0, 0, 0};
+                sbytes |= (uint32_t)(zero ? 0 : min(max(se + 127, 0), 254)) << (16 * s);
+            }
             if constexpr (WANT8) {
                 const int se8 = ex - 7;                                        // emax of the 8-bit formats: ours/quant_mxint8.py:191
                 // the quantizer's clamp to the format's maximum (quantize_kernel.h): finite blocks scale into
@@ -197,7 +201,13 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                 sbytes8 |= (uint32_t)(zero ? 0 : min(max(se8 + 127, 0), 254)) << (16 * s);
             }
         }
-        qsc = (int)(sbytes | (sbytes8 << 8));
+        if constexpr (WANT4) {
+            qsc = (int)(sbytes | (sbytes8 << 8));
+        } else {
+#pragma unroll
+            for (int s = 0; s < SST; ++s) qf[s] = q8f[s];
+            qsc = (int)sbytes8;
+        }
         if (i * TILE + 32 * wq + 31 >= a.nq) {            // a wave of the ragged last tile: zero codes and scales for its padding
 #pragma unroll                                            // rows, as the standalone quantizer pads them
             for (int s = 0; s < SST; ++s)
@@ -652,6 +662,8 @@ __global__ __launch_bounds__(512, 1) void attn_pp_kernel(AttnArgs a) {
                 *reinterpret_cast<v4i*>(park + (2 * s) * 8192) = (v4i){q8f[s][0], q8f[s][1], q8f[s][2], q8f[s][3]};
                 *reinterpret_cast<v4i*>(park + (2 * s + 1) * 8192) = (v4i){q8f[s][4], q8f[s][5], q8f[s][6], q8f[s][7]};
             }
+        } else if constexpr (MODE == MPSA_MODE_MIXED || K8ALL) {
+            load_q_raw(std::true_type{}, q8f);
         } else {
             load_q_raw(std::false_type{}, q8f);
         }
@@ -816,14 +828,12 @@ int launch_pp(const AttnArgs& a, hipStream_t st) {
 template <int PVT, bool QRAW>
 int launch_pp_mode(const AttnArgs& a, hipStream_t st) {
     if (a.mode == MPSA_MODE_MXFP4) return launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP4, QRAW>(a, st);
-    if constexpr (!QRAW) {
-        if (a.mode == MPSA_MODE_MIXED)
-            return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_MIXED, false>(a, st)
-                                           : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MIXED, false>(a, st);
-        if (a.mode == MPSA_MODE_MXFP8)
-            return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_MXFP8, false>(a, st)
-                                           : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP8, false>(a, st);
-    }
+    if (a.mode == MPSA_MODE_MIXED)
+        return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_MIXED, QRAW>(a, st)
+                                       : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MIXED, QRAW>(a, st);
+    if (a.mode == MPSA_MODE_MXFP8)
+        return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_MXFP8, QRAW>(a, st)
+                                       : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_MXFP8, QRAW>(a, st);
     return a.fmt8 == MPSA_FMT_E5M2 ? launch_pp<PVT, MPSA_FMT_E5M2, MPSA_MODE_DIAG, QRAW>(a, st)
                                    : launch_pp<PVT, MPSA_FMT_E4M3, MPSA_MODE_DIAG, QRAW>(a, st);
 }
@@ -840,7 +850,7 @@ bool attn_pp_supported(const AttnArgs& a, int pv_dtype) {
         return !(v && v[0] == '0');
     }();
     (void)pv_dtype;
-    const bool mode_ok = a.mode == MPSA_MODE_DIAG || a.mode == MPSA_MODE_MXFP4 || ((a.mode == MPSA_MODE_MIXED || a.mode == MPSA_MODE_MXFP8) && !a.q_raw);
+    const bool mode_ok = a.mode == MPSA_MODE_DIAG || a.mode == MPSA_MODE_MXFP4 || a.mode == MPSA_MODE_MIXED || a.mode == MPSA_MODE_MXFP8;
     if (!enabled || a.d != 128 || a.tile != 128 || a.nq != a.n || !mode_ok) return false;
     return a.nt >= (a.causal ? 2 : 6);
 }

@@ -19,10 +19,10 @@ _MODES = {"mxfp4": _lib.MODE_MXFP4, "mxfp8": _lib.MODE_MXFP8, "mxfp8e5": _lib.MO
 
 def q_fusable(q, k, tile, block_scale_type, is_causal):
     """True when the attention kernel can take this Q unquantized and quantize it itself (``mpsa_attn_fwd_q16``: the
-    paired-tile kernel's shapes -- D = 128, tile = 128, diag / mxfp4 types; causal from two tiles on, unmasked from six
-    tiles on, any length)."""
+    paired-tile kernel's shapes -- D = 128, tile = 128, every type but the routed ones; causal from two tiles on, unmasked
+    from six tiles on, any length)."""
     mode = _MODES.get(block_scale_type)
-    if mode not in (_lib.MODE_DIAG, _lib.MODE_MXFP4) or q.shape[2] != k.shape[2]:
+    if mode not in (_lib.MODE_DIAG, _lib.MODE_MXFP4, _lib.MODE_MIXED, _lib.MODE_MXFP8) or q.shape[2] != k.shape[2]:
         return False
     B, Hq, N, D = q.shape
     return bool(_lib.lib().mpsa_attn_fwd_q16_supported(B, Hq, k.shape[1], N, D, tile, 1 if is_causal else 0, mode))

@@ -520,7 +520,7 @@ def test_reference_call_sequence_quantize_package_attend(bst):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("bst", ["diag", "mxfp4", "diag_e5"])
+@pytest.mark.parametrize("bst", ["diag", "mxfp4", "diag_e5", "mixed", "mixed_e5", "mxfp8", "mxfp8e5"])
 @pytest.mark.parametrize("N,scale", [(256, None), (1024, 0.07), (1536, None)])
 def test_q_quantized_inside_the_attention_kernel_gives_the_same_bits(bst, N, scale, dtype):
     """mpsa_attn_fwd_q16 (Q handed over unquantized, MX-quantized in registers by the paired-tile kernel) against
@@ -534,7 +534,7 @@ def test_q_quantized_inside_the_attention_kernel_gives_the_same_bits(bst, N, sca
     kd, vd = k.to(DEV), v.to(DEV)
     assert not qd.is_contiguous() and q_fusable(qd, kd, 128, bst, True)
     assert q_fusable(qd, kd, 128, bst, False) == (N >= 768)       # without the mask: from six tiles on
-    assert not q_fusable(qd, kd, 64, bst, True) and not q_fusable(qd, kd, 128, "mxfp8", True)
+    assert not q_fusable(qd, kd, 64, bst, True) and not q_fusable(qd, kd, 128, "routed", True)
     a = torch.empty((2, 8, N, 128), dtype=dtype, device=DEV)
     b = torch.empty_like(a)
     attention_from_operands(prepare_operands(qd, kd, vd, 128, bst, scale), a, True)
@@ -545,7 +545,7 @@ def test_q_quantized_inside_the_attention_kernel_gives_the_same_bits(bst, N, sca
     # and the public entry point takes the fused route by itself
     c = mxfp_attn_kernel(qd, kd, vd, is_causal=True, scale=scale, block_scale_type=bst, output_dtype=dtype)
     assert torch.equal(a, c)
-    want = O.attn_mx(q, k, v, tile=128, causal=True, mode="diag" if bst.startswith("diag") else "mxfp4", scale=scale,
+    want = O.attn_mx(q, k, v, tile=128, causal=True, mode=bst.replace("_e5", "").replace("8e5", "8"), scale=scale,
                      fmt8=O.FMT_E5M2 if bst.endswith("e5") else O.FMT_E4M3, out_dtype=torch.float32)
     _compare(mxfp_attn_kernel(qd, kd, vd, is_causal=True, scale=scale, block_scale_type=bst, output_dtype=torch.float32), want, f"fused q {bst} N={N}")
 
@@ -721,7 +721,9 @@ def test_q16_entry_point_rejects_other_shapes():
     assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 128, 128, 128, 1, _lib.MODE_DIAG) == 0
     assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192 + 128, 128, 128, 1, _lib.MODE_DIAG) == 1
     assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 64, 128, 1, _lib.MODE_DIAG) == 0
-    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 128, 128, 1, _lib.MODE_MXFP8) == 0
+    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 128, 128, 1, _lib.MODE_MXFP8) == 1
+    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 128, 128, 1, _lib.MODE_MIXED) == 1
+    assert L.mpsa_attn_fwd_q16_supported(1, 32, 8, 8192, 128, 128, 1, _lib.MODE_ROUTED) == 0
     q, k, v = (t.to(DEV) for t in make_qkv(1, 2, 2, 384, 128, seed=9))
     from ours.mxfp_attn_kernel import prepare_operands
     ops = prepare_operands(q, k, v, 128, "diag")
