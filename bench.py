@@ -379,6 +379,39 @@ def router_study(args, device):
                       "reference": "float64 softmax(q k^T * scale) v of the unquantized inputs (torch, on the device)", "cases": table}))
 
 
+def skip_study(args, device):
+    """What the reference's tile skipping costs and buys on a workload (first ``--heads`` heads): the attention time with
+    the rule applied ahead of the attention kernel (mpsa_skip_route + mpsa_attn_fwd_routed) and inside it
+    (mpsa_attn_fwd_skip), next to the kernel without skipping, over thresholds that skip from nothing to nearly everything."""
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, skip_route
+    B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
+    causal = args.workload not in NON_CAUSAL
+    q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21, args.workload not in PLAIN_DRAWS)
+    group = Hq // Hkv
+    hq = max(min(args.heads, Hq) // group * group, group)
+    q, k, v = q[:, :hq].contiguous(), k[:, :hq // group].contiguous(), v[:, :hq // group].contiguous()
+    nt = (N + tile - 1) // tile
+    visited = (nt * (nt + 1) // 2 if causal else nt * nt) * B * hq
+    out = torch.empty((B, hq, N, D), dtype=torch.bfloat16, device=device)
+    table = []
+    for mode in ("mxfp4", "diag", "mxfp8"):
+        ops = prepare_operands(q, k, v, tile, mode)
+        attention_from_operands(ops, out, causal)
+        dense = time_events(lambda: attention_from_operands(ops, out, causal), args.steps)
+        route_ms = time_events(lambda: skip_route(ops, causal, 1.0), args.steps)
+        rows = []
+        for th in (0.0, 0.5, 0.9, 1.0, 1.1, 2.0):
+            skipped = torch.zeros((B, hq, nt), dtype=torch.int32, device=device)
+            attention_from_operands(ops, out, causal, skip_thresh=th, skipped=skipped)
+            share = float(skipped.sum()) / visited
+            ahead = time_events(lambda: attention_from_operands(ops, out, causal, skip_thresh=th, skipped=skipped), args.steps)
+            inside = time_events(lambda: attention_from_operands(ops, out, causal, skip_thresh=th, skipped=skipped, skip_in_kernel=True), args.steps)
+            rows.append({"skip_thresh": th, "skipped_share": round(share, 4), "ahead_ms": round(ahead, 4), "inside_ms": round(inside, 4)})
+        table.append({"mode": mode, "no_skipping_ms": round(dense, 4), "statistics_and_lists_ms": round(route_ms, 4), "thresholds": rows})
+        del ops
+    print(json.dumps({"kernel": "tile-skipping study", "workload": desc, "heads": hq, "cases": table}))
+
+
 def run_only(args, device):
     """Launch one kernel repeatedly (for rocprofv3 --pmc / --kernel-trace runs)."""
     from ours import _lib
@@ -387,6 +420,9 @@ def run_only(args, device):
     from ours.block_scaled_matmul import block_scaled_matmul, make_configs, pack_scale_5d
     if args.only == "router":
         router_study(args, device)
+        return
+    if args.only == "skip":
+        skip_study(args, device)
         return
     if args.only == "mfma":
         print(json.dumps({"kernel": "matrix-instruction stream", "rates": mfma_stream_rates(device, 0.2)}))
@@ -464,7 +500,7 @@ def main():
                     help="--only gemm4|gemm8|attn: the workload's random operands (default) or constant ones (the clock then stays up)")
     ap.add_argument("--linear-scales", action="store_true",
                     help="with --only gemm4/gemm8: row-major [rows, K/32] scales instead of the reference's packed form")
-    ap.add_argument("--only", default=None, choices=["attn", "copy", "quant", "gemm4", "gemm8", "gemm48", "mfma", "router"],
+    ap.add_argument("--only", default=None, choices=["attn", "copy", "quant", "gemm4", "gemm8", "gemm48", "mfma", "router", "skip"],
                     help="profiling aid: launch just this kernel --steps times and exit (copy = 1 GiB torch copy, "
                          "the calibration kernel for HBM counters)")
     args = ap.parse_args()

@@ -337,11 +337,37 @@ int mpsa_route_tiles(const uint8_t* qs4, const uint8_t* ks4, int64_t B, int64_t 
                      uint8_t* cls, int32_t* order, int32_t* counts, mpsa_stream_t stream);
 
 /*
+ * Tile skipping decided ahead of the attention kernel: the reference's rule (ours/mxfp_attn_kernel.py:272-297 -- the
+ * statistic of a score tile is the mean over its query rows of the row maximum of S; key tile 0 is always kept and sets
+ * the reference value, tile j > 0 is kept iff stat(j) >= stat(0) * skip_thresh; the diagonal tile of a causal run is
+ * kept, ours/online_routing.py:68-77) applied to the statistics of ALL tiles, which a score-product-only kernel takes
+ * first, and written out as the visiting lists of mpsa_attn_fwd_routed.  Same decisions as mpsa_attn_fwd_skip (which
+ * applies the rule inside the attention kernel, tile by tile); the attention call that follows visits the kept tiles
+ * only, so that skipped tiles cost a fifth of a tile's matrix work and nothing else.
+ * D = 128, tile = 128, mode MPSA_MODE_MXFP4 | MPSA_MODE_MXFP8 | MPSA_MODE_DIAG, at most MPSA_SKIP_ROUTE_MAX_TILES key
+ * tiles: mpsa_skip_route_supported() says whether a shape qualifies (1) or not (0).
+ *   q4 .. ks8, fmt8   the quantized operands of mpsa_attn_prepare (the sets the mode multiplies)
+ *   work       mpsa_skip_route_workspace(...) bytes of device memory (the statistics, float32 [B,Hq,ntq,ntk]), 4-byte aligned
+ *   cls        out, optional (may be NULL), uint8 [B,Hq,ntq,ntk]: 0 skipped, 1 4-bit, 2 8-bit, 255 not visited
+ *   order, counts   out, as mpsa_route_tiles writes them
+ *   skipped    out, optional, int32 [B,Hq,ntq]: number of skipped key tiles per query tile
+ */
+#define MPSA_SKIP_ROUTE_MAX_TILES 2048
+int mpsa_skip_route_supported(int64_t nq, int64_t nk, int64_t D, int tile, int causal, int mode);
+int64_t mpsa_skip_route_workspace(int64_t B, int64_t Hq, int64_t nq, int64_t nk, int tile);
+int mpsa_skip_route(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
+                    const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,
+                    int64_t B, int64_t Hq, int64_t Hkv, int64_t nq, int64_t nk, int64_t D, int tile, int causal, int mode,
+                    float skip_thresh, void* work, uint8_t* cls, int32_t* order, int32_t* counts, int32_t* skipped,
+                    mpsa_stream_t stream);
+
+/*
  * Fused attention forward over visiting lists (per-tile precision; BLKQ x BLKQ granularity as in mpsa_attn_fwd).
- * Arguments as mpsa_attn_fwd without mode (both operand sets are needed), plus order / counts as written by
- * mpsa_route_tiles -- or by the caller: any list of distinct key tiles works, as long as every tile that needs a mask
- * sits in a masked run.  Key tiles not on a query tile's list contribute nothing; a query tile with an empty list
- * returns zeros.  Out-of-range list entries and run lengths are clamped, never followed.
+ * Arguments as mpsa_attn_fwd without mode, plus order / counts as written by mpsa_route_tiles or mpsa_skip_route -- or
+ * by the caller: any list of distinct key tiles works, as long as every tile that needs a mask sits in a masked run.
+ * Both operand sets are needed unless the lists name tiles of one precision only: then the other set (q and k codes and
+ * scales of that width) may be NULL.  Key tiles not on a query tile's list contribute nothing; a query tile with an
+ * empty list returns zeros.  Out-of-range list entries and run lengths are clamped, never followed.
  */
 int mpsa_attn_fwd_routed(const uint8_t* q4, const uint8_t* qs4, const uint8_t* q8, const uint8_t* qs8,
                          const uint8_t* k4, const uint8_t* ks4, const uint8_t* k8, const uint8_t* ks8, int fmt8,

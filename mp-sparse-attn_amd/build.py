@@ -18,14 +18,14 @@ LIB = os.path.join(LIBDIR, "libmpsa.so")
 BENCH_LIB = os.path.join(LIBDIR, "libmpsa_bench.so")
 BENCH_SOURCES = ["bench/mfma_stream.hip"]
 
-SOURCES = ["api.hip", "formats.hip", "quantize.hip", "v_tiles.hip", "prepare.hip", "gemm_mx.hip", "attn_fwd.hip", "attn_fwd_skip.hip", "attn_fwd_routed.hip", "attn_fwd_pp.hip", "route.hip"]
+SOURCES = ["api.hip", "formats.hip", "quantize.hip", "v_tiles.hip", "prepare.hip", "gemm_mx.hip", "attn_fwd.hip", "attn_fwd_skip.hip", "attn_fwd_routed.hip", "attn_fwd_pp.hip", "route.hip", "skip_route.hip"]
 
 # packed-fp32 instructions are switched off on purpose (the flag is for the device pass; the host
 # pass warns that it does not know the feature, which is harmless)
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 PER_FILE = {"quantize.hip": ["-ffp-contract=off"], "formats.hip": ["-ffp-contract=off"], "prepare.hip": ["-ffp-contract=off"],
-            "route.hip": ["-ffp-contract=off"]}
+            "route.hip": ["-ffp-contract=off"], "skip_route.hip": ["-ffp-contract=off"]}
 
 
 def _hipcc():

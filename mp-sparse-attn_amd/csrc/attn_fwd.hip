@@ -79,12 +79,17 @@ static int attn_entry(const RawQ* rq, const uint8_t* q4, const uint8_t* qs4, con
         if ((need4 && (!k4 || !ks4)) || (k8_read && (!k8 || !ks8))) return mpsa_fail(MPSA_EINVAL, "attn: K operands missing");
     } else if (mixed) {
         if (!q8 || !qs8 || !k4 || !ks4) return mpsa_fail(MPSA_EINVAL, "attn: the mixed mode needs 8-bit Q and 4-bit K operands");
+    } else if (routed) {
+        // lists that name tiles of one precision only need that operand set only (the caller's promise); a set is whole or absent
+        const bool has4 = q4 && qs4 && k4 && ks4, has8 = q8 && qs8 && k8 && ks8;
+        const bool none4 = !q4 && !qs4 && !k4 && !ks4, none8 = !q8 && !qs8 && !k8 && !ks8;
+        if (!(has4 || none4) || !(has8 || none8) || (none4 && none8)) return mpsa_fail(MPSA_EINVAL, "attn: a routed run needs the whole 4-bit operand set, the whole 8-bit one, or both");
     } else {
         if (need4 && (!q4 || !qs4 || !k4 || !ks4)) return mpsa_fail(MPSA_EINVAL, "attn: 4-bit operands missing");
         if (need8 && (!q8 || !qs8 || !k8 || !ks8)) return mpsa_fail(MPSA_EINVAL, "attn: 8-bit operands missing");
     }
     if (!v_tiles || !o || !o_strides) return mpsa_fail(MPSA_EINVAL, "attn: null pointer");
-    if (need8 && fmt8 != MPSA_FMT_E4M3 && fmt8 != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "attn: 8-bit format must be E4M3 or E5M2");
+    if (need8 && (!routed || q8) && fmt8 != MPSA_FMT_E4M3 && fmt8 != MPSA_FMT_E5M2) return mpsa_fail(MPSA_EINVAL, "attn: 8-bit format must be E4M3 or E5M2");
     if (pv_dtype != MPSA_BF16 && pv_dtype != MPSA_F16) return mpsa_fail(MPSA_EINVAL, "attn: pv_dtype must be bf16 or f16");
     if (o_dtype != MPSA_BF16 && o_dtype != MPSA_F16 && o_dtype != MPSA_F32) return mpsa_fail(MPSA_EINVAL, "attn: bad output dtype");
     if (B <= 0 || Hq <= 0 || Hkv <= 0 || n <= 0 || nq <= 0 || Hq % Hkv) return mpsa_fail(MPSA_EINVAL, "attn: bad shape (B=%lld Hq=%lld Hkv=%lld nq=%lld nk=%lld)", (long long)B, (long long)Hq, (long long)Hkv, (long long)nq, (long long)n);

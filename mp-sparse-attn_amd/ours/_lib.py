@@ -55,6 +55,9 @@ SIGNATURES = {
                                   _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _vp, _vp]),
     "mpsa_route_workspace": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64, _int]),
     "mpsa_route_tiles": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _f32, _f32, _vp, _vp, _vp, _vp, _vp]),
+    "mpsa_skip_route_supported": (_int, [_i64, _i64, _i64, _int, _int, _int]),
+    "mpsa_skip_route_workspace": (_i64, [_i64, _i64, _i64, _i64, _int]),
+    "mpsa_skip_route": (_int, [_vp] * 8 + [_int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mpsa_attn_fwd_routed": (_int, [_vp] * 8 + [_int, _vp, _int, _vp, _int, _p64,
                                     _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp, _vp, _vp]),
 }

@@ -102,13 +102,54 @@ def route_tiles(ops, is_causal, route_thresh=None, skip_thresh=None):
     return cls, order, counts
 
 
-def attention_from_operands(ops, out, is_causal, skip_thresh=None, skipped=None, route=None):
+def skip_route(ops, is_causal, skip_thresh, skipped=None, want_cls=False):
+    """The reference's tile-skipping rule decided ahead of the attention kernel (``mpsa_skip_route``): a score-product-only
+    pass takes every tile's statistic, the rule turns them into the visiting lists ``mpsa_attn_fwd_routed`` walks.  Returns
+    ``(cls or None, order, counts)``; ``skipped`` (int32 ``[B,Hq,ntq]``) receives the number of skipped key tiles per query
+    tile.  Only where :func:`skip_routable` says so."""
+    B, Hq, Hkv, Nq, N, D = ops["shape"]
+    tile = ops["tile"]
+    dev = ops["v_tiles"].device
+    ntq, ntk = (Nq + tile - 1) // tile, (N + tile - 1) // tile
+    with torch.cuda.device(dev):
+        work = torch.empty(_lib.lib().mpsa_skip_route_workspace(B, Hq, Nq, N, tile), dtype=torch.uint8, device=dev)
+        cls = torch.empty((B, Hq, ntq, ntk), dtype=torch.uint8, device=dev) if want_cls else None
+        order = torch.empty((B, Hq, ntq, ntk), dtype=torch.int32, device=dev)
+        counts = torch.empty((B, Hq, ntq, 4), dtype=torch.int32, device=dev)
+        _lib.check(_lib.lib().mpsa_skip_route(
+            _lib.ptr(ops["q4"]), _lib.ptr(ops["qs4"]), _lib.ptr(ops["q8"]), _lib.ptr(ops["qs8"]),
+            _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]), _lib.ptr(ops["ks8"]), ops["fmt8"],
+            B, Hq, Hkv, Nq, N, D, tile, 1 if is_causal else 0, ops["mode"], float(skip_thresh),
+            _lib.ptr(work), _lib.ptr(cls), _lib.ptr(order), _lib.ptr(counts), _lib.ptr(skipped), _lib.stream_ptr(dev)))
+    return cls, order, counts
+
+
+def skip_routable(ops, is_causal):
+    """True when tile skipping can be decided ahead of the attention kernel for these operands (D = 128, tile = 128, the
+    mxfp4 / mxfp8 / diag types, quantized Q)."""
+    B, Hq, Hkv, Nq, N, D = ops["shape"]
+    return ops.get("q_raw") is None and bool(_lib.lib().mpsa_skip_route_supported(Nq, N, D, ops["tile"], 1 if is_causal else 0, ops["mode"]))
+
+
+def attention_from_operands(ops, out, is_causal, skip_thresh=None, skipped=None, route=None, skip_in_kernel=False):
     """Launch ``mpsa_attn_fwd`` on prepared operands; ``out`` is a ``[B,Hq,Nq,D]`` view (last dim contiguous).
-    With ``skip_thresh`` the tile-skipping entry point runs instead (``skipped``: optional int32 ``[B,Hq,nt]``
-    that receives the number of skipped key tiles per query tile).  Routed operands take ``route`` = the
+    With ``skip_thresh`` the reference's tile skipping runs (``skipped``: optional int32 ``[B,Hq,nt]`` that receives the
+    number of skipped key tiles per query tile): decided ahead of the attention kernel where :func:`skip_routable` says so
+    (the attention kernel then visits the kept tiles only), inside the attention kernel otherwise or with
+    ``skip_in_kernel`` (``mpsa_attn_fwd_skip``) -- same rule, same decisions.  Routed operands take ``route`` = the
     ``(cls, order, counts)`` of :func:`route_tiles`."""
     B, Hq, Hkv, Nq, N, D = ops["shape"]
     dev = out.device
+    if skip_thresh is not None and not skip_in_kernel and ops["mode"] != _lib.MODE_ROUTED and skip_routable(ops, is_causal):
+        _, order, counts = skip_route(ops, is_causal, skip_thresh, skipped)
+        with torch.cuda.device(dev):
+            _lib.check(_lib.lib().mpsa_attn_fwd_routed(
+                _lib.ptr(ops["q4"]), _lib.ptr(ops["qs4"]), _lib.ptr(ops["q8"]), _lib.ptr(ops["qs8"]),
+                _lib.ptr(ops["k4"]), _lib.ptr(ops["ks4"]), _lib.ptr(ops["k8"]), _lib.ptr(ops["ks8"]), ops["fmt8"],
+                _lib.ptr(ops["v_tiles"]), _lib.dtype_id(ops["v_tiles"].dtype), _lib.ptr(out), _lib.dtype_id(out.dtype),
+                _lib.strides4(out), B, Hq, Hkv, Nq, N, D, ops["tile"], 1 if is_causal else 0,
+                _lib.ptr(order), _lib.ptr(counts), _lib.stream_ptr(dev)))
+        return out
     if ops["mode"] == _lib.MODE_ROUTED:
         if route is None:
             raise ValueError("routed operands need route=(cls, order, counts) from route_tiles()")

@@ -379,6 +379,52 @@ def test_tile_skipping_follows_the_reference_rule(mode, causal, N, D, tile):
         _compare(only0, want0, "skip all but the sink")
 
 
+@pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "mxfp8e5", "diag", "diag_e5"])
+@pytest.mark.parametrize("causal,N", [(True, 1024), (False, 1024), (True, 1100), (False, 1100), (False, 640), (True, 2048)])
+def test_tile_skipping_decided_ahead_of_the_attention_kernel(mode, causal, N):
+    """mpsa_skip_route + mpsa_attn_fwd_routed (every tile's statistic from a score-product-only pass, the rule, visiting lists
+    of the kept tiles) against mpsa_attn_fwd_skip (the rule inside the attention kernel) and against the oracle: the same
+    tiles skipped per query tile, the class map the oracle's decisions imply, and the output at the float32 bar -- whole,
+    and ragged lengths, grouped heads, with and without the mask."""
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, skip_route, skip_routable
+    tile, D, H = 128, 128, 2
+    g = torch.Generator().manual_seed(3 * N + 17)
+    q = torch.randn(1, 2 * H, N, D, generator=g) + 1.0
+    nt = -(-N // tile)
+    k = torch.randn(1, H, N, D, generator=g) + torch.rand(nt, generator=g).repeat_interleave(tile)[:N].view(1, 1, N, 1) * 0.5
+    v = torch.randn(1, H, N, D, generator=g)
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    kw = dict(tile=tile, causal=causal, mode=mode.replace("_e5", "").replace("8e5", "8"), fmt8=O.FMT_E5M2 if mode.endswith("e5") else O.FMT_E4M3)
+    th = _robust_thresh(q, k, v, **kw)
+    want, want_sk = O.attn_mx(q, k, v, skip_thresh=th, return_skipped=True, out_dtype=torch.float32, **kw)
+    ops = prepare_operands(q.to(DEV), k.to(DEV), v.to(DEV), tile, mode)
+    assert skip_routable(ops, causal)
+    ahead = torch.full((1, 2 * H, N, D), float("nan"), dtype=torch.float32, device=DEV)
+    inside = torch.full_like(ahead, float("nan"))
+    sk_a = torch.full((1, 2 * H, nt), -1, dtype=torch.int32, device=DEV)
+    sk_i = torch.full_like(sk_a, -1)
+    attention_from_operands(ops, ahead, causal, th, sk_a)
+    attention_from_operands(ops, inside, causal, th, sk_i, skip_in_kernel=True)
+    assert torch.equal(sk_a.cpu(), want_sk) and torch.equal(sk_i.cpu(), want_sk)
+    _compare(ahead, want, f"skip ahead {mode} causal={causal} N={N} th={th}")
+    _compare(inside, want, f"skip inside {mode} causal={causal} N={N} th={th}")
+    # the class map: skipped tiles 0, kept ones by the mode's precision, tiles above the diagonal of a causal run 255
+    cls, order, counts = skip_route(ops, causal, th, want_cls=True)
+    cls = cls.cpu()
+    visited = torch.ones(nt, nt, dtype=torch.bool).tril() if causal else torch.ones(nt, nt, dtype=torch.bool)
+    assert (cls[0, :, ~visited] == 255).all()
+    assert torch.equal((cls == 0).sum(dim=-1).to(torch.int32), want_sk)
+    kept = (cls == 1) | (cls == 2)
+    assert kept[..., 0].all() and (not causal or kept[0, :, torch.arange(nt), torch.arange(nt)].all())
+    eight = torch.zeros(nt, nt, dtype=torch.bool)
+    if kw["mode"] == "mxfp8":
+        eight[:] = True
+    elif kw["mode"] == "diag":
+        eight = torch.eye(nt, dtype=torch.bool)
+    assert ((cls == 2) == (kept & eight)).all()
+    assert torch.equal(counts.sum(dim=-1).cpu(), kept.sum(dim=-1).to(torch.int32))
+
+
 @pytest.mark.parametrize("mode", ["diag", "mxfp4", "mxfp8e5"])
 @pytest.mark.parametrize("dtype,N,D,tile", [(torch.bfloat16, 1000, 128, 128), (torch.float16, 200, 64, 64)])
 def test_one_launch_preparation_equals_the_separate_calls(mode, dtype, N, D, tile):
