@@ -46,6 +46,11 @@ constexpr int stat_lds_bytes(int mode, int nt) { return NK * ((mode == MPSA_MODE
 // the mxfp8 mode; the one 8-bit tile of a diag run's query tile -- the diagonal one -- is read straight from global
 // memory) and are multiplied with both query tiles.  A tile's scale bytes ride along into LDS: the loop then holds no
 // global load the compiler counts, so that its waits never fall on the tiles in flight.
+// Measured (C5, 8 heads: 1.05 M wave-steps): 138 vector and 16 matrix instructions per wave and step; the matrix pipe is
+// busy 41 % of the kernel's cycles, the vector unit 50 %, and the two hardly overlap -- a wave that streams matrix
+// instructions leaves the SIMD's other wave almost no issue slots, so a step costs its matrix time plus its vector time.
+// Taking one query tile's row maxima in the gaps of the other tile's score instructions (a software pipeline inside the
+// wave) made every variant of this kernel spill (up to 119 registers): the loop body then exists in several forms.
 template <int FMT8, int MODE>
 __global__ __launch_bounds__(256, 2) void skip_stats_kernel(StatArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -61,7 +66,11 @@ __global__ __launch_bounds__(256, 2) void skip_stats_kernel(StatArgs a) {
     const int h = lane >> 5, r = lane & 31;
     // heavy pairs first (causal runs)
     const int npairs = (a.ntq + 1) >> 1;
-    const int64_t row_id = blockIdx.x;
+    // consecutive workgroup ids go to different XCDs: give each XCD a contiguous eighth of the (head-major) list, so that a
+    // head's K tiles stay in one L2
+    const int64_t total = (int64_t)gridDim.x;
+    int64_t row_id = blockIdx.x;
+    if ((total & 7) == 0) row_id = (row_id & 7) * (total >> 3) + (row_id >> 3);
     const int rank = (int)(row_id % npairs);
     const int pair = a.causal ? npairs - 1 - rank : rank;
     const int64_t bh = row_id / npairs;
