@@ -61,6 +61,21 @@ def test_host_side_argument_validation():
     assert L.mpsa_attn_fwd(*args) == -3                                                            # D = 96
     args = [one] * 8 + [0, one, 0, one, 0, so, 1, 4, 2, 128, 256, 128, 128, 1, 0, null]
     assert L.mpsa_attn_fwd(*args) == -1                                                            # causal with nq != nk
+    # tile skipping ahead of the attention kernel: the shapes it takes, the operands a mode multiplies, the lists' memory
+    assert L.mpsa_skip_route_supported(8192, 8192, 128, 128, 1, 2) == 1 and L.mpsa_skip_route_supported(8192, 8192, 64, 128, 1, 2) == 0
+    assert L.mpsa_skip_route_supported(8192, 8192, 128, 128, 1, 4) == 0                            # the mixed type
+    assert L.mpsa_skip_route_supported(300, 77, 128, 128, 0, 0) == 1 and L.mpsa_skip_route_supported(300, 77, 128, 128, 0, 2) == 0
+    assert L.mpsa_skip_route_supported(128 * 2049, 128 * 2049, 128, 128, 1, 0) == 0                # more key tiles than its LDS holds
+    assert L.mpsa_skip_route_workspace(1, 4, 1000, 300, 128) == 4 * 8 * 3 * 4
+    shape = [0, 1, 4, 2, 1024, 1024, 128, 128, 1]
+    assert L.mpsa_skip_route(*([one] * 8 + shape + [4, 1.0, one, null, one, one, null, null])) == -3          # mixed
+    assert L.mpsa_skip_route(*([one, one, null, null] + [one] * 4 + shape + [2, 1.0, one, null, one, one, null, null])) == -1   # diag without 8-bit Q
+    assert L.mpsa_skip_route(*([one] * 8 + shape + [2, float("nan"), one, null, one, one, null, null])) == -1
+    assert L.mpsa_skip_route(*([one] * 8 + shape + [2, 1.0, null, null, one, one, null, null])) == -1           # no workspace
+    assert L.mpsa_skip_route(*([one] * 8 + shape + [2, 1.0, one, null, ctypes.c_void_p(18), one, null, null])) == -2   # order misaligned
+    so2 = (ctypes.c_int64 * 4)(128 * 128, 128 * 128, 128, 1)
+    routed = [one, one, null, one] + [one] * 4 + [0, one, 0, one, 0, so2, 1, 4, 2, 128, 128, 128, 128, 1, one, one, null]
+    assert L.mpsa_attn_fwd_routed(*routed) == -1 and b"whole" in L.mpsa_last_error()               # half an operand set
     assert L.mpsa_e2m1_pack(null, 2, 3, 4, one, null) == -1                                         # null input
     assert L.mpsa_e2m1_pack(null, 0, 3, 4, null, null) == 0                                         # empty is fine
     assert L.mpsa_e2m1_encode(null, 4, one, null) == -1
