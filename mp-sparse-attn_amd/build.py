@@ -24,8 +24,11 @@ SOURCES = ["api.hip", "formats.hip", "quantize.hip", "v_tiles.hip", "prepare.hip
 # pass warns that it does not know the feature, which is harmless)
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# skip_route.hip: without -fno-honor-nans (device pass only: the host side tests its arguments for NaN) every two-input
+# maximum of the row-maximum trees gets an instruction per operand that only quiets signalling NaNs (a fifth of the trees'
+# instructions); scores are never NaN unless a scale byte is
 PER_FILE = {"quantize.hip": ["-ffp-contract=off"], "formats.hip": ["-ffp-contract=off"], "prepare.hip": ["-ffp-contract=off"],
-            "route.hip": ["-ffp-contract=off"], "skip_route.hip": ["-ffp-contract=off"]}
+            "route.hip": ["-ffp-contract=off"], "skip_route.hip": ["-ffp-contract=off", "-Xarch_device", "-fno-honor-nans"]}
 
 
 def _hipcc():

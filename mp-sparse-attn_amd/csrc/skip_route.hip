@@ -9,6 +9,7 @@
 // (a fifth of attention's matrix work, no exponentials, no P.V), one workgroup barrier per key tile; a second, small
 // kernel applies the rule and compacts the kept tiles into the visiting lists of mpsa_attn_fwd_routed, which then walks
 // the kept tiles only.  D = 128, 128-key tiles; modes mxfp4, mxfp8 and diag.
+#include <type_traits>
 #include "attn_common.h"
 
 namespace {
@@ -30,6 +31,13 @@ __device__ __forceinline__ float lane_move(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
 }
 
+__device__ __forceinline__ float max3f(float a, float b, float c) { return __builtin_fmaxf(__builtin_fmaxf(a, b), c); }
+__device__ __forceinline__ float tree_max16(const v16f& v) {
+    const float m0 = max3f(v[0], v[1], v[2]), m1 = max3f(v[3], v[4], v[5]), m2 = max3f(v[6], v[7], v[8]);
+    const float m3 = max3f(v[9], v[10], v[11]), m4 = max3f(v[12], v[13], v[14]);
+    return __builtin_fmaxf(max3f(m0, m1, m2), max3f(m3, m4, v[15]));
+}
+
 struct StatArgs {
     const uint8_t *q4, *qs4, *q8, *qs8, *k4, *ks4, *k8, *ks8;
     float* stats;                          // [B,Hq,ntq,nt]
@@ -38,7 +46,7 @@ struct StatArgs {
 
 constexpr int KS_BYTES = TILE * (D / 32);  // a K tile's scale bytes travel with it
 constexpr int QT = 2;                      // query tiles per workgroup: they share the staged K tiles
-constexpr int stat_lds_bytes(int mode, int nt) { return NK * ((mode == MPSA_MODE_MXFP8 ? K8_BYTES : K4_BYTES) + KS_BYTES) + QT * nt * NW * 4; }
+constexpr int stat_lds_bytes(int mode, int nt) { return NK * ((mode == MPSA_MODE_MXFP8 ? K8_BYTES : K4_BYTES) + KS_BYTES) + QT * nt * NW * 4 + NW * 64 * 4; }
 
 // One workgroup of four waves per (batch, query head, pair of query tiles 2P, 2P+1); wave w owns queries 32w .. 32w+31 of
 // both tiles, a lane pair one query of each (the score instruction's layout, see attn_fwd_kernel.h).  Key tiles in
@@ -46,11 +54,15 @@ constexpr int stat_lds_bytes(int mode, int nt) { return NK * ((mode == MPSA_MODE
 // the mxfp8 mode; the one 8-bit tile of a diag run's query tile -- the diagonal one -- is read straight from global
 // memory) and are multiplied with both query tiles.  A tile's scale bytes ride along into LDS: the loop then holds no
 // global load the compiler counts, so that its waits never fall on the tiles in flight.
-// Measured (C5, 8 heads: 1.05 M wave-steps): 138 vector and 16 matrix instructions per wave and step; the matrix pipe is
-// busy 41 % of the kernel's cycles, the vector unit 50 %, and the two hardly overlap -- a wave that streams matrix
-// instructions leaves the SIMD's other wave almost no issue slots, so a step costs its matrix time plus its vector time.
-// Taking one query tile's row maxima in the gaps of the other tile's score instructions (a software pipeline inside the
-// wave) made every variant of this kernel spill (up to 119 registers): the loop body then exists in several forms.
+// What bounds it (C5, 8 heads: 1.05 M wave-steps, measured): a wave issues in order and a SIMD holds two of them (the two
+// tiles of scores take half the registers), so a step costs what the wave's own instruction stream costs -- the matrix
+// pipe was busy 41 % of the cycles and the vector unit 50 % when the step did one thing after the other, and the two
+// workgroups of a CU did not fill each other's gaps.  Hence, in the steps that need no mask (nearly all): one query
+// tile's row maxima sit between the other tile's score instructions, both tiles' sums are taken by one chain of lane
+// moves, the fetch pointers and ring slots are running values and the wait for a tile is a constant.  That is 150
+// instructions per wave and step instead of 220 and 15 % less time; most of what is left over the 0.23 ms of the matrix
+// instructions is clock: with every operand element the same the pass takes 0.39 ms, with random ones 0.50 (the
+// matrix instructions' power draw, as in the attention kernel).
 template <int FMT8, int MODE>
 __global__ __launch_bounds__(256, 2) void skip_stats_kernel(StatArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -82,6 +94,7 @@ __global__ __launch_bounds__(256, 2) void skip_stats_kernel(StatArgs a) {
     const int64_t khead_row = ((int64_t)b * a.Hkv + kvh) * a.n_pad;
     const int q_local = 32 * w + r;
     float* part = reinterpret_cast<float*>(smem + NK * SLOT);              // [QT][nt][NW]
+    float* spare = part + QT * a.nt * NW;                                  // [NW][64]
 
     // Q fragments of both query tiles, in the widths the mode multiplies
     v8i qf4[QT][SST], qf8[QT][SST];
@@ -123,97 +136,153 @@ __global__ __launch_bounds__(256, 2) void skip_stats_kernel(StatArgs a) {
             koff[c] = (uint32_t)(row * ROW4 + (slot ^ ((row >> 2) & (CPR4 - 1))) * 16);
         }
     }
-    auto issue_k = [&](int t) __attribute__((always_inline)) {
-        const uint8_t* src = ALL8 ? a.k8 + (khead_row + (int64_t)t * TILE) * ROW8 : a.k4 + (khead_row + (int64_t)t * TILE) * ROW4;
-        uint8_t* slot = smem + (t % NK) * SLOT;
+    // The next K tile to fetch and the ring slot it goes to, kept as running values (a pointer and an offset that move by one
+    // tile) rather than worked out from the step number at every step.  Past the last tile the last one is fetched again, into
+    // a slot nobody reads any more: every step then finds the same number of loads in flight, and its wait is a constant.
+    const uint8_t* ksrc = ALL8 ? a.k8 + khead_row * ROW8 : a.k4 + khead_row * ROW4;
+    const uint8_t* ssrc = (ALL8 ? a.ks8 : a.ks4) + khead_row * (D / 32) + w * (KS_BYTES / NW);
+    uint32_t islot = 0, rslot = 0;
+    int issued = 0;
+    auto issue_next = [&]() __attribute__((always_inline)) {
+        uint8_t* slot = smem + islot;
 #pragma unroll
-        for (int c = 0; c < PIECES; ++c) load16_to_lds_sv(koff[c], src, slot + (w * PIECES + c) * 1024);
+        for (int c = 0; c < PIECES; ++c) load16_to_lds_sv(koff[c], ksrc, slot + (w * PIECES + c) * 1024);
         // the tile's 512 scale bytes, a quarter per wave (eight lanes of 16 bytes)
-        const uint8_t* ssrc = (ALL8 ? a.ks8 : a.ks4) + (khead_row + (int64_t)t * TILE) * (D / 32) + w * (KS_BYTES / NW);
         if (lane < KS_BYTES / NW / 16) load16_to_lds_sv((uint32_t)lane * 16u, ssrc, slot + KT_BYTES + w * (KS_BYTES / NW));
+        ++issued;
+        const bool more = issued < nsteps;
+        ksrc += more ? KT_BYTES : 0;
+        ssrc += more ? KS_BYTES : 0;
+        islot = islot == (NK - 1) * SLOT ? 0u : islot + SLOT;
     };
 
-#pragma unroll
-    for (int t = 0; t < NK - 1; ++t)
-        if (t < nsteps) issue_k(t);
-    for (int t = 0; t < nsteps; ++t) {
-        // K(t) has landed: its loads are older than those of the (at most NK - 2) tiles issued after it
+    const int i0 = 2 * pair, i1 = 2 * pair + 1;
+    const bool has1 = i1 < a.ntq;
+    v4i kf[KB][SST][ALL8 ? 2 : 1];
+    int ksc[KB];
+    v16f st0[KB], st1[KB];
+    // A step begins: its K tile has landed (its loads are older than those of the NK - 2 tiles fetched after it), everybody is
+    // past the tile before, whose slot takes the next fetch; then the staged tile's fragments and scales, once for both query tiles
+    auto begin_step = [&]() __attribute__((always_inline)) {
         __builtin_amdgcn_sched_barrier(0);
-        switch (min(NK - 2, nsteps - 1 - t)) {
-            case 0: __builtin_amdgcn_s_waitcnt(vm_imm(0)); break;
-            case 1: __builtin_amdgcn_s_waitcnt(vm_imm(G)); break;
-            case 2: __builtin_amdgcn_s_waitcnt(vm_imm(2 * G)); break;
-            case 3: __builtin_amdgcn_s_waitcnt(vm_imm(3 * G)); break;
-            default: __builtin_amdgcn_s_waitcnt(vm_imm(4 * G)); break;
-        }
+        __builtin_amdgcn_s_waitcnt(vm_imm((NK - 2) * G));
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        if (t + NK - 1 < nsteps) issue_k(t + NK - 1);      // into the buffer of K(t-1): everybody is past its last read
-
-        const int j = t;
-        const uint8_t* kl = smem + (t % NK) * SLOT;
-        // the staged tile's fragments and scales, once for both query tiles
-        v4i kf[KB][SST][ALL8 ? 2 : 1];
-        int ksc[KB];
+        issue_next();
+        // one address per step for the fragments of each half of the head dimension and one for the scales: the key blocks are
+        // constant offsets from them (the swizzle depends on the row inside a block only), which the opaque values keep
+        // in the instructions' offset fields instead of a vector addition per read
+        const uint32_t slot = rslot;
+        rslot = rslot == (NK - 1) * SLOT ? 0u : rslot + SLOT;
+        uint32_t fa[SST], sa = slot + KT_BYTES + r * (D / 32);
+        asm volatile("" : "+v"(sa));
+#pragma unroll
+        for (int s = 0; s < SST; ++s) {
+            fa[s] = slot + (ALL8 ? r * ROW8 + (((4 * s + h) ^ ((r >> 1) & (CPR8 - 1))) * 16) : r * ROW4 + (((2 * s + h) ^ ((r >> 2) & (CPR4 - 1))) * 16));
+            asm volatile("" : "+v"(fa[s]));
+        }
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
-            const int krow = 32 * kb + r;
-            ksc[kb] = (int)(*reinterpret_cast<const uint32_t*>(kl + KT_BYTES + krow * (D / 32)) >> (8 * h));
+            ksc[kb] = (int)(*reinterpret_cast<const uint32_t*>(smem + sa + 32 * kb * (D / 32)) >> (8 * h));
 #pragma unroll
             for (int s = 0; s < SST; ++s) {
                 if constexpr (ALL8) {
-                    const int f = (krow >> 1) & (CPR8 - 1);
-                    kf[kb][s][0] = *reinterpret_cast<const v4i*>(kl + krow * ROW8 + (((4 * s + h) ^ f) * 16));
-                    kf[kb][s][1] = *reinterpret_cast<const v4i*>(kl + krow * ROW8 + (((4 * s + h + 2) ^ f) * 16));
+                    // the second half's 16 bytes sit two chunks on: bit 1 of the chunk index, which the swizzle leaves to 4*s+h
+                    kf[kb][s][0] = *reinterpret_cast<const v4i*>(smem + fa[s] + 32 * kb * ROW8);
+                    kf[kb][s][1] = *reinterpret_cast<const v4i*>(smem + (fa[s] ^ 32u) + 32 * kb * ROW8);
                 } else {
-                    const int f = (krow >> 2) & (CPR4 - 1);
-                    kf[kb][s][0] = *reinterpret_cast<const v4i*>(kl + krow * ROW4 + (((2 * s + h) ^ f) * 16));
+                    kf[kb][s][0] = *reinterpret_cast<const v4i*>(smem + fa[s] + 32 * kb * ROW4);
                 }
             }
         }
+    };
+    // the eight score instructions of query tile x on the staged K tile
+    auto scores = [&](v16f (&st)[KB], int x) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) st[kb][e] = 0.0f;
+        // the four key blocks of one half of the head dimension, then of the other: no instruction waits for the one before it
+#pragma unroll
+        for (int s = 0; s < SST; ++s) {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                if constexpr (ALL8) {
+                    const v4i x0 = kf[kb][s][0], x1 = kf[kb][s][1];
+                    const v8i kd = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+                    st[kb] = score_mfma8<FMT8>(kd, qf8[x][s], st[kb], s, ksc[kb], qsc8[x]);
+                } else {
+                    const v4i v = kf[kb][s][0];
+                    const v8i kd = (v8i){v[0], v[1], v[2], v[3], 0, 0, 0, 0};
+                    st[kb] = score_mfma4(kd, qf4[x][s], st[kb], s, ksc[kb], qsc4[x]);
+                }
+            }
+        }
+    };
+    // a diag run's one 8-bit tile of query tile x (key tile j == its own index), operands straight from global memory
+    auto scores_diag = [&](v16f (&st)[KB], int x, int j) __attribute__((always_inline)) {
+        if constexpr (MODE == MPSA_MODE_DIAG) {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                const int krow = 32 * kb + r;
+                const int ks = (int)(*reinterpret_cast<const uint32_t*>(a.ks8 + (khead_row + (int64_t)j * TILE + krow) * (D / 32)) >> (8 * h));
+                const uint8_t* src = a.k8 + (khead_row + (int64_t)j * TILE + krow) * ROW8 + h * 16;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) st[kb][e] = 0.0f;
+#pragma unroll
+                for (int s = 0; s < SST; ++s) {
+                    const v4i x0 = *reinterpret_cast<const v4i*>(src + s * 64);
+                    const v4i x1 = *reinterpret_cast<const v4i*>(src + s * 64 + 32);
+                    const v8i kd = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+                    st[kb] = score_mfma8<FMT8>(kd, qf8[x][s], st[kb], s, ks, qsc8[x]);
+                }
+            }
+        }
+    };
+    // this lane's maximum over its 64 scores of a tile: 26 three-input maxima, which go into the gaps of the other query
+    // tile's score instructions in the plain steps
+    auto row_max = [&](const v16f (&st)[KB]) __attribute__((always_inline)) {
+        float mk[KB];
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) mk[kb] = tree_max16(st[kb]);
+        return max3f(mk[0], mk[1], __builtin_fmaxf(mk[2], mk[3]));
+    };
+    auto interleave = [&](auto per) __attribute__((always_inline)) {
+#pragma unroll
+        for (int g = 0; g < KB * SST; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        // one matrix instruction
+            __builtin_amdgcn_sched_group_barrier(0x002, decltype(per)::value, 0);      // some vector instructions
+        }
+    };
+    // this wave's share of the statistic of (query tile x, step t): the row maxima of its valid queries summed in the order
+    // the attention kernel adds them (attn_fwd_kernel.h: a butterfly over lanes 0-31; written with lane-permuting moves
+    // instead of the LDS shuffles of __shfl_xor, whose five dependent round trips cost more than the score instructions:
+    // lanes 1, 2 apart inside a quad, then -- every lane of a group holding the group's sum by then -- the mirrored lane
+    // of the 8- and the 16-lane group, then lane 0 + lane 16; float addition commutes, so lane 0 ends with the butterfly's bits)
+    auto finish = [&](float rm, int x, int t) __attribute__((always_inline)) {
+        const float mx = max_lane_pair(rm);
+        float sv = ((2 * pair + x) * TILE + q_local < a.nq) ? mx : 0.0f;
+        sv += lane_move<0xB1>(sv);                     // quad_perm [1,0,3,2]
+        sv += lane_move<0x4E>(sv);                     // quad_perm [2,3,0,1]
+        sv += lane_move<0x141>(sv);                    // row_half_mirror
+        sv += lane_move<0x140>(sv);                    // row_mirror
+        const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sv), 0));
+        const float s16 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sv), 16));
+        // lane 0 writes the sum; the other lanes write it to a spare word each, because a branch around the store would
+        // split the step into basic blocks and the score instructions would be moved out of the vector work they are to hide
+        float* dst = lane == 0 ? part + (x * a.nt + t) * NW + w : spare + 64 * w + lane;
+        *dst = s0 + s16;
+    };
+    // A step that needs a mask, an 8-bit tile from global memory, or has one of the two query tiles only: one thing after the other.
+    auto slow_step = [&](int t) __attribute__((always_inline)) {
+        begin_step();
+        const int j = t;
 #pragma unroll
         for (int x = 0; x < QT; ++x) {
             const int i = 2 * pair + x;
             if (i >= a.ntq || (a.causal && j > i)) continue;               // no such query tile, or a tile it does not visit
-            const bool diag8 = MODE == MPSA_MODE_DIAG && j == i;
-            v16f st[KB];
-            if (diag8) {
-                if constexpr (MODE == MPSA_MODE_DIAG) {                    // this query tile's one 8-bit tile, from global memory
-#pragma unroll
-                    for (int kb = 0; kb < KB; ++kb) {
-                        const int krow = 32 * kb + r;
-                        const int ks = (int)(*reinterpret_cast<const uint32_t*>(a.ks8 + (khead_row + (int64_t)j * TILE + krow) * (D / 32)) >> (8 * h));
-                        const uint8_t* src = a.k8 + (khead_row + (int64_t)j * TILE + krow) * ROW8 + h * 16;
-#pragma unroll
-                        for (int e = 0; e < 16; ++e) st[kb][e] = 0.0f;
-#pragma unroll
-                        for (int s = 0; s < SST; ++s) {
-                            const v4i x0 = *reinterpret_cast<const v4i*>(src + s * 64);
-                            const v4i x1 = *reinterpret_cast<const v4i*>(src + s * 64 + 32);
-                            const v8i kd = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-                            st[kb] = score_mfma8<FMT8>(kd, qf8[x][s], st[kb], s, ks, qsc8[x]);
-                        }
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int kb = 0; kb < KB; ++kb) {
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) st[kb][e] = 0.0f;
-#pragma unroll
-                    for (int s = 0; s < SST; ++s) {
-                        if constexpr (ALL8) {
-                            const v4i x0 = kf[kb][s][0], x1 = kf[kb][s][1];
-                            const v8i kd = (v8i){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-                            st[kb] = score_mfma8<FMT8>(kd, qf8[x][s], st[kb], s, ksc[kb], qsc8[x]);
-                        } else {
-                            const v4i v = kf[kb][s][0];
-                            const v8i kd = (v8i){v[0], v[1], v[2], v[3], 0, 0, 0, 0};
-                            st[kb] = score_mfma4(kd, qf4[x][s], st[kb], s, ksc[kb], qsc4[x]);
-                        }
-                    }
-                }
-            }
+            if (MODE == MPSA_MODE_DIAG && j == i) scores_diag(st0, x, j);
+            else scores(st0, x);
             // the masks the attention kernel applies before it takes the statistic: the causal diagonal, the keys past the end
             const bool diag_mask = a.causal && j == i;
             const int kmax = (j == a.nt - 1) ? a.n - j * TILE : TILE;
@@ -227,29 +296,77 @@ __global__ __launch_bounds__(256, 2) void skip_stats_kernel(StatArgs a) {
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int key = 32 * kb + 8 * (e >> 2) + 4 * h + (e & 3);
-                        if (key >= limit) st[kb][e] = -__builtin_inff();
+                        if (key >= limit) st0[kb][e] = -__builtin_inff();
                     }
             }
-            float mx = st[0][0];
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) mx = __builtin_fmaxf(mx, st[kb][e]);
-            mx = max_lane_pair(mx);
-            // summed over the wave's valid queries, in the order the attention kernel adds them (attn_fwd_kernel.h: a
-            // butterfly over lanes 0-31; written with lane-permuting moves instead of the LDS shuffles of __shfl_xor, whose
-            // five dependent round trips were most of a step: lanes 1, 2 apart inside a quad, then -- every lane of a group
-            // holding the group's sum by then -- the mirrored lane of the 8- and the 16-lane group, then lane 0 + lane 16;
-            // float addition commutes, so lane 0 ends with the bits of the butterfly)
-            float sv = (i * TILE + q_local < a.nq) ? mx : 0.0f;
-            sv += lane_move<0xB1>(sv);                     // quad_perm [1,0,3,2]
-            sv += lane_move<0x4E>(sv);                     // quad_perm [2,3,0,1]
-            sv += lane_move<0x141>(sv);                    // row_half_mirror
-            sv += lane_move<0x140>(sv);                    // row_mirror
-            const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sv), 0));
-            const float s16 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sv), 16));
-            if (lane == 0) part[(x * a.nt + t) * NW + w] = s0 + s16;
+            finish(row_max(st0), x, t);
         }
+    };
+    // The same sums for both query tiles of a plain step at once.  One exchange of the upper and lower 32 lanes of the two
+    // tiles' lane maxima and one maximum leave tile 0's row maxima in lanes 0-31 and tile 1's in lanes 32-63; the lane moves
+    // above sum each row of 16 lanes; lane 15 of a row broadcast into the next row adds rows 0 + 1 and rows 2 + 3 (the
+    // operands of "lane 0 + lane 16", so the same bits).  Lanes 16 and 48 store: 12 vector instructions for two tiles.
+    const bool pair_valid = (2 * pair + h) * TILE + q_local < a.nq;
+    const uint32_t pair_step = r == 16 ? NW * 4u : 0u;
+    const uint32_t pair_dst = (uint32_t)(NK * SLOT) + (r == 16 ? (uint32_t)(h * a.nt * NW + w) * 4u : (uint32_t)(QT * a.nt * NW + 64 * w + lane) * 4u);
+    auto finish_pair = [&](float rm0, float rm1, int t) __attribute__((always_inline)) {
+        int x0 = __builtin_bit_cast(int, rm0), x1 = __builtin_bit_cast(int, rm1);
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x0), "+v"(x1));
+        const float mx = __builtin_fmaxf(__builtin_bit_cast(float, x0), __builtin_bit_cast(float, x1));
+        float sv = pair_valid ? mx : 0.0f;
+        sv += lane_move<0xB1>(sv);
+        sv += lane_move<0x4E>(sv);
+        sv += lane_move<0x141>(sv);
+        sv += lane_move<0x140>(sv);
+        // row_bcast:15 into rows 1 and 3
+        sv += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sv), 0x142, 0xA, 0xF, false));
+        *reinterpret_cast<float*>(smem + pair_dst + (uint32_t)t * pair_step) = sv;
+    };
+    // Plain steps ta .. tb-1 (both query tiles, 4-bit tiles from LDS, no mask).  Vector instructions run under a wave's own
+    // matrix instructions but hardly under the other wave's, and a wave issues in order: what counts is the length of the
+    // wave's own instruction stream and how much of it sits between its matrix instructions.  Query tile 0's row maxima go
+    // into the gaps of tile 1's score instructions, tile 1's and the step's sums into those of tile 0 in the next step.
+    auto plain_steps = [&](int ta, int tb) __attribute__((always_inline)) {
+        if (ta >= tb) return;
+        begin_step();
+        scores(st0, 0);
+        for (int t = ta;; ++t) {
+            scores(st1, 1);
+            const float rm0 = row_max(st0);
+            interleave(std::integral_constant<int, 4>{});
+            if (t + 1 >= tb) {
+                finish_pair(rm0, row_max(st1), t);
+                break;
+            }
+            begin_step();
+            scores(st0, 0);
+            finish_pair(rm0, row_max(st1), t);
+            interleave(std::integral_constant<int, 6>{});
+        }
+    };
+    // steps that are not plain, in ascending order: (causal) everything from tile 0's diagonal on; (diag mode) the two diagonal
+    // tiles; the ragged last tile; and every step of a pair that has one query tile only
+    auto next_special = [&](int t) __attribute__((always_inline)) {
+        // an all-8-bit run holds twice the K fragments: they and two tiles of scores do not fit the registers, and its matrix
+        // instructions take twice as long against the same vector work, so it gains the least
+        if (ALL8 || !has1) return t;
+        int e = nsteps;
+        if (a.n < a.n_pad) e = a.nt - 1;
+        if (a.causal) return max(t, min(e, i0));
+        if constexpr (MODE == MPSA_MODE_DIAG) {
+            if (t <= i0) e = min(e, i0);
+            else if (t <= i1) e = min(e, i1);
+        }
+        return max(t, e);
+    };
+
+#pragma unroll
+    for (int t = 0; t < NK - 1; ++t) issue_next();
+    for (int t = 0; t < nsteps;) {
+        const int te = min(next_special(t), nsteps);
+        plain_steps(t, te);
+        if (te < nsteps) slow_step(te);
+        t = te + 1;
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
