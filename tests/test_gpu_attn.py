@@ -380,7 +380,8 @@ def test_tile_skipping_follows_the_reference_rule(mode, causal, N, D, tile):
 
 
 @pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "mxfp8e5", "diag", "diag_e5"])
-@pytest.mark.parametrize("causal,N", [(True, 1024), (False, 1024), (True, 1100), (False, 1100), (False, 640), (True, 2048)])
+@pytest.mark.parametrize("causal,N", [(True, 1024), (False, 1024), (True, 1100), (False, 1100), (False, 640), (True, 2048),
+                                      (True, 1000), (False, 1000)])
 def test_tile_skipping_decided_ahead_of_the_attention_kernel(mode, causal, N):
     """mpsa_skip_route + mpsa_attn_fwd_routed (every tile's statistic from a score-product-only pass, the rule, visiting lists
     of the kept tiles) against mpsa_attn_fwd_skip (the rule inside the attention kernel) and against the oracle: the same
@@ -423,6 +424,37 @@ def test_tile_skipping_decided_ahead_of_the_attention_kernel(mode, causal, N):
         eight = torch.eye(nt, dtype=torch.bool)
     assert ((cls == 2) == (kept & eight)).all()
     assert torch.equal(counts.sum(dim=-1).cpu(), kept.sum(dim=-1).to(torch.int32))
+
+
+@pytest.mark.parametrize("mode", ["mxfp4", "mxfp8"])
+@pytest.mark.parametrize("Nq,Nk", [(1000, 1300), (1300, 1000), (300, 700), (1024, 130)])
+def test_tile_skipping_ahead_with_different_query_and_key_lengths(mode, Nq, Nk):
+    """The same with Nq queries over Nk keys (no mask): pairs of query tiles whose second tile is ragged or missing, a
+    ragged last key tile, more and fewer key tiles than query tiles."""
+    from ours.mxfp_attn_kernel import prepare_operands, attention_from_operands, skip_route, skip_routable
+    tile, D, H = 128, 128, 2
+    g = torch.Generator().manual_seed(7 * Nq + Nk)
+    ntq, nt = -(-Nq // tile), -(-Nk // tile)
+    q = (torch.randn(1, 2 * H, Nq, D, generator=g) + 1.0).bfloat16()
+    k = (torch.randn(1, H, Nk, D, generator=g) + torch.rand(nt, generator=g).repeat_interleave(tile)[:Nk].view(1, 1, Nk, 1) * 0.5).bfloat16()
+    v = torch.randn(1, H, Nk, D, generator=g).bfloat16()
+    kw = dict(tile=tile, causal=False, mode=mode, fmt8=O.FMT_E4M3)
+    th = _robust_thresh(q, k, v, **kw)
+    want, want_sk = O.attn_mx(q, k, v, skip_thresh=th, return_skipped=True, out_dtype=torch.float32, **kw)
+    ops = prepare_operands(q.to(DEV), k.to(DEV), v.to(DEV), tile, mode)
+    assert skip_routable(ops, False)
+    ahead = torch.full((1, 2 * H, Nq, D), float("nan"), dtype=torch.float32, device=DEV)
+    inside = torch.full_like(ahead, float("nan"))
+    sk_a = torch.full((1, 2 * H, ntq), -1, dtype=torch.int32, device=DEV)
+    sk_i = torch.full_like(sk_a, -1)
+    attention_from_operands(ops, ahead, False, th, sk_a)
+    attention_from_operands(ops, inside, False, th, sk_i, skip_in_kernel=True)
+    assert torch.equal(sk_a.cpu(), want_sk) and torch.equal(sk_i.cpu(), want_sk)
+    _compare(ahead, want, f"skip ahead {mode} {Nq}x{Nk} th={th}")
+    _compare(inside, want, f"skip inside {mode} {Nq}x{Nk} th={th}")
+    cls, order, counts = skip_route(ops, False, th, want_cls=True)
+    assert cls.shape == (1, 2 * H, ntq, nt)
+    assert torch.equal((cls.cpu() == 0).sum(dim=-1).to(torch.int32), want_sk)
 
 
 @pytest.mark.parametrize("mode", ["diag", "mxfp4", "mxfp8e5"])
