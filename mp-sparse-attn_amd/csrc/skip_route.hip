@@ -345,11 +345,10 @@ __global__ __launch_bounds__(256, 2) void skip_stats_kernel(StatArgs a) {
         }
     };
     // steps that are not plain, in ascending order: (causal) everything from tile 0's diagonal on; (diag mode) the two diagonal
-    // tiles; the ragged last tile; and every step of a pair that has one query tile only
+    // tiles; the ragged last tile; and every step of a pair that has one query tile only.  (The mxfp8 mode's plain steps fit
+    // the registers with nothing to spare: twice the K fragments beside the two tiles of scores.)
     auto next_special = [&](int t) __attribute__((always_inline)) {
-        // an all-8-bit run holds twice the K fragments: they and two tiles of scores do not fit the registers, and its matrix
-        // instructions take twice as long against the same vector work, so it gains the least
-        if (ALL8 || !has1) return t;
+        if (!has1) return t;
         int e = nsteps;
         if (a.n < a.n_pad) e = a.nt - 1;
         if (a.causal) return max(t, min(e, i0));
