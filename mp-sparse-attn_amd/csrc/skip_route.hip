@@ -60,8 +60,8 @@ constexpr int stat_lds_bytes(int mode, int nt) { return NK * ((mode == MPSA_MODE
 // workgroups of a CU did not fill each other's gaps.  Hence, in the steps that need no mask (nearly all): one query
 // tile's row maxima sit between the other tile's score instructions, both tiles' sums are taken by one chain of lane
 // moves, the fetch pointers and ring slots are running values and the wait for a tile is a constant.  That is 150
-// instructions per wave and step instead of 220 and 15 % less time; most of what is left over the 0.23 ms of the matrix
-// instructions is clock: with every operand element the same the pass takes 0.39 ms, with random ones 0.50 (the
+// instructions per wave and step instead of 220, 31 % fewer cycles (matrix pipe busy 60 % of them) and 20 % less time;
+// most of what is left over the 0.23 ms of the matrix instructions is clock, which falls as the matrix work gets denser: with every operand element the same the pass takes 0.39 ms, with random ones 0.50 (the
 // matrix instructions' power draw, as in the attention kernel).
 template <int FMT8, int MODE>
 __global__ __launch_bounds__(256, 2) void skip_stats_kernel(StatArgs a) {
