@@ -387,6 +387,8 @@ def skip_study(args, device):
     B, Hq, Hkv, N, D, tile, seed, desc = WORKLOADS[args.workload]
     causal = args.workload not in NON_CAUSAL
     q, k, v = make_inputs(B, Hq, Hkv, N, D, seed, device, 0 if causal else 21, args.workload not in PLAIN_DRAWS)
+    if args.operands != "random":     # every element the same: what the statistics pass takes without the operands' bit toggling
+        q, k, v = (torch.full_like(t, 1.0 if args.operands == "ones" else 0.0) for t in (q, k, v))
     group = Hq // Hkv
     hq = max(min(args.heads, Hq) // group * group, group)
     q, k, v = q[:, :hq].contiguous(), k[:, :hq // group].contiguous(), v[:, :hq // group].contiguous()
@@ -497,7 +499,7 @@ def main():
     ap.add_argument("--no-c5", action="store_true", help="leave the video-DiT figures out of `secondary`")
     ap.add_argument("--eager", action="store_true", help="time plain launches instead of replaying the step as a HIP graph")
     ap.add_argument("--operands", default="random", choices=["random", "ones", "zeros"],
-                    help="--only gemm4|gemm8|attn: the workload's random operands (default) or constant ones (the clock then stays up)")
+                    help="--only gemm4|gemm8|attn|skip: the workload's random operands (default) or constant ones (the clock then stays up)")
     ap.add_argument("--linear-scales", action="store_true",
                     help="with --only gemm4/gemm8: row-major [rows, K/32] scales instead of the reference's packed form")
     ap.add_argument("--only", default=None, choices=["attn", "copy", "quant", "gemm4", "gemm8", "gemm48", "mfma", "router", "skip"],
