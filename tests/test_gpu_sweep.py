@@ -180,3 +180,35 @@ def test_quantizer_sweep():
         assert torch.equal(c4[:, :, :N].cpu(), w4) and torch.equal(s4[:, :, :N].cpu(), ws4), f"{what} dual 4-bit"
         assert torch.equal(c8[:, :, :N].cpu(), w8) and torch.equal(s8[:, :, :N].cpu(), ws8), f"{what} dual 8-bit"
 
+
+
+def test_tile_skipping_ahead_and_inside_agree_over_shapes():
+    """The rule decided ahead of the attention kernel (statistics pass + visiting lists + routed attention) against the rule
+    inside the attention kernel -- which the oracle pins (test_gpu_attn.py) -- from one tile to sixteen, whole and ragged
+    lengths, even and odd tile counts, with and without the mask, grouped heads: the same tiles skipped per query tile
+    and the same output, at thresholds on both sides of the sink's statistic."""
+    from ours.mxfp_attn_kernel import skip_routable
+    cases = 0
+    for N in [128, 129, 200, 256, 257, 300, 384, 385, 500, 512, 513, 640, 700, 769, 896, 1000, 1025, 1152, 1300, 1537, 2000]:
+        for causal in (True, False):
+            for mode in ("mxfp4", "diag", "mxfp8"):
+                H, G = (4, 2) if N % 3 else (2, 1)
+                g = torch.Generator().manual_seed(N * 7 + H)
+                nt = -(-N // 128)
+                q = (torch.randn(1, H, N, 128, generator=g) + 1.0).bfloat16().to(DEV)
+                k = (torch.randn(1, H // G, N, 128, generator=g) + torch.rand(nt, generator=g).repeat_interleave(128)[:N].view(1, 1, N, 1) * 0.5).bfloat16().to(DEV)
+                v = torch.randn(1, H // G, N, 128, generator=g).bfloat16().to(DEV)
+                ops = prepare_operands(q, k, v, 128, mode)
+                assert skip_routable(ops, causal)
+                for th in (0.98, 1.02):
+                    ahead = torch.full((1, H, N, 128), float("nan"), dtype=torch.float32, device=DEV)
+                    inside = torch.full_like(ahead, float("nan"))
+                    sk_a = torch.full((1, H, nt), -1, dtype=torch.int32, device=DEV)
+                    sk_i = torch.full_like(sk_a, -1)
+                    attention_from_operands(ops, ahead, causal, th, sk_a)
+                    attention_from_operands(ops, inside, causal, th, sk_i, skip_in_kernel=True)
+                    what = f"N={N} causal={causal} {mode} H={H} G={G} th={th}"
+                    assert torch.equal(sk_a, sk_i), what
+                    assert torch.equal(ahead, inside), what      # both walk the kept tiles through the same kernel code
+                    cases += 1
+    assert cases == 21 * 2 * 3 * 2
